@@ -1,0 +1,127 @@
+// Row gathers (embedding, logits rows), RMSNorm fused with the residual sum, SiLU-gating.
+//
+// What the reference does with eager torch ops: layers/embed_head.py:10-11 (gather),
+// layers/layernorm.py:11-24 (RMSNorm, residual add), layers/activation.py:5-7 (SiLU*up).
+// Here each is one kernel; the residual stream is kept in float32 and the sum, the
+// mean of squares and the scaling are computed in float32.
+#include "common.h"
+
+
+// ------------------------------------------------------------------ gather rows
+// out[r, :] = src[idx[r], :], rows of `row_bytes` bytes. One workgroup per row.
+template <typename V>
+__global__ void gather_rows_kernel(const V* __restrict__ src, const int32_t* __restrict__ idx,
+                                   V* __restrict__ out, int64_t row_vecs, int64_t num_src_rows) {
+  const int64_t r = blockIdx.x;
+  int64_t s = idx[r];
+  if (s < 0 || s >= num_src_rows) s = 0;  // the binding checks ids on the host; never read outside
+  const V* a = src + s * row_vecs;
+  V* b = out + r * row_vecs;
+  for (int64_t i = threadIdx.x; i < row_vecs; i += blockDim.x) b[i] = a[i];
+}
+
+extern "C" int me_gather_rows(const void* src, const int32_t* idx, void* out, int64_t num_rows,
+                              int64_t row_bytes, int64_t num_src_rows, hipStream_t stream) {
+  if (num_rows == 0) return 0;
+  ME_CHECK(row_bytes > 0 && num_src_rows > 0, "gather_rows: empty source");
+  const bool a16 = row_bytes % 16 == 0 && (reinterpret_cast<uintptr_t>(src) % 16 == 0) &&
+                   (reinterpret_cast<uintptr_t>(out) % 16 == 0);
+  if (a16) {
+    int64_t n = row_bytes / 16;
+    int threads = n >= 256 ? 256 : (n > 64 ? 128 : 64);
+    gather_rows_kernel<uint4><<<dim3(num_rows), dim3(threads), 0, stream>>>(
+        (const uint4*)src, idx, (uint4*)out, n, num_src_rows);
+  } else if (row_bytes % 2 == 0) {
+    int64_t n = row_bytes / 2;
+    gather_rows_kernel<uint16_t><<<dim3(num_rows), dim3(256), 0, stream>>>(
+        (const uint16_t*)src, idx, (uint16_t*)out, n, num_src_rows);
+  } else {
+    gather_rows_kernel<uint8_t><<<dim3(num_rows), dim3(256), 0, stream>>>(
+        (const uint8_t*)src, idx, (uint8_t*)out, row_bytes, num_src_rows);
+  }
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------ RMSNorm (+ residual)
+// r = x (+ res_in)           summed in float32, kept in float32 as the new residual
+// y = w * r * rsqrt(mean(r^2) + eps)
+// x may be `num_partials` stacked float32 partial sums [P, T, n] (a split-K product whose
+// partial results are added here, in a fixed order) or one tensor of the compute dtype.
+template <typename TX, typename TY>
+__global__ void rms_norm_kernel(const TX* __restrict__ x, int num_partials, int64_t partial_stride,
+                                const float* __restrict__ res_in, float* __restrict__ res_out,
+                                const float* __restrict__ w, TY* __restrict__ y, int n, float eps) {
+  __shared__ float scratch[16];
+  extern __shared__ float row[];  // n floats: the summed row, so that it is read from memory once
+  const int64_t t = blockIdx.x;
+  const TX* xr = x + t * n;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = to_f32<TX>(xr[i]);
+    for (int p = 1; p < num_partials; ++p) v += to_f32<TX>(xr[p * partial_stride + i]);
+    if (res_in) v += res_in[t * n + i];
+    if (res_out) res_out[t * n + i] = v;
+    row[i] = v;
+    ss += v * v;
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = rsqrtf(total / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) y[t * n + i] = from_f32<TY>(w[i] * (row[i] * inv));
+}
+
+extern "C" int me_rms_norm(const void* x, int x_dtype, int num_partials, int64_t partial_stride,
+                           const float* res_in, float* res_out, const float* w, void* y, int y_dtype,
+                           int64_t num_rows, int n, float eps, hipStream_t stream) {
+  if (num_rows == 0) return 0;
+  ME_CHECK(n > 0 && n <= 36864, "rms_norm: width %d outside 1..36864", n);
+  ME_CHECK(num_partials >= 1, "rms_norm: num_partials must be >= 1");
+  ME_CHECK(num_partials == 1 || x_dtype == ME_F32, "rms_norm: partial sums must be float32");
+  int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : (n >= 128 ? 128 : 64));
+  size_t lds = (size_t)n * sizeof(float);
+  dim3 grid(num_rows), block(threads);
+#define LAUNCH(TX, TY)                                                                       \
+  rms_norm_kernel<TX, TY><<<grid, block, lds, stream>>>((const TX*)x, num_partials,          \
+                                                        partial_stride, res_in, res_out, w, \
+                                                        (TY*)y, n, eps)
+  if (x_dtype == ME_BF16 && y_dtype == ME_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (x_dtype == ME_F32 && y_dtype == ME_BF16) LAUNCH(float, bf16_t);
+  else if (x_dtype == ME_F32 && y_dtype == ME_F32) LAUNCH(float, float);
+  else if (x_dtype == ME_BF16 && y_dtype == ME_F32) LAUNCH(bf16_t, float);
+  else ME_CHECK(false, "rms_norm: bad dtype codes %d %d", x_dtype, y_dtype);
+#undef LAUNCH
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------ SiLU(gate) * up
+// gu: [T, 2I] with gate = first I columns (reference layers/activation.py:6); out: [T, I].
+template <typename T>
+__global__ void silu_and_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t rows, int inter) {
+  const int64_t total = rows * (int64_t)inter;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = e / inter;
+    const int i = (int)(e - t * inter);
+    const float g = to_f32<T>(gu[t * 2 * inter + i]);
+    const float u = to_f32<T>(gu[t * 2 * inter + inter + i]);
+    out[e] = from_f32<T>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int me_silu_and_mul(const void* gu, void* out, int dtype, int64_t rows, int inter,
+                               hipStream_t stream) {
+  if (rows == 0) return 0;
+  ME_CHECK(inter > 0, "silu_and_mul: intermediate size must be positive");
+  const int64_t total = rows * (int64_t)inter;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == ME_BF16)
+    silu_and_mul_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, rows, inter);
+  else if (dtype == ME_F32)
+    silu_and_mul_kernel<float><<<dim3(blocks), dim3(256), 0, stream>>>((const float*)gu, (float*)out, rows, inter);
+  else
+    ME_CHECK(false, "silu_and_mul: bad dtype code %d", dtype);
+  ME_LAUNCH_CHECK();
+  return 0;
+}

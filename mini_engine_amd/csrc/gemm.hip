@@ -1,0 +1,182 @@
+// Matrix products y[M, N] = x[M, K] . w[N, K]^T (weights stored [out, in] as in the checkpoint;
+// the reference calls F.linear for all of them: layers/linear.py:26,45, models/qwen3.py:21,47,
+// layers/embed_head.py:23).
+//
+//  * me_gemm_tiled: any shape, float32 or bfloat16 inputs, float32 accumulation with plain FMAs
+//    (no matrix-core, no reduced precision). Each output element is one thread's sequential sum
+//    over K, so a row's result does not depend on the other rows of the batch. This is the
+//    float32 path and the fallback for bf16 shapes the MFMA kernel refuses.
+//  * me_gemm_skinny_bf16: the decode product, M small. Pure weight streaming: each workgroup
+//    owns 16 output features, its 4 waves split K, every lane reads 64 contiguous bytes of a
+//    weight row per step (whole cache lines per row and wave), products on
+//    v_mfma_f32_16x16x32_bf16 with the tokens as the 16-wide B operand, waves merged through
+//    LDS. Optional split of K over workgroups writes float32 partial sums [S, M, N] that the
+//    consumer (the fused residual + RMSNorm kernel) adds in a fixed order.
+#include "common.h"
+
+
+// ------------------------------------------------------------------ tiled FMA product
+#define GT_TILE 64
+#define GT_BK 16
+
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256)
+gemm_tiled_kernel(const TI* __restrict__ x, int64_t ldx, const TI* __restrict__ w, int64_t ldw,
+                  TO* __restrict__ y, int64_t ldy, int M, int N, int K) {
+  __shared__ float xs[GT_BK][GT_TILE + 1];
+  __shared__ float ws[GT_BK][GT_TILE + 1];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * GT_TILE, n0 = blockIdx.x * GT_TILE;
+  const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += GT_BK) {
+    // 64 rows x 16 k = 1024 elements per operand, 4 per thread; consecutive threads read along k
+    for (int e = tid; e < GT_TILE * GT_BK; e += 256) {
+      const int r = e / GT_BK, kk = e % GT_BK;
+      const int k = k0 + kk;
+      xs[kk][r] = (m0 + r < M && k < K) ? to_f32<TI>(x[(int64_t)(m0 + r) * ldx + k]) : 0.f;
+      ws[kk][r] = (n0 + r < N && k < K) ? to_f32<TI>(w[(int64_t)(n0 + r) * ldw + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GT_BK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { a[i] = xs[kk][tm + i]; b[i] = ws[kk][tn + i]; }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = m0 + tm + i, n = n0 + tn + j;
+      if (m < M && n < N) y[(int64_t)m * ldy + n] = from_f32<TO>(acc[i][j]);
+    }
+}
+
+extern "C" int me_gemm_tiled(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
+                             int in_dtype, int out_dtype, int M, int N, int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  ME_CHECK(K >= 1 && ldx >= K && ldw >= K && ldy >= N, "gemm: bad leading dimensions");
+  dim3 grid((N + GT_TILE - 1) / GT_TILE, (M + GT_TILE - 1) / GT_TILE), block(256);
+  ME_CHECK(grid.y <= 65535, "gemm: too many rows (%d) for one launch", M);
+#define LAUNCH(TI, TO) \
+  gemm_tiled_kernel<TI, TO><<<grid, block, 0, stream>>>((const TI*)x, ldx, (const TI*)w, ldw, (TO*)y, ldy, M, N, K)
+  if (in_dtype == ME_F32 && out_dtype == ME_F32) LAUNCH(float, float);
+  else if (in_dtype == ME_BF16 && out_dtype == ME_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (in_dtype == ME_BF16 && out_dtype == ME_F32) LAUNCH(bf16_t, float);
+  else ME_CHECK(false, "gemm: unsupported dtype pair %d -> %d", in_dtype, out_dtype);
+#undef LAUNCH
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------ skinny bf16 product on MFMA
+__device__ __forceinline__ bf16x8 gz8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = static_cast<bf16_t>(0.f);
+  return z;
+}
+
+// MT: 16-token tiles per workgroup. Grid (ceil(N/16), ceil(M/(16*MT)), ksplit).
+// k-slot mapping of MFMA j (0..3) inside a 128-wide macro step s: lane group g supplies
+// k = 128 s + 32 g + 8 j + 0..7 for both operands, so a lane's four loads are 64 contiguous bytes.
+template <int MT, typename TO>
+__global__ void __launch_bounds__(256)
+gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
+                   TO* __restrict__ y, int64_t ldy, float* __restrict__ partials, int M, int N, int K,
+                   int steps_per_split) {
+  __shared__ float red[4][MT][256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16 * MT;
+  const int split = blockIdx.z;
+  const int s_begin = split * steps_per_split;
+  const int total_steps = (K + 127) / 128;
+  const int s_end = min(total_steps, s_begin + steps_per_split);
+
+  const bool wrow_ok = n0 + r < N;
+  const bf16_t* wrow = w + (int64_t)(wrow_ok ? n0 + r : 0) * ldw;
+  const bf16_t* xrow[MT];
+  bool xrow_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + 16 * mt + r;
+    xrow_ok[mt] = m < M;
+    xrow[mt] = x + (int64_t)(xrow_ok[mt] ? m : 0) * ldx;
+  }
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int s = s_begin + wave; s < s_end; s += 4) {
+    const int kb = 128 * s + 32 * g;
+    bf16x8 a[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = kb + 8 * j;
+      a[j] = (wrow_ok && k < K) ? *reinterpret_cast<const bf16x8*>(wrow + k) : gz8();
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = kb + 8 * j;
+        const bf16x8 b = (xrow_ok[mt] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[mt] + k) : gz8();
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b, acc[mt], 0, 0, 0);
+      }
+    }
+  }
+  // accumulator: lane (token r, g) holds features n0 + 4g + i
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][mt][r * 16 + 4 * g + i] = acc[mt][i];
+  __syncthreads();
+  for (int e = threadIdx.x; e < MT * 256; e += 256) {
+    const int mt = e >> 8, idx = e & 255;
+    const int m = m0 + 16 * mt + (idx >> 4), n = n0 + (idx & 15);
+    if (m < M && n < N) {
+      const float v = red[0][mt][idx] + red[1][mt][idx] + red[2][mt][idx] + red[3][mt][idx];
+      if (partials) partials[((int64_t)split * M + m) * N + n] = v;
+      else y[(int64_t)m * ldy + n] = from_f32<TO>(v);
+    }
+  }
+}
+
+// y: bf16 or float32 [M, N]; or, when ksplit > 1, `partials` float32 [ksplit, M, N] (y unused).
+extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y,
+                                   int64_t ldy, int out_dtype, float* partials, int ksplit, int M, int N,
+                                   int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  ME_CHECK(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
+           "skinny gemm: K=%d and the row strides must be multiples of 8", K);
+  ME_CHECK((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0),
+           "skinny gemm: operands must be 16-byte aligned");
+  ME_CHECK(ksplit >= 1 && (ksplit == 1) == (partials == nullptr), "skinny gemm: partials iff ksplit > 1");
+  const int total_steps = (K + 127) / 128;
+  ME_CHECK(ksplit <= total_steps, "skinny gemm: ksplit %d exceeds the %d K-steps of 128", ksplit, total_steps);
+  const int steps_per_split = (total_steps + ksplit - 1) / ksplit;
+  const int mt = M > 32 ? 4 : (M > 16 ? 2 : 1);
+  dim3 grid((N + 15) / 16, (M + 16 * mt - 1) / (16 * mt), ksplit), block(256);
+  ME_CHECK(grid.y <= 65535, "skinny gemm: too many rows (%d)", M);
+#define LAUNCH(MTV, TO) \
+  gemm_skinny_kernel<MTV, TO><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, \
+                                                           (TO*)y, ldy, partials, M, N, K, steps_per_split)
+  if (out_dtype == ME_F32 || partials) {
+    if (mt == 4) LAUNCH(4, float); else if (mt == 2) LAUNCH(2, float); else LAUNCH(1, float);
+  } else if (out_dtype == ME_BF16) {
+    if (mt == 4) LAUNCH(4, bf16_t); else if (mt == 2) LAUNCH(2, bf16_t); else LAUNCH(1, bf16_t);
+  } else {
+    ME_CHECK(false, "skinny gemm: bad output dtype code %d", out_dtype);
+  }
+#undef LAUNCH
+  ME_LAUNCH_CHECK();
+  return 0;
+}

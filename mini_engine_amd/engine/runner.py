@@ -1,0 +1,217 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+Reference counterpart: engine/model_runner.py:87-145 (`prepare` + `run`). Differences by
+design: the step returns float32 logits at the places the caller names (sampling is a
+separate call), the metadata of a step travels to the GPU as one packed int32 array, and
+the runner owns the device side of the cache (`CachePool`) while the `CacheManager` it is
+given owns the bookkeeping.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.pool import CachePool, page_bytes
+from ..kernels import ops
+from .context import GroupStep, StepContext
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: `tokens` are its tokens at positions start..start+n-1
+    (start = how many of its tokens are already in the cache); `want` lists the places among
+    these tokens whose logits are asked for."""
+
+    req: object
+    tokens: list
+    start: int
+    want: list = field(default_factory=list)
+
+
+def _pad4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class ModelRunner:
+    def __init__(self, model, manager: CacheManager, dtype: torch.dtype, device, max_positions: int,
+                 poison_cache: bool = False):
+        self.model = model
+        self.manager = manager
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.max_positions = max_positions
+        self.plan = model.cache_plan()
+        if len(self.plan.group_needs) != manager.num_groups and self.plan.group_needs:
+            raise ValueError(f"the model needs {len(self.plan.group_needs)} page groups, "
+                             f"the cache manager has {manager.num_groups}")
+        self.pool = CachePool(self.plan, [manager.num_pages(g) for g in range(len(self.plan.group_needs))],
+                              manager.page_size, manager.num_state_slots, dtype, self.device, poison=poison_cache)
+        if self.pool.has_state and manager.num_state_slots < 1:
+            raise ValueError("the model keeps per-request state but the cache manager has no state slots")
+        self.vocab_size = model.embedding.vocab_size if hasattr(model.embedding, "vocab_size") else None
+        self._host = [None, None]
+        self._events = [None, None]
+        self._dev = None
+        self._flip = 0
+
+    # -- sizing ----------------------------------------------------------------------------
+    @staticmethod
+    def windows_of(model) -> list:
+        return [need.window for need in model.cache_plan().group_needs]
+
+    @staticmethod
+    def pages_that_fit(model, page_size: int, dtype: torch.dtype, budget_bytes: int) -> int:
+        """Pages per group such that all groups together fit `budget_bytes`."""
+        per_page = sum(page_bytes(model.cache_plan(), page_size, dtype))
+        return max(0, int(budget_bytes // max(1, per_page)))
+
+    # -- staging ---------------------------------------------------------------------------
+    def _staging(self, n: int):
+        i = self._flip
+        self._flip ^= 1
+        on_gpu = self.device.type == "cuda"
+        if self._host[i] is None or self._host[i].numel() < n:
+            cap = max(n, 4096) * 2
+            self._host[i] = torch.empty(cap, dtype=torch.int32, pin_memory=on_gpu)
+            self._events[i] = None
+        elif self._events[i] is not None:
+            self._events[i].synchronize()      # the copy that last used this buffer has finished
+        if self._dev is None or self._dev.numel() < n:
+            self._dev = torch.empty(max(n, 4096) * 2, dtype=torch.int32, device=self.device)
+        return i, self._host[i]
+
+    # -- the step --------------------------------------------------------------------------
+    @torch.inference_mode()
+    def step(self, entries: list) -> torch.Tensor | None:
+        """Run the given tokens as one batch. Returns float32 logits [R, vocab] for the wanted
+        places, in the order of `entries` and of each entry's `want`; None if nothing is wanted.
+
+        The pages (and state slot) of every request must have been allocated by the caller
+        through the cache manager for positions up to start + len(tokens)."""
+        if not entries:
+            return None
+        ps = self.manager.page_size
+        seen = set()
+        for e in entries:
+            if e.req in seen:
+                raise ValueError(f"request {e.req!r} appears twice in one step")
+            seen.add(e.req)
+            if not e.tokens:
+                raise ValueError(f"request {e.req!r} brings no tokens")
+            if e.start < 0 or e.start + len(e.tokens) > self.max_positions:
+                raise ValueError(f"request {e.req!r}: positions {e.start}..{e.start + len(e.tokens) - 1} "
+                                 f"exceed the engine's limit of {self.max_positions} tokens")
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise ValueError(f"request {e.req!r}: wanted place {w} outside its {len(e.tokens)} tokens")
+        # decodes (one new token) first, the others after, each kept in the caller's order
+        order = [i for i, e in enumerate(entries) if len(e.tokens) == 1] + \
+                [i for i, e in enumerate(entries) if len(e.tokens) != 1]
+        Dn = sum(1 for e in entries if len(e.tokens) == 1)
+        B = len(entries)
+        q_lens = [len(entries[i].tokens) for i in order]
+        starts = [entries[i].start for i in order]
+        T = sum(q_lens)
+        cu = np.zeros(B + 1, dtype=np.int64)
+        np.cumsum(q_lens, out=cu[1:])
+        G = self.manager.num_groups if self.plan.group_needs else 0
+        tables = [[self.manager.block_table(entries[i].req, g) for i in order] for g in range(G)]
+        MB = [max(1, max(len(t) for t in tables[g])) for g in range(G)]
+        # rows that want logits, in the caller's order
+        offset_of = {order[j]: int(cu[j]) for j in range(B)}
+        rows = [offset_of[i] + w for i, e in enumerate(entries) for w in e.want]
+        R = len(rows)
+
+        # ---- one packed int32 array: offsets (each segment padded to 16 bytes)
+        seg, n = {}, 0
+        for name, size in (("tokens", T), ("positions", T), ("seq_of_token", T), ("context_lens", B),
+                           ("cu", B + 1), ("prefill_cu", B - Dn + 1), ("state_slots", B), ("first_chunk", B),
+                           ("rows", max(R, 1))):
+            seg[name] = (n, size)
+            n += _pad4(size)
+        for g in range(G):
+            seg[f"slots{g}"] = (n, T); n += _pad4(T)
+            seg[f"bt{g}"] = (n, B * MB[g]); n += _pad4(B * MB[g])
+        buf_i, host = self._staging(n)
+        a = host.numpy()[:n]
+
+        def put(name, values):
+            o, size = seg[name]
+            a[o:o + size] = values
+
+        tok = np.concatenate([np.asarray(entries[i].tokens, dtype=np.int64) for i in order])
+        if self.vocab_size is not None and (tok.min() < 0 or tok.max() >= self.vocab_size):
+            raise ValueError(f"token id outside 0..{self.vocab_size - 1}")
+        pos = np.concatenate([np.arange(s, s + q, dtype=np.int64) for s, q in zip(starts, q_lens)])
+        put("tokens", tok)
+        put("positions", pos)
+        put("seq_of_token", np.repeat(np.arange(B), q_lens))
+        put("context_lens", [s + q for s, q in zip(starts, q_lens)])
+        put("cu", cu)
+        put("prefill_cu", cu[Dn:] - cu[Dn])
+        slots_of = [self.manager.state_slot(entries[i].req) for i in order]
+        put("state_slots", slots_of)
+        put("first_chunk", [1 if s == 0 else 0 for s in starts])
+        if R:
+            put("rows", rows)
+        for g in range(G):
+            bt = np.full((B, MB[g]), -1, dtype=np.int64)
+            slot = np.empty(T, dtype=np.int64)
+            for j in range(B):
+                t = tables[g][j]
+                bt[j, :len(t)] = t
+                p = pos[cu[j]:cu[j + 1]]
+                pages = bt[j, p // ps]
+                if (pages < 0).any():
+                    raise RuntimeError(f"request {entries[order[j]].req!r} has no page for a position it is "
+                                       f"about to write (group {g}); allocate before stepping")
+                slot[cu[j]:cu[j + 1]] = pages * ps + p % ps
+            put(f"slots{g}", slot)
+            put(f"bt{g}", bt.reshape(-1))
+
+        dev = self._dev[:n]
+        dev.copy_(host[:n], non_blocking=True)
+        if self.device.type == "cuda":
+            ev = torch.cuda.Event()
+            ev.record()
+            self._events[buf_i] = ev
+
+        def view(name):
+            o, size = seg[name]
+            return dev[o:o + size]
+
+        ctx = StepContext(
+            num_tokens=T, num_seqs=B, num_decodes=Dn, positions=view("positions"),
+            seq_of_token=view("seq_of_token"), context_lens=view("context_lens"), cu_seqlens=view("cu"),
+            prefill_cu=view("prefill_cu") if Dn < B else None,
+            max_decode_context=max((s + 1 for s, q in zip(starts, q_lens) if q == 1), default=0),
+            groups=[GroupStep(view(f"bt{g}").view(B, MB[g]), view(f"slots{g}")) for g in range(G)],
+            state_slots=view("state_slots"), first_chunk=view("first_chunk"), q_lens=q_lens, starts=starts)
+
+        # a request whose tokens start at position 0 starts from empty state
+        if self.pool.has_state:
+            fresh = [s for s, st in zip(slots_of, starts) if st == 0 and s >= 0]
+            if fresh:
+                idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
+                for st in self.pool.states:
+                    if st is not None:
+                        st.index_fill_(0, idx, 0)
+
+        h, residual = self.model.forward(view("tokens"), ctx, self.pool.views, self.pool.states)
+        if not R:
+            return None
+        return self.model.logits(h, residual, view("rows")[:R])
+
+    # -- sampling --------------------------------------------------------------------------
+    @torch.inference_mode()
+    def sample(self, logits: torch.Tensor, temperatures: list, keys: list) -> list:
+        """Token ids for float32 logits [S, V]; keys: (k0, k1) 32-bit pairs per row."""
+        S = logits.shape[0]
+        t = torch.tensor(temperatures, dtype=torch.float32).to(self.device, non_blocking=True)
+        k = torch.tensor(np.asarray(keys, dtype=np.uint32).astype(np.int64).reshape(S, 2) % (1 << 32),
+                         dtype=torch.int64)
+        k = torch.where(k >= (1 << 31), k - (1 << 32), k).to(torch.int32).to(self.device, non_blocking=True)
+        return ops.sample(logits, t, k).tolist()

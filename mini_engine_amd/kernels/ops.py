@@ -1,0 +1,384 @@
+"""The engine's operations: thin, checked calls into the HIP libraries.
+
+Every function takes torch tensors on the GPU, checks on the host what the
+kernel assumes about shapes, strides and dtypes, and launches on torch's current
+stream. There is no other implementation behind these names: without a GPU or
+without the built library a call raises. (Tests may install another backend with
+`set_backend` to exercise the engine's bookkeeping on a machine without a GPU.)
+
+Reference counterparts: layers/ops.py:23-57 (attention/cache bindings and the
+v1/v2 decode dispatcher), and the eager torch ops named in each docstring.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from . import build
+
+ME_BF16, ME_F32 = 0, 1
+_DT = {torch.bfloat16: ME_BF16, torch.float32: ME_F32}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {dtype}; the kernels take bfloat16 and float32") from None
+
+
+# --------------------------------------------------------------------------- libraries
+
+class _Lib:
+    def __init__(self, path: str, protos: dict):
+        self.path = path
+        self.cdll = ctypes.CDLL(path)
+        self.cdll.me_last_error.restype = c_char_p
+        for name, argtypes in protos.items():
+            fn = getattr(self.cdll, name)
+            fn.argtypes = argtypes
+            fn.restype = c_int
+        self.protos = protos
+
+    def call(self, name: str, *args):
+        rc = getattr(self.cdll, name)(*args)
+        if rc != 0:
+            raise KernelError(f"{name}: {self.cdll.me_last_error().decode()}")
+
+
+P, I, L, F = c_void_p, c_int, c_int64, c_float
+_CORE_PROTOS = {
+    "me_gather_rows": [P, P, P, L, L, L, P],
+    "me_rms_norm": [P, I, I, L, P, P, P, P, I, L, I, F, P],
+    "me_silu_and_mul": [P, P, I, L, I, P],
+    "me_qk_norm_rope_store": [P, I, L, L, P, P, F, P, L, P, P, P, P, I, I, I, I, I, P],
+    "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
+    "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, L, I, I, I, I, F, I, P],
+    "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
+    "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
+    "me_sample": [P, L, P, P, P, I, I, P],
+}
+_ATTN_PROTOS = {
+    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, P],
+    "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, P],
+}
+
+_core: _Lib | None = None
+_attn: dict = {}
+
+
+def _require_gpu() -> None:
+    if not torch.cuda.is_available():
+        raise KernelError("mini_engine_amd needs an AMD GPU (gfx950): torch.cuda.is_available() is False "
+                          "and there is no CPU implementation")
+
+
+def core() -> _Lib:
+    global _core
+    if _core is None:
+        _require_gpu()
+        _core = _Lib(build.core_library(), _CORE_PROTOS)
+    return _core
+
+
+def attn_lib(head_dim: int) -> _Lib:
+    lib = _attn.get(head_dim)
+    if lib is None:
+        _require_gpu()
+        lib = _Lib(build.attention_library(head_dim), _ATTN_PROTOS)
+        lib.cdll.me_attn_head_dim.restype = c_int
+        if lib.cdll.me_attn_head_dim() != head_dim:
+            raise KernelError(f"{lib.path} was built for head size {lib.cdll.me_attn_head_dim()}, not {head_dim}")
+        _attn[head_dim] = lib
+    return lib
+
+
+def loaded_libraries() -> list:
+    return ([_core.path] if _core else []) + [l.path for l in _attn.values()]
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _is_i32(t: torch.Tensor, n: int | None = None) -> bool:
+    return t.dtype == torch.int32 and t.is_contiguous() and (n is None or t.numel() >= n)
+
+
+# --------------------------------------------------------------------------- the HIP backend
+
+class HipBackend:
+    """Each method is one kernel (or one dispatch among kernels of the same meaning)."""
+
+    name = "hip"
+
+    # -- rows ----------------------------------------------------------------------------
+    def gather_rows(self, src: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+        """out[r] = src[idx[r]] (embedding lookup: reference layers/embed_head.py:10-11;
+        rows that want logits: layers/embed_head.py:20-22)."""
+        _check(src.dim() == 2 and src.is_contiguous(), "gather_rows: source must be a contiguous matrix")
+        _check(_is_i32(idx) and idx.dim() == 1, "gather_rows: indices must be int32 [n]")
+        out = torch.empty((idx.numel(), src.shape[1]), dtype=src.dtype, device=src.device)
+        core().call("me_gather_rows", src.data_ptr(), idx.data_ptr(), out.data_ptr(), idx.numel(),
+                    src.shape[1] * src.element_size(), src.shape[0], _stream())
+        return out
+
+    # -- norm ----------------------------------------------------------------------------
+    def rms_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None,
+                 out_dtype: torch.dtype, want_residual: bool = True):
+        """y = w * r * rsqrt(mean(r^2) + eps), r = x (+ residual) in float32 (reference
+        layers/layernorm.py:11-24). x: [T, n], or float32 partial sums [P, T, n] that are added
+        first. Returns (y [T, n] in out_dtype, r [T, n] float32 or None)."""
+        parts = 1
+        if x.dim() == 3:
+            parts = x.shape[0]
+            _check(x.dtype == torch.float32, "rms_norm: stacked partial sums must be float32")
+        _check(x.is_contiguous(), "rms_norm: x must be contiguous")
+        T, n = x.shape[-2], x.shape[-1]
+        _check(weight.dtype == torch.float32 and weight.shape == (n,) and weight.is_contiguous(),
+               "rms_norm: weight must be float32 [n]")
+        if residual is not None:
+            _check(residual.dtype == torch.float32 and residual.shape == (T, n) and residual.is_contiguous(),
+                   "rms_norm: residual must be contiguous float32 [T, n]")
+        y = torch.empty((T, n), dtype=out_dtype, device=x.device)
+        res_out = torch.empty((T, n), dtype=torch.float32, device=x.device) if want_residual else None
+        core().call("me_rms_norm", x.data_ptr(), _code(x.dtype), parts, T * n, _ptr(residual), _ptr(res_out),
+                    weight.data_ptr(), y.data_ptr(), _code(out_dtype), T, n, float(eps), _stream())
+        return y, res_out
+
+    # -- feed-forward activation ---------------------------------------------------------
+    def silu_and_mul(self, gu: torch.Tensor) -> torch.Tensor:
+        """silu(gu[:, :I]) * gu[:, I:] (reference layers/activation.py:5-7)."""
+        _check(gu.dim() == 2 and gu.is_contiguous() and gu.shape[1] % 2 == 0, "silu_and_mul: [T, 2I] contiguous")
+        inter = gu.shape[1] // 2
+        out = torch.empty((gu.shape[0], inter), dtype=gu.dtype, device=gu.device)
+        core().call("me_silu_and_mul", gu.data_ptr(), out.data_ptr(), _code(gu.dtype), gu.shape[0], inter, _stream())
+        return out
+
+    # -- q/k norm + rotary + cache write -------------------------------------------------
+    def qk_norm_rope_store(self, qkv, q_weight, k_weight, eps, table, positions, slots, k_cache, v_cache,
+                           Hq: int, Hkv: int, D: int, page: int, store: bool = True) -> None:
+        """In place on packed rows: per-head RMSNorm of q and k (weights float32 [D] or None), then
+        rotary by `table` [P, D/2, 2] float32 (or None), q written back.
+
+        store=True: rows are [T, (Hq+2Hkv)*D]; k and v are scattered to the pages at `slots`
+        (slots < 0 skipped). store=False: rows are [T, (Hq+Hkv)*D] (Hkv may be 0); k is written
+        back in place and nothing is cached. (reference models/qwen3.py:34-36,
+        layers/rotary_embedding.py:20-25, csrc/kv_cache.cu:10-31.)"""
+        T = qkv.shape[0]
+        width = (Hq + (2 * Hkv if store else Hkv)) * D
+        _check(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == width,
+               f"qk_norm_rope_store: rows must be [T, {width}] with unit inner stride, got {tuple(qkv.shape)}")
+        for w in (q_weight, k_weight):
+            _check(w is None or (w.dtype == torch.float32 and w.shape == (D,) and w.is_contiguous()),
+                   "qk_norm_rope_store: norm weights must be float32 [D]")
+        _check((q_weight is None) == (k_weight is None), "qk_norm_rope_store: give both norm weights or neither")
+        if table is not None:
+            _check(table.dtype == torch.float32 and table.is_contiguous() and table.shape[1:] == (D // 2, 2),
+                   "qk_norm_rope_store: rotary table must be float32 [P, D/2, 2]")
+        _check(_is_i32(positions, T), "qk_norm_rope_store: positions must be int32 [T]")
+        if store:
+            _check(_is_i32(slots, T), "qk_norm_rope_store: slots must be int32 [T]")
+            _check(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and k_cache.is_contiguous()
+                   and v_cache.is_contiguous(), "qk_norm_rope_store: caches must be contiguous and of the rows' dtype")
+            _check(k_cache.shape[1:] == (Hkv, page, D) and v_cache.shape[1:] == (Hkv, D, page),
+                   "qk_norm_rope_store: caches must be K [pages, Hkv, page, D] and V [pages, Hkv, D, page]")
+        core().call("me_qk_norm_rope_store", qkv.data_ptr(), _code(qkv.dtype), T, qkv.stride(0), _ptr(q_weight),
+                    _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0],
+                    positions.data_ptr(), _ptr(slots) if store else None, _ptr(k_cache) if store else None,
+                    _ptr(v_cache) if store else None, Hq, Hkv, D, page, int(store), _stream())
+
+    def store_kv(self, k, v, slots, k_cache, v_cache, page: int) -> None:
+        """Scatter k, v [T, Hkv, D] (views with a token stride are fine) into the pages; slots < 0
+        are skipped (reference csrc/kv_cache.cu:10-31; the copy is bit-exact)."""
+        T, Hkv, D = k.shape
+        _check(v.shape == k.shape and k.dtype == v.dtype == k_cache.dtype == v_cache.dtype, "store_kv: dtype/shape mismatch")
+        for t in (k, v):
+            _check(t.stride(2) == 1 and t.stride(1) == D, "store_kv: heads of a token must be one contiguous row")
+        _check(k_cache.shape[1:] == (Hkv, page, D) and v_cache.shape[1:] == (Hkv, D, page) and k_cache.is_contiguous()
+               and v_cache.is_contiguous(), "store_kv: caches must be K [pages, Hkv, page, D], V [pages, Hkv, D, page]")
+        _check(_is_i32(slots, T), "store_kv: slots must be int32 [T]")
+        core().call("me_store_kv", k.data_ptr(), v.data_ptr(), _code(k.dtype), T, k.stride(0), v.stride(0),
+                    slots.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), Hkv, D, page, _stream())
+
+    # -- attention -----------------------------------------------------------------------
+    def paged_attention(self, q, k_cache, v_cache, page: int, block_tables, context_lens, seq_of_token,
+                        positions, prefill_cu, num_decodes: int, max_decode_context: int, scale: float,
+                        window: int | None, Hq: int, Hkv: int, D: int, force_simple: bool = False):
+        """Causal attention of this step's tokens over the paged keys of their requests.
+
+        q: [T, Hq*D] (a strided view is fine). Rows are ordered decode requests first (one token
+        each, `num_decodes` of them), then the others; `prefill_cu` int32 [B - num_decodes + 1]
+        are prefix sums of the new-token counts of the others. `context_lens` int32 [B] counts keys
+        after this step's write; `block_tables` int32 [B, MB]. Returns [T, Hq*D].
+        (reference layers/attention.py:63-76: decode rows to the decode kernel, the rest to the
+        prefill kernel; csrc/paged_decode.cu, csrc/paged_prefill.cu.)"""
+        T = q.shape[0]
+        B = context_lens.numel()
+        _check(q.dim() == 2 and q.shape[1] == Hq * D and q.stride(1) == 1, "attention: q must be [T, Hq*D], unit inner stride")
+        _check(k_cache.shape[1:] == (Hkv, page, D) and v_cache.shape[1:] == (Hkv, D, page), "attention: cache layout mismatch")
+        _check(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "attention: cache dtype differs from q")
+        _check(block_tables.dim() == 2 and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
+               and block_tables.shape[0] >= B, "attention: block tables must be int32 [B, MB]")
+        _check(_is_i32(context_lens) and _is_i32(seq_of_token, T) and _is_i32(positions, T), "attention: metadata must be int32")
+        _check(0 <= num_decodes <= B and num_decodes <= T, "attention: bad decode count")
+        out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
+        win = int(window or 0)
+        mfma = (q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page % 8 == 0 and not force_simple)
+        if not mfma:
+            core().call("me_attn_simple", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _code(q.dtype),
+                        k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
+                        seq_of_token.data_ptr(), positions.data_ptr(), T, Hq, Hkv, D, page, float(scale), win, _stream())
+            return out
+        lib = attn_lib(D)
+        es = q.element_size()
+        if num_decodes > 0:
+            part_size, num_parts = decode_partitions(num_decodes, Hq, Hkv, max_decode_context)
+            scratch = _scratch(num_decodes * Hq * num_parts * (D + 2), q.device) if num_parts > 1 else None
+            lib.call("me_attn_decode", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_cache.data_ptr(),
+                     v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
+                     num_decodes, Hq, Hkv, page, float(scale), win, part_size, num_parts, _ptr(scratch), _stream())
+        if T > num_decodes:
+            _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
+            lib.call("me_attn_prefill", q.data_ptr() + num_decodes * q.stride(0) * es, q.stride(0),
+                     out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
+                     v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
+                     block_tables.stride(0), context_lens.data_ptr() + num_decodes * 4, prefill_cu.data_ptr(),
+                     B - num_decodes, T - num_decodes, Hq, Hkv, page, float(scale), win, _stream())
+        return out
+
+    # -- matrix products -----------------------------------------------------------------
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
+               allow_partials: bool = False):
+        """x [M, K] . w[N, K]^T (reference layers/linear.py:25-26: F.linear, no bias).
+
+        float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for M <= 64 or float32 output,
+        the library product (hipBLASLt through torch) above that, the FMA kernel for shapes the
+        MFMA kernel refuses. With allow_partials a skinny product with few output features may
+        split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
+        adds them."""
+        _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: {tuple(x.shape)} x {tuple(w.shape)}^T")
+        _check(x.dtype == w.dtype, f"linear: activation {x.dtype} and weight {w.dtype} differ")
+        _check(x.stride(1) == 1 and w.stride(1) == 1, "linear: rows must be contiguous")
+        M, K = x.shape
+        N = w.shape[0]
+        out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.float32:
+            _check(out_dtype == torch.float32, "linear: float32 inputs give float32 outputs")
+            y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+            core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
+                        ME_F32, ME_F32, M, N, K, _stream())
+            return y
+        aligned = (K % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+                   and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+        if not aligned:
+            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
+                        ME_BF16, _code(out_dtype), M, N, K, _stream())
+            return y
+        if M <= SKINNY_MAX_M or out_dtype == torch.float32:
+            ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= SKINNY_MAX_M) else 1
+            if ksplit > 1:
+                parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
+                core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
+                            ME_F32, parts.data_ptr(), ksplit, M, N, K, _stream())
+                return parts
+            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
+                        _code(out_dtype), None, 1, M, N, K, _stream())
+            return y
+        return torch.matmul(x, w.t())
+
+    # -- sampling ------------------------------------------------------------------------
+    def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:
+        """Token ids int32 [S] from float32 logits [S, V]: argmax where temperature is 0, else
+        argmax(logits/T - log E) with E ~ Exp(1) a hash of (keys[s], vocabulary id)
+        (reference layers/sampler.py:5-11)."""
+        S, V = logits.shape
+        _check(logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be float32 rows")
+        _check(temperatures.dtype == torch.float32 and temperatures.numel() == S and temperatures.is_contiguous(),
+               "sample: temperatures must be float32 [S]")
+        _check(keys.dtype == torch.int32 and keys.shape == (S, 2) and keys.is_contiguous(), "sample: keys must be int32 [S, 2]")
+        out = torch.empty((S,), dtype=torch.int32, device=logits.device)
+        core().call("me_sample", logits.data_ptr(), logits.stride(0), temperatures.data_ptr(), keys.data_ptr(),
+                    out.data_ptr(), S, V, _stream())
+        return out
+
+
+SKINNY_MAX_M = 64
+_TARGET_WORKGROUPS = 512
+_scratch_buf: dict = {}
+
+
+def _scratch(num_floats: int, device) -> torch.Tensor:
+    buf = _scratch_buf.get(device)
+    if buf is None or buf.numel() < num_floats:
+        buf = torch.empty((max(num_floats, 1 << 20),), dtype=torch.float32, device=device)
+        _scratch_buf[device] = buf
+    return buf
+
+
+def choose_ksplit(M: int, N: int, K: int) -> int:
+    """Workgroups over K for a skinny product: 1 when the N/16 feature tiles already fill the
+    compute units, else enough to reach the target, each split keeping >= 256 of K."""
+    tiles = -(-N // 16) * -(-M // 64)
+    if tiles >= _TARGET_WORKGROUPS // 2:
+        return 1
+    return max(1, min(-(-_TARGET_WORKGROUPS // tiles), K // 256, 8))
+
+
+def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int) -> tuple:
+    """(keys per partition, number of partitions) for the split decode kernel: enough workgroups
+    to fill the GPU's compute units, partitions of at least 128 keys (the reference's rule is
+    layers/ops.py:44-51: split when sequences x kv heads cannot fill the SMs, 256-key partitions)."""
+    col_tiles = (Hq // Hkv + 15) // 16
+    base = max(1, num_seqs * Hkv * col_tiles)
+    want = max(1, -(-_TARGET_WORKGROUPS // base))
+    part = max(128, -(-max(1, max_context) // want))
+    part = -(-part // 128) * 128
+    parts = max(1, -(-max(1, max_context) // part))
+    return part, parts
+
+
+# --------------------------------------------------------------------------- dispatch
+
+_backend = None
+
+
+def backend():
+    global _backend
+    if _backend is None:
+        _require_gpu()
+        _backend = HipBackend()
+    return _backend
+
+
+def set_backend(b) -> None:
+    """Install another object with HipBackend's methods (tests only); None restores the default."""
+    global _backend
+    _backend = b
+
+
+def gather_rows(*a, **k): return backend().gather_rows(*a, **k)
+def rms_norm(*a, **k): return backend().rms_norm(*a, **k)
+def silu_and_mul(*a, **k): return backend().silu_and_mul(*a, **k)
+def qk_norm_rope_store(*a, **k): return backend().qk_norm_rope_store(*a, **k)
+def store_kv(*a, **k): return backend().store_kv(*a, **k)
+def paged_attention(*a, **k): return backend().paged_attention(*a, **k)
+def linear(*a, **k): return backend().linear(*a, **k)
+def sample(*a, **k): return backend().sample(*a, **k)

@@ -1,0 +1,212 @@
+"""What every model part is: a small tree of named parameters plus a forward.
+
+A model is assembled from parts (mixer, feed-forward, norm, position encoding,
+embedding/head, block arrangement). A part takes its sizes and constants as
+constructor arguments, declares the parameters it needs (`ParamSpec`), and never
+learns which model it sits in. The weight loader fills declared parameters by
+name; the step function hands each part the per-step metadata it may need.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Iterator
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One parameter tensor of a part.
+
+    ``init`` names the distribution used by the random-weights mode:
+    ``"matrix"`` ~ N(0, 0.02) (linears, embeddings), ``"norm"`` ~ 1 + U(-0.1, 0.1).
+    ``dtype`` is ``"compute"`` (the engine's dtype: bfloat16 or float32),
+    ``"float32"`` (always 32-bit: norm weights, exact for both stored forms) or
+    ``"int32"`` (integer tables).
+    """
+
+    shape: tuple
+    init: str = "matrix"
+    dtype: str = "compute"
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a mixer wants from the paged key/value cache.
+
+    ``window``: None keeps every key; n keeps the last n positions (pages that
+    the window has passed are given back). Layers with equal needs share one
+    group of pages and one block table per request.
+    """
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+    def group_key(self) -> tuple:
+        return (self.num_kv_heads, self.head_dim, self.window)
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Fixed-size per-request state of a mixer: one tensor ``[num_slots, *shape]``."""
+
+    shape: tuple
+    dtype: str = "float32"
+
+
+class Part:
+    """Base of all parts: named parameters and named child parts."""
+
+    def __init__(self):
+        self._specs: dict[str, ParamSpec] = {}
+        self._children: dict[str, "Part"] = {}
+
+    # -- declaration -------------------------------------------------------
+    def add_param(self, name: str, spec: ParamSpec) -> None:
+        self._specs[name] = spec
+        setattr(self, name, None)
+
+    def add_child(self, name: str, part: "Part") -> "Part":
+        self._children[name] = part
+        setattr(self, name, part)
+        return part
+
+    # -- traversal ---------------------------------------------------------
+    def named_specs(self, prefix: str = "") -> Iterator[tuple]:
+        """Yield (full name, owning part, local name, spec) over the whole tree."""
+        seen: set[int] = set()
+        yield from self._named_specs(prefix, seen)
+
+    def _named_specs(self, prefix, seen):
+        if id(self) in seen:        # a part shared by several parents declares its parameters once
+            return
+        seen.add(id(self))
+        for local, spec in self._specs.items():
+            yield prefix + local, self, local, spec
+        for cname, child in self._children.items():
+            yield from child._named_specs(prefix + cname + ".", seen)
+
+    def parts(self) -> Iterator["Part"]:
+        seen: set[int] = set()
+        stack = [self]
+        while stack:
+            p = stack.pop()
+            if id(p) in seen:
+                continue
+            seen.add(id(p))
+            yield p
+            stack.extend(p._children.values())
+
+    # -- binding -----------------------------------------------------------
+    def set_param(self, local: str, tensor: torch.Tensor) -> None:
+        spec = self._specs[local]
+        if tuple(tensor.shape) != tuple(spec.shape):
+            raise ValueError(f"{type(self).__name__}.{local}: shape {tuple(tensor.shape)} != {tuple(spec.shape)}")
+        setattr(self, local, tensor)
+
+    def finalize(self, device: torch.device, dtype: torch.dtype, max_positions: int) -> None:
+        """Called once after all parameters are bound (build tables, derived layouts)."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, residual: torch.Tensor | None):
+        """-> (normalised x in the compute dtype, new residual in float32).
+
+        ``residual`` None starts the residual stream from ``x``; otherwise the new
+        residual is ``x + residual`` (summed in 32-bit) and that sum is normalised.
+        """
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Something applied to queries and keys as a function of token positions."""
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
+        """Rotate/shift ``q`` [T, Hq, D] and ``k`` [T, Hkv, D] in place."""
+        raise NotImplementedError
+
+    def rotary_table(self) -> torch.Tensor | None:
+        """[P, D/2, 2] float32 (cos, sin) if this is a half-split rotary encoding that the
+        fused query/key kernel can apply; None means ``apply`` must be called."""
+        return None
+
+
+class Mixer(Part):
+    """Token mixing: the only part that looks at other positions of a request."""
+
+    def cache_need(self) -> CacheNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(self, x: torch.Tensor, step, cache, state) -> torch.Tensor:
+        """x: [T, hidden] -> [T, hidden].
+
+        ``step``: the `StepContext` of this step. ``cache``: a `CacheView` (pages of this
+        call's layer, or of the layer it reads) or None. ``state``: this call's state
+        tensor ``[num_slots, *shape]`` or None; rows are ``step.state_slots``.
+        """
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+@dataclass
+class LayerCall:
+    """One entry of a model's run order.
+
+    ``layer``: index into the model's layers (a layer may be named by several
+    entries: its weights are then shared, each entry has a cache of its own).
+    ``cache_of``: index of an *earlier entry* whose cache this entry reads
+    instead of owning one; it then writes nothing.
+    """
+
+    layer: int
+    cache_of: int | None = None
+
+
+@dataclass
+class CacheView:
+    """The pages one layer call reads and writes."""
+
+    group: int                 # index of the page group (selects block table and slot mapping)
+    k: torch.Tensor            # [num_pages, Hkv, page, D]
+    v: torch.Tensor            # [num_pages, Hkv, D, page]  (transposed within a page)
+    page_size: int
+    write: bool = True
+
+
+# ---------------------------------------------------------------- registries
+
+_REGISTRIES: dict[str, dict[str, type]] = {
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position_encoding": {}, "block": {},
+}
+
+
+def register_part(kind: str, name: str):
+    """Class decorator: make a part constructible by ``make_part(kind, name, ...)``."""
+    if kind not in _REGISTRIES:
+        raise KeyError(f"unknown part kind {kind!r}; kinds: {sorted(_REGISTRIES)}")
+
+    def deco(cls):
+        _REGISTRIES[kind][name] = cls
+        return cls
+
+    return deco
+
+
+def make_part(kind: str, name: str, **kwargs) -> Part:
+    try:
+        cls = _REGISTRIES[kind][name]
+    except KeyError:
+        raise KeyError(f"no {kind} named {name!r}; registered: {sorted(_REGISTRIES.get(kind, {}))}") from None
+    return cls(**kwargs)
+
+
+def registered(kind: str) -> list:
+    return sorted(_REGISTRIES[kind])

@@ -1,0 +1,25 @@
+"""Dense gated feed-forward (reference models/qwen3.py:42-51)."""
+from __future__ import annotations
+
+from ..kernels import ops
+from .base import FeedForward, register_part
+from .linear import Linear
+
+
+@register_part("feed_forward", "swiglu")
+class SwiGLU(FeedForward):
+    """down(silu(gate(x)) * up(x)); gate and up are one packed product with gate's rows first
+    (reference layers/linear.py:29-45, layers/activation.py:5-7)."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.add_child("gate_up", Linear(hidden_size, 2 * intermediate_size,
+                                         parts={"gate": intermediate_size, "up": intermediate_size}))
+        self.add_child("down", Linear(intermediate_size, hidden_size))
+
+    def forward(self, x):
+        gu = self.gate_up.forward(x)
+        act = ops.silu_and_mul(gu)
+        return self.down.forward(act, allow_partials=True)

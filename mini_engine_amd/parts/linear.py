@@ -1,0 +1,24 @@
+"""Bias-free linear maps with weights stored [out, in] (reference layers/linear.py:4-45)."""
+from __future__ import annotations
+
+from ..kernels import ops
+from .base import ParamSpec, Part
+
+
+class Linear(Part):
+    """y = x . W^T. `parts` names row blocks of W that are stored separately in a checkpoint
+    (packed projections: reference layers/linear.py:13-22,37-42); the loader concatenates them."""
+
+    def __init__(self, in_features: int, out_features: int, parts: dict | None = None):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.row_blocks = dict(parts) if parts else None   # name -> rows, in storage order
+        if self.row_blocks is not None and sum(self.row_blocks.values()) != out_features:
+            raise ValueError("row blocks do not add up to out_features")
+        self.add_param("weight", ParamSpec((out_features, in_features), init="matrix", dtype="compute"))
+
+    def forward(self, x, out_dtype=None, allow_partials: bool = False):
+        """With allow_partials the result may be float32 partial sums [P, M, N] (a product whose K
+        range was split over workgroups); the consumer, a norm, adds them."""
+        return ops.linear(x, self.weight, out_dtype, allow_partials)

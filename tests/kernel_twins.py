@@ -1,0 +1,145 @@
+"""Plain torch twins of every kernel: same arguments and cache layout, straightforward math.
+
+Two uses: (1) each HIP kernel is compared with its twin on the GPU; (2) installed as the
+ops backend (`PlainBackend`) they let the engine's bookkeeping (step function, cache manager,
+scheduler, replay) be exercised on a machine without a GPU. They are test code: the engine
+itself has no implementation but the HIP kernels.
+
+All arithmetic is float32 (or float64 where a test asks), whatever the storage dtype; results
+are rounded once to the output dtype.
+"""
+from __future__ import annotations
+
+import torch
+
+
+def gather_rows(src, idx):
+    return src[idx.long()].clone()
+
+
+def rms_norm(x, weight, eps, residual, out_dtype, want_residual=True):
+    r = x.float().sum(0) if x.dim() == 3 else x.float()
+    if residual is not None:
+        r = r + residual
+    y = weight * (r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps))
+    return y.to(out_dtype), (r if want_residual else None)
+
+
+def silu_and_mul(gu):
+    inter = gu.shape[1] // 2
+    g, u = gu[:, :inter].float(), gu[:, inter:].float()
+    return (g * torch.sigmoid(g) * u).to(gu.dtype)
+
+
+def _norm_rope(x, w, eps, table, positions):
+    """x: [T, H, D] float32."""
+    if w is not None:
+        x = w * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps))
+    if table is not None:
+        cs = table[positions.long()]                        # [T, D/2, 2]
+        c, s = cs[..., 0].unsqueeze(1), cs[..., 1].unsqueeze(1)
+        half = x.shape[-1] // 2
+        x1, x2 = x[..., :half], x[..., half:]
+        x = torch.cat((x1 * c - x2 * s, x2 * c + x1 * s), dim=-1)
+    return x
+
+
+def write_pages(k, v, slots, k_cache, v_cache, page):
+    """k, v: [T, Hkv, D] -> K [pages, Hkv, page, D], V [pages, Hkv, D, page]."""
+    keep = slots >= 0
+    s = slots[keep].long()
+    pg, off = s // page, s % page
+    k_cache[pg, :, off, :] = k[keep].to(k_cache.dtype)
+    v_cache[pg, :, :, off] = v[keep].to(v_cache.dtype)
+
+
+def qk_norm_rope_store(qkv, q_weight, k_weight, eps, table, positions, slots, k_cache, v_cache,
+                       Hq, Hkv, D, page, store=True):
+    T = qkv.shape[0]
+    q = _norm_rope(qkv[:, :Hq * D].float().view(T, Hq, D), q_weight, eps, table, positions)
+    if Hkv:
+        k = _norm_rope(qkv[:, Hq * D:(Hq + Hkv) * D].float().view(T, Hkv, D), k_weight, eps, table, positions)
+    qkv[:, :Hq * D] = q.reshape(T, Hq * D).to(qkv.dtype)
+    if store:
+        v = qkv[:, (Hq + Hkv) * D:].view(T, Hkv, D)
+        write_pages(k.to(qkv.dtype), v, slots, k_cache, v_cache, page)
+    elif Hkv:
+        qkv[:, Hq * D:(Hq + Hkv) * D] = k.reshape(T, Hkv * D).to(qkv.dtype)
+
+
+def store_kv(k, v, slots, k_cache, v_cache, page):
+    write_pages(k, v, slots, k_cache, v_cache, page)
+
+
+def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_of_token, positions,
+                    prefill_cu, num_decodes, max_decode_context, scale, window, Hq, Hkv, D,
+                    force_simple=False, compute_dtype=torch.float32):
+    """Token by token: gather the keys this token may see through its request's block table
+    and nothing else (so unowned pages are never read), softmax, weighted sum."""
+    T = q.shape[0]
+    out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
+    G = Hq // Hkv
+    for t in range(T):
+        b = int(seq_of_token[t])
+        pos = int(positions[t])
+        lo = max(0, pos - window + 1) if window else 0
+        js = torch.arange(lo, pos + 1, device=q.device)
+        pages = block_tables[b, (js // page).long()].long()
+        assert (pages >= 0).all(), "attention would read a page the request does not hold"
+        offs = js % page
+        k = k_cache[pages, :, offs, :].to(compute_dtype)             # [n, Hkv, D]
+        v = v_cache[pages, :, :, offs].to(compute_dtype)             # [n, Hkv, D]
+        qt = q[t].to(compute_dtype).view(Hq, D)
+        for h in range(Hq):
+            kh = h // G
+            s = (k[:, kh, :] @ qt[h]) * scale
+            p = torch.softmax(s, dim=0)
+            out[t, h * D:(h + 1) * D] = (p @ v[:, kh, :]).to(q.dtype)
+    return out
+
+
+def linear(x, w, out_dtype=None, allow_partials=False):
+    return (x.float() @ w.float().t()).to(out_dtype or x.dtype)
+
+
+def _fmix32(h):
+    m = 0xFFFFFFFF
+    h = h & m
+    h ^= h >> 16
+    h = (h * 0x85EBCA6B) & m
+    h ^= h >> 13
+    h = (h * 0xC2B2AE35) & m
+    h ^= h >> 16
+    return h
+
+
+def exp_noise(keys, V, device):
+    """E ~ Exp(1), [S, V], the kernel's hash: fmix32(fmix32(v ^ k0) + k1) -> 24 bits -> -log(u)."""
+    k = keys.to(torch.int64) & 0xFFFFFFFF
+    v = torch.arange(V, dtype=torch.int64, device=device)[None, :]
+    r = _fmix32((_fmix32(v ^ k[:, 0:1]) + k[:, 1:2]) & 0xFFFFFFFF)
+    u = ((r >> 8).to(torch.float32) + 0.5) * (1.0 / 16777216.0)
+    return -torch.log(u)
+
+
+def sample_scores(logits, temperatures, keys):
+    """The quantity whose argmax the sampler returns, [S, V] float32."""
+    t = temperatures[:, None]
+    noisy = logits / torch.where(t > 0, t, torch.ones_like(t)) - torch.log(exp_noise(keys, logits.shape[1], logits.device))
+    return torch.where(t > 0, noisy, logits)
+
+
+def sample(logits, temperatures, keys):
+    return sample_scores(logits, temperatures, keys).argmax(dim=-1).to(torch.int32)
+
+
+class PlainBackend:
+    name = "plain"
+    gather_rows = staticmethod(gather_rows)
+    rms_norm = staticmethod(rms_norm)
+    silu_and_mul = staticmethod(silu_and_mul)
+    qk_norm_rope_store = staticmethod(qk_norm_rope_store)
+    store_kv = staticmethod(store_kv)
+    paged_attention = staticmethod(paged_attention)
+    linear = staticmethod(linear)
+    sample = staticmethod(sample)
