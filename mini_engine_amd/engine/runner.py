@@ -164,7 +164,7 @@ class ModelRunner:
                 t = tables[g][j]
                 bt[j, :len(t)] = t
                 p = pos[cu[j]:cu[j + 1]]
-                pages = bt[j, p // ps]
+                pages = bt[j, p // ps] if p[-1] // ps < MB[g] else np.array([-1])
                 if (pages < 0).any():
                     raise RuntimeError(f"request {entries[order[j]].req!r} has no page for a position it is "
                                        f"about to write (group {g}); allocate before stepping")

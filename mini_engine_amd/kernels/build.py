@@ -72,9 +72,8 @@ def _hash(sources: list, extra: list) -> str:
 def _writable_dir(path: str) -> bool:
     try:
         os.makedirs(path, exist_ok=True)
-        probe = os.path.join(path, f".w{os.getpid()}")
-        with open(probe, "w"):
-            pass
+        fd, probe = tempfile.mkstemp(prefix=".w", dir=path)
+        os.close(fd)
         os.remove(probe)
         return True
     except OSError:

@@ -1,0 +1,39 @@
+"""Greedy and temperature sampling (reference layers/sampler.py:4-11).
+
+The reference draws exponential noise for the whole [S, V] matrix from the global generator,
+so a request's tokens depend on who shares its batch. Here the noise is a hash of
+(seed, request, output index, vocabulary id): the same request gives the same tokens under any
+batching, chunking or preemption.
+"""
+from __future__ import annotations
+
+_MASK64 = (1 << 64) - 1
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK64
+    x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & _MASK64
+    x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & _MASK64
+    return x ^ (x >> 31)
+
+
+def row_key(seed: int, request: int, output_index: int) -> tuple:
+    """Two 32-bit words that key the noise of one sampled token."""
+    x = _splitmix64(seed & _MASK64)
+    x = _splitmix64(x ^ (request & _MASK64))
+    x = _splitmix64(x ^ (output_index & _MASK64))
+    return x & 0xFFFFFFFF, x >> 32
+
+
+class Sampler:
+    def __init__(self, runner, seed: int = 0):
+        self.runner = runner
+        self.seed = seed
+
+    def __call__(self, logits, seqs: list) -> list:
+        """One token per row of float32 logits [S, V]; seqs[s] gives temperature, seed, identity
+        and how many tokens the request has generated so far."""
+        temps = [s.sampling_params.temperature for s in seqs]
+        keys = [row_key(self.seed if s.sampling_params.seed is None else s.sampling_params.seed,
+                        s.sample_stream, s.num_completion_tokens) for s in seqs]
+        return self.runner.sample(logits, temps, keys)

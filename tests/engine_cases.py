@@ -1,0 +1,177 @@
+"""The engine against the plain implementation under every way of cutting the work.
+Each case takes `env`, an object with .device, .dtype, .tol and .runner(name, pages) ->
+(runner, manager, folder); the same cases run on the CPU (plain kernel twins, float32)
+and on the GPU (HIP kernels, float32 and bfloat16). Every pool is filled with NaN first,
+so a read of a key that the request does not own poisons its logits.
+"""
+from __future__ import annotations
+
+import torch
+
+import helpers
+from helpers import Driver, plain_logits, random_ids, rel_err
+
+
+def _vocab(name):
+    return helpers.CONFIGS[name]["vocab_size"]
+
+
+def _check(env, folder, ids, got, what):
+    ref = plain_logits(folder, ids)[: got.shape[0]]
+    err = rel_err(got, ref)
+    assert err <= env.tol, f"{what}: error {err:.3g} > {env.tol:g}; first bad position {helpers.first_bad_row(got, ref, env.tol)}"
+
+
+def whole(env, name):
+    """Each request alone and whole, lengths around page and tile edges."""
+    page = helpers.PAGE[name]
+    for n in (1, 2, page - 1, page, page + 1, 31, 32, 33, 64, 65, 97, 130):
+        runner, manager, folder = env.runner(name, -(-n // page))
+        ids = random_ids(n, _vocab(name), 100 + n)
+        d = Driver(runner, manager)
+        d.step({"r": ids}, end=["r"])
+        _check(env, folder, ids, d.result("r"), f"{name} whole n={n}")
+
+
+def tail_one_by_one(env, name):
+    """Most of a request in one step, its last 32 tokens one by one."""
+    page = helpers.PAGE[name]
+    for n in (33, 40, 100, 161):
+        runner, manager, folder = env.runner(name, -(-n // page))
+        ids = random_ids(n, _vocab(name), 200 + n)
+        d = Driver(runner, manager)
+        head = n - 32
+        d.step({"r": ids[:head]})
+        for t in range(head, n):
+            d.step({"r": ids[t:t + 1]})
+        _check(env, folder, ids, d.result("r"), f"{name} tail n={n}")
+
+
+def changing_portions(env, name):
+    """Portions of changing size, down to two tokens and one."""
+    page = helpers.PAGE[name]
+    n = 150
+    ids = random_ids(n, _vocab(name), 300)
+    for pattern in ([2, 3, 5, 8, 13, 21, 34, 2, 2], [17, 2, 40, 1, 1, 2, 31, 16, 16, 2], [page, page, 2, page + 1, page - 1]):
+        runner, manager, folder = env.runner(name, -(-n // page))
+        d = Driver(runner, manager)
+        pos, i = 0, 0
+        while pos < n:
+            c = min(pattern[i % len(pattern)], n - pos)
+            d.step({"r": ids[pos:pos + c]})
+            pos += c; i += 1
+        _check(env, folder, ids, d.result("r"), f"{name} portions {pattern}")
+
+
+def mixed_with_reuse(env, name):
+    """Up to four live requests: portions of some beside single decoded tokens of others, in a
+    pool so small that pages are used again by later requests while others are still live."""
+    page = helpers.PAGE[name]
+    V = _vocab(name)
+    lens = {"a": 70, "b": 45, "c": 33, "d": 97, "e": 58, "f": 21, "g": 80}
+    ids = {r: random_ids(n, V, 400 + i) for i, (r, n) in enumerate(lens.items())}
+    need = lambda r: -(-lens[r] // page)
+    # pool: enough for the four largest live at once, less than all seven together
+    pages = need("a") + need("d") + need("g") + need("e")
+    runner, manager, folder = env.runner(name, pages)
+    d = Driver(runner, manager)
+    waiting = list(lens)
+    live, pos = [], {}
+    # chunk plan per request: a prompt part in changing portions, then the rest token by token
+    portions = {"a": [30, 2, 20], "b": [45 - 12], "c": [2, 2, 9], "d": [50, 17, 2], "e": [7, 31], "f": [3], "g": [64]}
+    step_i = 0
+    used_again = False
+    seen_pages: set = set()
+    while waiting or live:
+        while waiting and len(live) < 4:
+            r = waiting[0]
+            held = sum(len([p for p in manager.block_table(x) if p >= 0]) for x in live)
+            if held + need(r) > pages:
+                break
+            waiting.pop(0); live.append(r); pos[r] = 0
+            assert manager.allocate(r, 0, lens[r])          # reserve its pages so the plan cannot run dry
+            t = set(manager.block_table(r))
+            used_again |= bool(t & seen_pages)
+            seen_pages |= t
+        parts, ended = {}, []
+        for r in live:
+            plan = portions[r]
+            k = len([1 for _ in range(0)])
+            if plan:
+                c = plan.pop(0)
+            else:
+                c = 1
+            c = min(c, lens[r] - pos[r])
+            parts[r] = ids[r][pos[r]:pos[r] + c]
+            pos[r] += c
+            if pos[r] == lens[r]:
+                ended.append(r)
+        d.step(parts, end=ended)
+        for r in ended:
+            live.remove(r)
+        step_i += 1
+        assert step_i < 1000
+    assert used_again, "the pool was large enough that no page was used twice: the case tests nothing"
+    for r in lens:
+        _check(env, folder, ids[r], d.result(r), f"{name} mixed request {r}")
+    assert all(manager.num_free_pages(g) == manager.num_pages(g) for g in range(manager.num_groups))
+
+
+def long_decode(env, name):
+    """A short prompt, then hundreds of tokens one by one (page edges, split partitions)."""
+    page = helpers.PAGE[name]
+    n = 420
+    ids = random_ids(n, _vocab(name), 500)
+    runner, manager, folder = env.runner(name, -(-n // page))
+    d = Driver(runner, manager)
+    d.step({"r": ids[:3]})
+    for t in range(3, n):
+        d.step({"r": ids[t:t + 1]})
+    _check(env, folder, ids, d.result("r"), f"{name} long decode")
+
+
+def batch_of_decodes(env, name):
+    """Several requests of different lengths decoding together, contexts across partition sizes."""
+    page = helpers.PAGE[name]
+    V = _vocab(name)
+    lens = {"a": 300, "b": 17, "c": 129, "d": 64}
+    ids = {r: random_ids(n + 8, V, 600 + i) for i, (r, n) in enumerate(lens.items())}
+    runner, manager, folder = env.runner(name, sum(-(-(n + 8) // page) for n in lens.values()))
+    d = Driver(runner, manager)
+    d.step({r: ids[r][:lens[r]] for r in lens})
+    for t in range(8):
+        d.step({r: ids[r][lens[r] + t: lens[r] + t + 1] for r in lens})
+    for r in lens:
+        _check(env, folder, ids[r], d.result(r), f"{name} decode batch request {r}")
+
+
+def first_tokens(env, name):
+    """The first tokens of a sequence, one by one from position 0."""
+    ids = random_ids(6, _vocab(name), 700)
+    runner, manager, folder = env.runner(name, 2)
+    d = Driver(runner, manager)
+    for t in range(6):
+        d.step({"r": ids[t:t + 1]})
+    _check(env, folder, ids, d.result("r"), f"{name} first tokens")
+
+
+def wanted_rows_only(env, name):
+    """Logits only where asked, in the order of entries and of `want`; none asked gives None."""
+    from mini_engine_amd.engine.runner import StepEntry
+    V = _vocab(name)
+    a, b = random_ids(20, V, 800), random_ids(9, V, 801)
+    runner, manager, folder = env.runner(name, 8)
+    assert manager.allocate("a", 0, 20) and manager.allocate("b", 0, 9)
+    out = runner.step([StepEntry("a", a, 0, [19, 0, 7]), StepEntry("b", b[:8], 0, [])])
+    ref = plain_logits(folder, a)
+    assert out.shape == (3, V)
+    assert rel_err(out, ref[[19, 0, 7]]) <= env.tol
+    out = runner.step([StepEntry("b", b[8:], 8, [0])])          # a decode entry listed alone
+    assert rel_err(out, plain_logits(folder, b)[8:9]) <= env.tol
+    manager.free("a")
+    assert manager.allocate("a", 0, 20)
+    assert runner.step([StepEntry("a", a, 0, [])]) is None
+
+
+ALL = [whole, tail_one_by_one, changing_portions, mixed_with_reuse, long_decode, batch_of_decodes, first_tokens,
+       wanted_rows_only]

@@ -1,0 +1,152 @@
+"""The engine's bookkeeping (model assembly, step function, cache manager, replay, scheduler,
+entry point) on the CPU, with the plain twins of the kernels, in float32."""
+import io
+import json
+import os
+
+import pytest
+import torch
+
+import engine_cases
+import helpers
+import plain_qwen3
+from mini_engine_amd.cache.manager import CacheManager
+from mini_engine_amd.engine.runner import ModelRunner, StepEntry
+from mini_engine_amd.weights.loader import load_model
+
+
+class Env:
+    device, dtype, tol = "cpu", torch.float32, helpers.TOL_F32
+
+    def __init__(self, folders):
+        self.folders = folders
+        self.models = {}
+
+    def runner(self, name, pages):
+        folder = self.folders(name)
+        if name not in self.models:
+            self.models[name] = load_model(folder, self.device, self.dtype, 512)
+        model = self.models[name]
+        manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
+        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True), manager, folder
+
+
+@pytest.fixture(scope="module")
+def env(folders):
+    return Env(folders)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("case", [c for c in engine_cases.ALL if c.__name__ not in ("long_decode",)], ids=lambda c: c.__name__)
+def test_cuts(env, plain_backend, case, name):
+    case(env, name)
+
+
+def test_runner_refuses_bad_input(env, plain_backend):
+    runner, manager, _ = env.runner("A", 4)
+    assert manager.allocate("r", 0, 3)
+    with pytest.raises(ValueError, match="token id"):
+        runner.step([StepEntry("r", [1, 2, 999], 0, [])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.step([StepEntry("r", [1], 0, []), StepEntry("r", [2], 1, [])])
+    with pytest.raises(ValueError, match="wanted place"):
+        runner.step([StepEntry("r", [1, 2], 0, [2])])
+    with pytest.raises(ValueError, match="limit"):
+        runner.step([StepEntry("r", [1], 600, [])])
+    with pytest.raises(RuntimeError, match="no page"):
+        runner.step([StepEntry("r", list(range(40)), 0, [])])      # only 3 tokens were allocated
+
+
+def _llm(folder, **kw):
+    from mini_engine_amd import LLM
+    return LLM(folder, dtype="float32", device="cpu", poison_cache=True, **kw)
+
+
+def test_generate_greedy_matches_plain(folders, plain_backend):
+    """Tiny A as BASELINE names it: prompts 5/17/33, 8 greedy tokens each."""
+    from mini_engine_amd import SamplingParams
+    folder = folders("A")
+    cfg, w = plain_qwen3.read_model_folder(folder, torch.float64)
+    prompts = [helpers.random_ids(n, 256, 900 + n) for n in (5, 17, 33)]
+    llm = _llm(folder, kvcache_block_size=16, num_kvcache_blocks=12, max_num_seqs=4, max_num_batched_tokens=64, max_model_len=64)
+    outs = llm.generate(prompts, SamplingParams(temperature=0, max_tokens=8), use_tqdm=False)
+    for p, o in zip(prompts, outs):
+        assert o["token_ids"] == plain_qwen3.greedy_generate(cfg, w, p, 8)
+    llm.manager.check_invariants()
+    assert llm.manager.num_free_pages() == 12
+
+
+def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(folders, plain_backend):
+    """Tiny B as BASELINE names it: prompts 1/9/24/40/63, budget 16, temperature 0.8, 12 tokens.
+    The same seed must give the same tokens whether requests run together under a tight budget,
+    alone, or through a pool so small that requests are preempted and recomputed."""
+    from mini_engine_amd import SamplingParams
+    folder = folders("B")
+    prompts = [helpers.random_ids(n, 384, 950 + n) for n in (1, 9, 24, 40, 63)]
+    sp = SamplingParams(temperature=0.8, max_tokens=12, ignore_eos=True)
+    common = dict(kvcache_block_size=8, max_num_seqs=16, max_model_len=128, seed=3)
+    together = _llm(folder, num_kvcache_blocks=64, max_num_batched_tokens=16, **common)
+    out_together = [o["token_ids"] for o in together.generate(prompts, sp, use_tqdm=False)]
+    assert all(len(o) == 12 for o in out_together)
+    alone = _llm(folder, num_kvcache_blocks=64, max_num_batched_tokens=128, **common)
+    for i, p in enumerate(prompts):
+        seq = alone.add_request(p, sp, sample_stream=i)
+        toks = None
+        while not alone.is_finished():
+            for sid, t in alone.step()[0]:
+                toks = t
+        assert toks == out_together[i], f"request {i} differs when run alone"
+    tight = _llm(folder, num_kvcache_blocks=21, max_num_batched_tokens=16, enable_prefix_caching=False, **common)
+    out_tight = [o["token_ids"] for o in tight.generate(prompts, sp, use_tqdm=False)]
+    assert tight.scheduler.num_preemptions > 0, "the pool was large enough that nothing was preempted"
+    assert out_tight == out_together
+    other_seed = _llm(folder, num_kvcache_blocks=64, max_num_batched_tokens=16, **dict(common, seed=4))
+    assert [o["token_ids"] for o in other_seed.generate(prompts, sp, use_tqdm=False)] != out_together
+
+
+def test_prefix_hits_give_the_same_tokens(folders, plain_backend):
+    from mini_engine_amd import SamplingParams
+    folder = folders("A")
+    shared = helpers.random_ids(40, 256, 990)
+    prompts = [shared + helpers.random_ids(5, 256, 991), shared + helpers.random_ids(9, 256, 992)]
+    sp = SamplingParams(temperature=0, max_tokens=6)
+    kw = dict(kvcache_block_size=16, num_kvcache_blocks=16, max_num_seqs=4, max_num_batched_tokens=256, max_model_len=128)
+    cold = _llm(folder, enable_prefix_caching=False, **kw)
+    want = [o["token_ids"] for o in cold.generate(prompts, sp, use_tqdm=False)]
+    warm = _llm(folder, **kw)
+    first = warm.generate(prompts[:1], sp, use_tqdm=False)[0]["token_ids"]
+    sid = warm.add_request(prompts[1], sp)
+    seqs = warm.scheduler.waiting
+    assert warm.manager.find_prefix_hit(prompts[1]).num_pages == 2          # 32 of the 40 shared tokens
+    second = None
+    while not warm.is_finished():
+        for _, t in warm.step()[0]:
+            second = t
+    assert [first, second] == want
+
+
+def test_replay_program_on_cpu(folders, plain_backend, tmp_path, monkeypatch, capsys):
+    """bin/trace_run's loop, in process: steps from stdin, <step>.f32 files, `done` lines."""
+    from mini_engine_amd import replay
+    folder = folders("B")
+    a, b = helpers.random_ids(30, 384, 1), helpers.random_ids(12, 384, 2)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:20], "want": [19]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[20:21], "want": [0]}, {"id": "b", "tokens": b[:7], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[7:], "want": [0, 4]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[21:], "want": list(range(9))}], "end": ["a"]},
+    ]
+    monkeypatch.setattr("sys.stdin", io.StringIO("\n".join(json.dumps(s) for s in steps) + "\n"))
+    real = replay.Replayer
+    monkeypatch.setattr(replay, "Replayer", lambda m, d, n, p: real(m, d, n, p, device="cpu", poison_cache=True))
+    assert replay.main(["--model", folder, "--dtype", "float32", "--out", str(tmp_path / "o"), "--max-tokens", "128",
+                        "--page-size", "8"]) == 0
+    assert capsys.readouterr().out.split("\n")[:4] == ["done 0", "done 1", "done 2", "done 3"]
+    import numpy as np
+    ra, rb = helpers.plain_logits(folder, a), helpers.plain_logits(folder, b)
+    def rd(i):
+        return torch.from_numpy(np.fromfile(str(tmp_path / "o" / f"{i}.f32"), dtype="<f4").reshape(-1, 384))
+    assert helpers.rel_err(rd(0), ra[19:20]) <= helpers.TOL_F32
+    assert helpers.rel_err(rd(1), ra[20:21]) <= helpers.TOL_F32
+    assert helpers.rel_err(rd(2), rb[[7, 11]]) <= helpers.TOL_F32
+    assert helpers.rel_err(rd(3), ra[21:]) <= helpers.TOL_F32

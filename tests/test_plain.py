@@ -1,0 +1,189 @@
+"""Pins the plain implementation by what fixes it beside the reference's text: special cases
+that reduce to library routines, and invariants, each chosen so that a plausible mistake
+(a wrong sign or pairing, a norm in the wrong place, a wrong head grouping) fails it.
+
+The reference publishes no test vectors (its checks are git-ignored, reference .gitignore:10-12),
+so none can be used here: parity with its numbers is unpinned, parity with its formulas is
+what these tests hold.
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import helpers
+import plain_qwen3 as P
+
+torch.manual_seed(0)
+D64 = torch.float64
+
+
+def test_rms_norm_is_library_rms_norm():
+    x = torch.randn(5, 7, 24, dtype=D64)
+    w = torch.rand(24, dtype=D64) + 0.5
+    got = P.rms_norm(x, w, 1e-5)
+    assert torch.allclose(got, F.rms_norm(x, (24,), w, 1e-5), atol=1e-12)
+    # weight is a plain multiplier (a "1 + w" convention would double this)
+    assert torch.allclose(P.rms_norm(x, torch.ones(24, dtype=D64), 0.0).pow(2).mean(-1),
+                          torch.ones(5, 7, dtype=D64), atol=1e-12)
+    # eps sits inside the square root, added to the mean of squares
+    tiny = torch.full((1, 4), 1e-4, dtype=D64)
+    assert torch.allclose(P.rms_norm(tiny, torch.ones(4, dtype=D64), 1e-6),
+                          tiny / math.sqrt(1e-8 + 1e-6), atol=1e-12)
+
+
+def test_add_rms_norm_returns_sum_as_residual():
+    x, r = torch.randn(3, 8, dtype=D64), torch.randn(3, 8, dtype=D64)
+    w = torch.rand(8, dtype=D64)
+    y, res = P.add_rms_norm(x, r, w, 1e-6)
+    assert torch.equal(res, x + r)
+    assert torch.allclose(y, P.rms_norm(x + r, w, 1e-6))
+
+
+def test_rope_tables_and_pairing():
+    Dh, n, theta = 16, 50, 10000.0
+    cos, sin = P.rope_tables(Dh, n, theta)
+    inv = theta ** (-torch.arange(0, Dh, 2, dtype=D64) / Dh)
+    ang = torch.outer(torch.arange(n, dtype=D64), inv)
+    assert torch.allclose(cos[:, :Dh // 2], ang.cos()) and torch.allclose(cos[:, Dh // 2:], ang.cos())
+    assert torch.allclose(sin[:, Dh // 2:], ang.sin())
+    x = torch.randn(n, 3, Dh, dtype=D64)
+    pos = torch.arange(n)
+    y = P.apply_rope(x, cos, sin, pos)
+    # position 0 is the identity
+    assert torch.allclose(y[0], x[0])
+    # equals a complex multiplication of the pairs (x_i, x_{i+D/2}) by e^{i p theta_i}:
+    # an interleaved pairing (x_2i, x_2i+1) or a flipped sign fails this
+    z = torch.complex(x[..., :Dh // 2], x[..., Dh // 2:]) * torch.polar(torch.ones_like(ang), ang)[:, None, :]
+    assert torch.allclose(y[..., :Dh // 2], z.real) and torch.allclose(y[..., Dh // 2:], z.imag)
+    # each pair keeps its norm
+    assert torch.allclose(y[..., :Dh // 2] ** 2 + y[..., Dh // 2:] ** 2,
+                          x[..., :Dh // 2] ** 2 + x[..., Dh // 2:] ** 2)
+
+
+def test_rope_scores_depend_only_on_distance():
+    Dh = 32
+    cos, sin = P.rope_tables(Dh, 200, 1e6)
+    q, k = torch.randn(1, 1, Dh, dtype=D64), torch.randn(1, 1, Dh, dtype=D64)
+    def score(m, n):
+        return (P.apply_rope(q, cos, sin, torch.tensor([m])) * P.apply_rope(k, cos, sin, torch.tensor([n]))).sum()
+    assert torch.allclose(score(17, 5), score(117, 105), atol=1e-10)
+    assert not torch.allclose(score(17, 5), score(17, 6), atol=1e-6)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (6, 2), (4, 1), (1, 1)])
+def test_attention_is_library_causal_attention(Hq, Hkv):
+    T, Dh = 19, 16
+    q, k, v = torch.randn(T, Hq, Dh, dtype=D64), torch.randn(T, Hkv, Dh, dtype=D64), torch.randn(T, Hkv, Dh, dtype=D64)
+    got = P.causal_attention(q, k, v, Dh ** -0.5)
+    ref = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                         is_causal=True, scale=Dh ** -0.5, enable_gqa=True)[0].transpose(0, 1)
+    assert torch.allclose(got, ref, atol=1e-12)
+    # grouped heads == every kv head repeated for its consecutive query heads
+    rep = Hq // Hkv
+    full = P.causal_attention(q, k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1), Dh ** -0.5)
+    assert torch.allclose(got, full, atol=1e-12)
+
+
+def test_attention_special_cases():
+    Dh = 8
+    q, k, v = torch.randn(5, 2, Dh, dtype=D64), torch.randn(5, 1, Dh, dtype=D64), torch.randn(5, 1, Dh, dtype=D64)
+    out = P.causal_attention(q, k, v, 0.3)
+    # the first token sees only itself: output is its own value row
+    assert torch.allclose(out[0, 0], v[0, 0]) and torch.allclose(out[0, 1], v[0, 0])
+    # scale 0 -> uniform average of the visible values
+    out0 = P.causal_attention(q, k, v, 0.0)
+    assert torch.allclose(out0[3, 0], v[:4, 0].mean(0))
+    # window w keeps exactly the last w keys, the query's own included
+    outw = P.causal_attention(q, k, v, 0.0, window=2)
+    assert torch.allclose(outw[4, 0], v[3:5, 0].mean(0))
+    # a window as long as the sequence changes nothing
+    assert torch.allclose(P.causal_attention(q, k, v, 0.3, window=5), out)
+
+
+def test_far_key_dominates():
+    """One key scaled to stand out among hundreds must receive (almost) all the weight."""
+    T, Dh = 300, 16
+    q, k, v = torch.randn(T, 1, Dh, dtype=D64), torch.randn(T, 1, Dh, dtype=D64), torch.randn(T, 1, Dh, dtype=D64)
+    k[7, 0] = q[T - 1, 0] * 50
+    out = P.causal_attention(q, k, v, Dh ** -0.5)
+    assert torch.allclose(out[T - 1, 0], v[7, 0], atol=1e-6)
+
+
+def test_silu_and_mul_is_library_silu():
+    g, u = torch.randn(4, 9, dtype=D64), torch.randn(4, 9, dtype=D64)
+    assert torch.allclose(P.silu_and_mul(g, u), F.silu(g) * u, atol=1e-14)
+
+
+def _folder(tmp_path, name):
+    return helpers.make_folder(name, str(tmp_path / name), torch.float32)
+
+
+def test_model_reduces_to_hand_composition(tmp_path):
+    """One layer, written out by hand with library routines only."""
+    cfgd = dict(helpers.CONFIGS["B"], num_hidden_layers=1)
+    from mini_engine_amd.config.model_config import Qwen3Config
+    from mini_engine_amd.weights.random_init import write_random_model
+    d = write_random_model(Qwen3Config.from_dict(cfgd), 5, str(tmp_path / "one"), torch.float32)
+    cfg, w = P.read_model_folder(d, D64)
+    ids = helpers.random_ids(11, cfg["vocab_size"], 3)
+    got = P.logits(cfg, w, ids)
+    Hq, Hkv, Dh, eps = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rms_norm_eps"]
+    h = F.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    p = "model.layers.0."
+    x = F.rms_norm(h, (h.shape[-1],), w[p + "input_layernorm.weight"], eps)
+    q = F.linear(x, w[p + "self_attn.q_proj.weight"]).view(-1, Hq, Dh)
+    k = F.linear(x, w[p + "self_attn.k_proj.weight"]).view(-1, Hkv, Dh)
+    v = F.linear(x, w[p + "self_attn.v_proj.weight"]).view(-1, Hkv, Dh)
+    q = F.rms_norm(q, (Dh,), w[p + "self_attn.q_norm.weight"], eps)
+    k = F.rms_norm(k, (Dh,), w[p + "self_attn.k_norm.weight"], eps)
+    cos, sin = P.rope_tables(Dh, 11, cfg["rope_theta"])
+    q, k = P.apply_rope(q, cos, sin, torch.arange(11)), P.apply_rope(k, cos, sin, torch.arange(11))
+    o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                       is_causal=True, scale=Dh ** -0.5, enable_gqa=True)[0].transpose(0, 1)
+    res = h + F.linear(o.reshape(11, -1), w[p + "self_attn.o_proj.weight"])
+    x = F.rms_norm(res, (res.shape[-1],), w[p + "post_attention_layernorm.weight"], eps)
+    m = F.linear(F.silu(F.linear(x, w[p + "mlp.gate_proj.weight"])) * F.linear(x, w[p + "mlp.up_proj.weight"]),
+                 w[p + "mlp.down_proj.weight"])
+    x = F.rms_norm(m + res, (res.shape[-1],), w["model.norm.weight"], eps)
+    ref = F.linear(x, w["lm_head.weight"])
+    assert torch.allclose(got, ref, atol=1e-10)
+
+
+def test_model_is_causal_and_shift_invariant(tmp_path):
+    d = _folder(tmp_path, "A")
+    cfg, w = P.read_model_folder(d, D64)
+    ids = helpers.random_ids(30, cfg["vocab_size"], 1)
+    full = P.logits(cfg, w, ids)
+    # causality: a prefix gives the same logits
+    assert torch.allclose(P.logits(cfg, w, ids[:12]), full[:12], atol=1e-10)
+    # only distances count: shifting every position by the same amount changes nothing
+    shifted = P.logits(cfg, w, ids, positions=torch.arange(30) + 100)
+    assert torch.allclose(shifted, full, atol=1e-9)
+    # tied head: the head is the embedding matrix
+    assert "lm_head.weight" not in w
+
+
+def test_window_layers_limit_what_is_seen(tmp_path):
+    d = _folder(tmp_path, "C")
+    cfg, w = P.read_model_folder(d, D64)
+    assert P._windows(cfg) == [None, 24, None, 24]
+    cfg_w = dict(cfg, layer_types=["sliding_attention"] * 4)
+    ids = helpers.random_ids(60, cfg["vocab_size"], 2)
+    ids2 = list(ids)
+    ids2[0] = (ids2[0] + 1) % cfg["vocab_size"]
+    # with every layer windowed (24) over 4 layers, position 100 > 4*23 cannot see token 0 ...
+    a = P.logits(cfg_w, w, ids + ids)[-1]
+    b = P.logits(cfg_w, w, ids2 + ids)[-1]
+    assert torch.allclose(a, b, atol=1e-9)
+    # ... while the mixed model (full layers) does
+    assert not torch.allclose(P.logits(cfg, w, ids + ids)[-1], P.logits(cfg, w, ids2 + ids)[-1], atol=1e-9)
+
+
+def test_sampler_formula():
+    """argmax(softmax(z/T)/E) == argmax(z/T - log E); temperature 0 is argmax whatever the noise."""
+    z = torch.randn(50, dtype=D64)
+    e = torch.empty(50, dtype=D64).exponential_(1.0)
+    assert P.sample_gumbel_reference(z, 0.7, e) == int(torch.argmax(z / 0.7 - torch.log(e)))
+    assert P.sample_gumbel_reference(z, 0.0, e) == int(torch.argmax(z))
