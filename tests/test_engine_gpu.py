@@ -1,0 +1,130 @@
+"""The engine on the GPU with its HIP kernels, in float32 and in bfloat16, against the plain
+implementation, under every way of cutting the work; generation through the entry point."""
+import pytest
+import torch
+
+import engine_cases
+import helpers
+import plain_qwen3
+from mini_engine_amd.cache.manager import CacheManager
+from mini_engine_amd.engine.runner import ModelRunner
+from mini_engine_amd.weights.loader import load_model
+
+pytestmark = pytest.mark.gpu
+
+
+class Env:
+    device = "cuda"
+
+    def __init__(self, folders, dtype):
+        self.folders, self.dtype = folders, dtype
+        self.tol = helpers.TOL_F32 if dtype == torch.float32 else helpers.TOL_BF16
+        self.models = {}
+
+    def runner(self, name, pages):
+        folder = self.folders(name)
+        if name not in self.models:
+            self.models[name] = load_model(folder, self.device, self.dtype, 512)
+        model = self.models[name]
+        manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
+        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True), manager, folder
+
+
+@pytest.fixture(scope="module", params=[torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def env(request, folders):
+    return Env(folders, request.param)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("case", engine_cases.ALL, ids=lambda c: c.__name__)
+def test_cuts(env, case, name):
+    case(env, name)
+
+
+def test_hip_libraries_are_the_ones_running(env):
+    from mini_engine_amd.kernels import ops
+    env.runner("A", 2)
+    engine_cases.first_tokens(env, "A")
+    assert isinstance(ops.backend(), ops.HipBackend)
+    libs = ops.loaded_libraries()
+    assert any("libme_core.so" in p for p in libs)
+    if env.dtype == torch.bfloat16:
+        assert any("libme_attn_d16.so" in p for p in libs)
+
+
+def _llm(folder, dtype, **kw):
+    from mini_engine_amd import LLM
+    return LLM(folder, dtype=dtype, poison_cache=True, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generate_greedy_matches_plain(folders, dtype):
+    """Tiny A as BASELINE names it (prompts 5/17/33, 8 greedy tokens) and untied tiny B. In bfloat16
+    a token may differ only where the plain model's two best logits are closer than the tolerance."""
+    from mini_engine_amd import SamplingParams
+    for name, page in (("A", 16), ("B", 8)):
+        folder = folders(name)
+        cfg, w = plain_qwen3.read_model_folder(folder, torch.float64)
+        V = cfg["vocab_size"]
+        prompts = [helpers.random_ids(n, V, 900 + n) for n in (5, 17, 33)]
+        llm = _llm(folder, dtype, kvcache_block_size=page, num_kvcache_blocks=24, max_num_seqs=4,
+                   max_num_batched_tokens=64, max_model_len=64)
+        outs = llm.generate(prompts, SamplingParams(temperature=0, max_tokens=8), use_tqdm=False)
+        for p, o in zip(prompts, outs):
+            ids = list(p)
+            for tok in o["token_ids"]:
+                z = plain_qwen3.logits(cfg, w, ids)[-1]
+                best = int(torch.argmax(z))
+                if tok != best:
+                    assert dtype == "bfloat16" and float(z[best] - z[tok]) <= helpers.TOL_BF16 * float(z.abs().max()), \
+                        f"{name}: token {tok} instead of {best}"
+                ids.append(tok)
+        llm.manager.check_invariants()
+        assert llm.manager.num_free_pages() == 24
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(folders, dtype):
+    """Tiny B as BASELINE names it: prompts 1/9/24/40/63, budget 16, temperature 0.8, 12 tokens each.
+    In float32 the same seed gives the same tokens together, alone, and under preemption."""
+    from mini_engine_amd import SamplingParams
+    folder = folders("B")
+    prompts = [helpers.random_ids(n, 384, 950 + n) for n in (1, 9, 24, 40, 63)]
+    sp = SamplingParams(temperature=0.8, max_tokens=12, ignore_eos=True)
+    common = dict(kvcache_block_size=8, max_num_seqs=16, max_model_len=128, seed=3)
+    together = _llm(folder, dtype, num_kvcache_blocks=64, max_num_batched_tokens=16, **common)
+    out_together = [o["token_ids"] for o in together.generate(prompts, sp, use_tqdm=False)]
+    assert all(len(o) == 12 for o in out_together)
+    again = _llm(folder, dtype, num_kvcache_blocks=64, max_num_batched_tokens=16, **common)
+    assert [o["token_ids"] for o in again.generate(prompts, sp, use_tqdm=False)] == out_together
+    if dtype == "float32":
+        tight = _llm(folder, dtype, num_kvcache_blocks=21, max_num_batched_tokens=16, enable_prefix_caching=False, **common)
+        out_tight = [o["token_ids"] for o in tight.generate(prompts, sp, use_tqdm=False)]
+        assert tight.scheduler.num_preemptions > 0
+        assert out_tight == out_together
+        wide = _llm(folder, dtype, num_kvcache_blocks=64, max_num_batched_tokens=128, **common)
+        assert [o["token_ids"] for o in wide.generate(prompts, sp, use_tqdm=False)] == out_together
+
+
+def test_float32_logits_do_not_depend_on_the_cut_bitwise(folders):
+    """The float32 kernels fix the order of every sum per token, so cuts agree to the last bit."""
+    env = Env(folders, torch.float32)
+    ids = helpers.random_ids(90, 384, 5)
+    runner, manager, folder = env.runner("B", 12)
+    d = helpers.Driver(runner, manager); d.step({"r": ids})
+    whole = d.result("r")
+    runner, manager, folder = env.runner("B", 14)
+    d = helpers.Driver(runner, manager)
+    other = helpers.random_ids(9, 384, 6)
+    d.step({"r": ids[:31], "x": other[:2]}); d.step({"x": other[2:3], "r": ids[31:33]})
+    for t in range(33, 90):
+        d.step({"r": ids[t:t + 1]})
+    assert torch.equal(d.result("r"), whole)
+
+
+def test_pool_sizing_from_free_memory(folders):
+    from mini_engine_amd import LLM, SamplingParams
+    llm = LLM(folders("A"), max_num_seqs=4, max_num_batched_tokens=64, max_model_len=128, gpu_memory_utilization=0.5)
+    assert llm.config.num_kvcache_blocks == 4 * 8          # capped by what max_num_seqs requests can hold
+    out = llm.generate([[1, 2, 3]], SamplingParams(temperature=0, max_tokens=3), use_tqdm=False)
+    assert len(out[0]["token_ids"]) == 3

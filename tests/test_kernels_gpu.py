@@ -1,0 +1,309 @@
+"""Each HIP kernel alone against its plain twin, at sizes other than the engine tests use.
+Inputs are built so that faults show: NaN in every cache slot nobody owns, a far key made to
+dominate among hundreds, window edges, page edges, sizes that are no power of two."""
+import math
+
+import pytest
+import torch
+
+import kernel_twins as twin
+from mini_engine_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def hip():
+    return ops.HipBackend()
+
+
+def close(a, b, tol):
+    a, b = a.double().cpu(), b.double().cpu()
+    assert torch.isfinite(a).all()
+    err = float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+    assert err <= tol, f"relative error {err:.3g} > {tol:g}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(7, 100), (300, 1024), (5, 3)])
+def test_gather_rows(dtype, rows, width):
+    src = torch.randn(rows, width, device=DEV).to(dtype)
+    idx = torch.randint(0, rows, (41,), device=DEV, dtype=torch.int32)
+    assert torch.equal(hip().gather_rows(src, idx), twin.gather_rows(src, idx))
+
+
+@pytest.mark.parametrize("T,n", [(1, 80), (13, 1000), (64, 4096), (3, 5120)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rms_norm(dtype, T, n):
+    torch.manual_seed(T * n)
+    x = (torch.randn(T, n, device=DEV) * 3).to(dtype)
+    res = torch.randn(T, n, device=DEV)
+    w = torch.rand(n, device=DEV) + 0.5
+    tol = 1e-6 if dtype == torch.float32 else 4e-3
+    y, r = hip().rms_norm(x, w, 1e-5, res, dtype)
+    yt, rt = twin.rms_norm(x, w, 1e-5, res, dtype)
+    close(y, yt, tol); close(r, rt, 1e-6)
+    y, r = hip().rms_norm(x, w, 1e-5, None, dtype)            # start of the residual stream
+    yt, rt = twin.rms_norm(x, w, 1e-5, None, dtype)
+    close(y, yt, tol); assert torch.equal(r, x.float())
+    y, r = hip().rms_norm(x, w, 1e-5, res, dtype, want_residual=False)
+    assert r is None
+    parts = torch.randn(3, T, n, device=DEV)                  # stacked float32 partial sums
+    y, r = hip().rms_norm(parts, w, 1e-6, res, dtype)
+    yt, rt = twin.rms_norm(parts, w, 1e-6, res, dtype)
+    close(y, yt, tol); close(r, rt, 1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_and_mul(dtype):
+    gu = (torch.randn(37, 2 * 224, device=DEV) * 4).to(dtype)
+    close(hip().silu_and_mul(gu), twin.silu_and_mul(gu), 1e-6 if dtype == torch.float32 else 4e-3)
+    big = torch.tensor([[-100.0, 100.0, 0.0, 1.0, 2.0, 3.0]], device=DEV).to(dtype)   # no overflow at the ends
+    assert torch.isfinite(hip().silu_and_mul(big)).all()
+
+
+def _caches(pages, Hkv, page, D, dtype):
+    k = torch.full((pages, Hkv, page, D), float("nan"), device=DEV, dtype=dtype)
+    v = torch.full((pages, Hkv, D, page), float("nan"), device=DEV, dtype=dtype)
+    return k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 16, 16), (6, 2, 32, 8), (5, 5, 48, 4), (16, 8, 128, 16), (2, 1, 256, 32)])
+def test_qk_norm_rope_store(dtype, Hq, Hkv, D, page):
+    torch.manual_seed(D)
+    T, P = 29, 64
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * D, device=DEV).to(dtype)
+    qw, kw = torch.rand(D, device=DEV) + 0.5, torch.rand(D, device=DEV) + 0.5
+    ang = torch.outer(torch.arange(P, dtype=torch.float32), 1.0 / (1e4 ** (torch.arange(0, D, 2).float() / D)))
+    table = torch.stack((ang.cos(), ang.sin()), -1).contiguous().to(DEV)
+    pos = torch.randint(0, P, (T,), device=DEV, dtype=torch.int32)
+    slots = torch.randperm(8 * page, device=DEV)[:T].to(torch.int32)
+    slots[3] = -1                                              # a skipped token
+    tol = 2e-6 if dtype == torch.float32 else 4e-3
+    for use_norm, use_rope in ((True, True), (False, True), (True, False)):
+        a, b = qkv.clone(), qkv.clone()
+        ka, va = _caches(8, Hkv, page, D, dtype); kb, vb = _caches(8, Hkv, page, D, dtype)
+        args = (qw if use_norm else None, kw if use_norm else None, 1e-5, table if use_rope else None, pos, slots)
+        hip().qk_norm_rope_store(a, *args, ka, va, Hq, Hkv, D, page, True)
+        twin.qk_norm_rope_store(b, *args, kb, vb, Hq, Hkv, D, page, True)
+        close(a[:, :Hq * D], b[:, :Hq * D], tol)
+        assert torch.equal(torch.isnan(ka), torch.isnan(kb)) and torch.equal(torch.isnan(va), torch.isnan(vb))
+        close(torch.nan_to_num(ka), torch.nan_to_num(kb), tol)
+        assert torch.equal(torch.nan_to_num(va), torch.nan_to_num(vb))          # values are copied bit-exactly
+        assert torch.equal(a[:, Hq * D:], qkv[:, Hq * D:])                       # k, v rows themselves untouched
+    # in-place form: q and k rewritten, nothing cached; and q-only rows
+    a, b = qkv[:, :(Hq + Hkv) * D].clone(), qkv[:, :(Hq + Hkv) * D].clone()
+    hip().qk_norm_rope_store(a, qw, kw, 1e-5, table, pos, None, None, None, Hq, Hkv, D, page, False)
+    twin.qk_norm_rope_store(b, qw, kw, 1e-5, table, pos, None, None, None, Hq, Hkv, D, page, False)
+    close(a, b, tol)
+    a, b = qkv[:, :Hq * D].clone(), qkv[:, :Hq * D].clone()
+    hip().qk_norm_rope_store(a, qw, qw, 1e-5, table, pos, None, None, None, Hq, 0, D, page, False)
+    twin.qk_norm_rope_store(b, qw, qw, 1e-5, table, pos, None, None, None, Hq, 0, D, page, False)
+    close(a, b, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_store_kv_is_bit_exact_and_skips_negative_slots(dtype):
+    T, Hkv, D, page = 50, 3, 40, 8
+    packed = torch.randn(T, (2 + 2 * Hkv) * D, device=DEV).to(dtype)
+    k = packed[:, 2 * D:(2 + Hkv) * D].view(T, Hkv, D)        # strided views of a packed row
+    v = packed[:, (2 + Hkv) * D:].view(T, Hkv, D)
+    slots = torch.randperm(9 * page, device=DEV)[:T].to(torch.int32)
+    slots[[0, 17]] = -1
+    ka, va = _caches(9, Hkv, page, D, dtype); kb, vb = _caches(9, Hkv, page, D, dtype)
+    hip().store_kv(k, v, slots, ka, va, page)
+    twin.store_kv(k, v, slots, kb, vb, page)
+    for x, y in ((ka, kb), (va, vb)):
+        assert torch.equal(torch.isnan(x), torch.isnan(y)) and torch.equal(torch.nan_to_num(x), torch.nan_to_num(y))
+    assert int((~torch.isnan(ka)).sum()) == (T - 2) * Hkv * D
+
+
+# ------------------------------------------------------------------------------- attention
+
+def _attention_case(dtype, Hq, Hkv, D, page, seqs, window=None, seed=0, peak=None):
+    """seqs: list of (context length after the step, new tokens). Builds a paged cache with
+    shuffled pages and NaN everywhere else, runs kernel and twin."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    order = sorted(range(len(seqs)), key=lambda i: seqs[i][1] != 1)          # decodes first
+    seqs = [seqs[i] for i in order]
+    B = len(seqs)
+    need = [-(-L // page) for L, _ in seqs]
+    total_pages = sum(need) + 3
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    k_cache, v_cache = _caches(total_pages, Hkv, page, D, dtype)
+    MB = max(need)
+    bt = torch.full((B, MB + 1), -1, dtype=torch.int32)
+    q_rows, seq_of, positions, ctx, cu = [], [], [], [], [0]
+    for b, (L, n) in enumerate(seqs):
+        pages = [perm.pop() for _ in range(need[b])]
+        bt[b, :need[b]] = torch.tensor(pages, dtype=torch.int32)
+        K = torch.randn(L, Hkv, D, generator=g)
+        V = torch.randn(L, Hkv, D, generator=g)
+        Q = torch.randn(n, Hq, D, generator=g) * 2
+        if peak is not None:                                     # one far key dominates the last query
+            far = peak if peak < L else 0
+            K[far] = Q[-1, ::Hq // Hkv][:Hkv] * 6
+        lo = 0
+        if window:                                               # pages wholly behind the window are not held
+            lo = max(0, (L - n) - window + 1)
+            for pi in range(lo // page):
+                bt[b, pi] = -1
+        for t in range(lo // page * page, L):
+            pg, off = pages[t // page], t % page
+            k_cache[pg, :, off, :] = K[t].to(dtype)
+            v_cache[pg, :, :, off] = V[t].to(dtype)
+        q_rows.append(Q.reshape(n, Hq * D))
+        seq_of += [b] * n
+        positions += list(range(L - n, L))
+        ctx.append(L); cu.append(cu[-1] + n)
+    Dn = sum(1 for _, n in seqs if n == 1)
+    T = cu[-1]
+    # q as a strided view of a wider row, as in the engine
+    wide = torch.zeros(T, Hq * D + 2 * Hkv * D, device=DEV, dtype=dtype)
+    wide[:, :Hq * D] = torch.cat(q_rows).to(DEV).to(dtype)
+    q = wide[:, :Hq * D]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    args = (q, k_cache, v_cache, page, bt.to(DEV), i32(ctx), i32(seq_of), i32(positions),
+            i32([c - cu[Dn] for c in cu[Dn:]]) if Dn < B else None, Dn,
+            max([L for L, n in seqs if n == 1], default=0), D ** -0.5, window, Hq, Hkv, D)
+    return args
+
+
+SHAPES = [(4, 2, 16, 16), (6, 2, 32, 8), (4, 1, 48, 16), (16, 8, 128, 16), (8, 8, 64, 32), (32, 1, 64, 16), (2, 2, 128, 64)]
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_prefill_ragged(dtype, Hq, Hkv, D, page):
+    """Ragged prompts, chunks that attend to earlier chunks, lengths at tile and page edges."""
+    seqs = [(5, 5), (33, 33), (64, 2), (65, 33), (129, 17), (page, page), (page + 1, 2), (200, 64), (31, 31)]
+    args = _attention_case(dtype, Hq, Hkv, D, page, seqs, seed=D + page)
+    close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_decode_batches(dtype, Hq, Hkv, D, page):
+    """Decode alone (small, long, mixed lengths: one partition and many) and beside prefill rows."""
+    for seqs in ([(1, 1)], [(7, 1), (130, 1), (2, 1)], [(1500, 1)], [(700, 1), (33, 1), (900, 1), (128, 1), (129, 1)],
+                 [(40, 1), (300, 1), (50, 50), (90, 7), (2, 2)]):
+        args = _attention_case(dtype, Hq, Hkv, D, page, seqs, seed=len(seqs))
+        close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_far_key_stands_out(dtype):
+    """One key among hundreds gets all the weight: a kernel that drops or misplaces a block,
+    a partition or a page shows an O(1) error here that random scores would average away."""
+    for peak in (0, 15, 16, 255, 256, 700, 1023):
+        args = _attention_case(dtype, 4, 2, 64, 16, [(1024, 1), (1024, 40)], seed=peak, peak=peak)
+        close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 7, 16, 24, 100])
+def test_attention_window_edges(dtype, window):
+    """Keys just inside and just outside the window; pages behind it are not held (-1 in the
+    table, NaN in memory)."""
+    seqs = [(150, 1), (33, 1), (window, 1), (window + 1, 1), (150, 40), (70, 70), (window + 5, 3)]
+    for peak in (None, 150 - window, 150 - window - 1):
+        args = _attention_case(dtype, 6, 2, 32, 8, seqs, window=window, seed=window, peak=peak)
+        close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
+
+
+def test_attention_generic_path_takes_odd_sizes():
+    """Head size 24 and page 5 are outside the matrix-core kernel: the generic kernel takes them."""
+    for dtype in (torch.float32, torch.bfloat16):
+        args = _attention_case(dtype, 3, 1, 24, 5, [(40, 1), (23, 23), (9, 2)], seed=1)
+        close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
+    args = _attention_case(torch.bfloat16, 4, 2, 64, 16, [(300, 1), (70, 70)], seed=2)
+    close(hip().paged_attention(*args, force_simple=True), hip().paged_attention(*args), 1.5e-2)
+
+
+def test_decode_partitions_rule():
+    for S, Hq, Hkv, ctx in ((1, 16, 8, 2048), (8, 16, 8, 2048), (64, 16, 8, 2304), (1, 32, 8, 100), (3, 6, 2, 130000)):
+        part, parts = ops.decode_partitions(S, Hq, Hkv, ctx)
+        assert part % 128 == 0 and part * parts >= ctx and part * (parts - 1) < ctx
+
+
+# ------------------------------------------------------------------------------- products
+
+@pytest.mark.parametrize("M,N,K", [(1, 100, 72), (5, 384, 80), (64, 1000, 224), (130, 96, 200), (300, 300, 31)])
+def test_linear_float32_is_exact_product(M, N, K):
+    x, w = torch.randn(M, K, device=DEV), torch.randn(N, K, device=DEV)
+    close(hip().linear(x, w), x.double() @ w.double().t(), 2e-6)
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(384, 80), (1000, 224), (3072, 1024), (1024, 3072), (100, 2048)])
+def test_linear_skinny_bf16(M, N, K):
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    ref = x.double() @ w.double().t()
+    close(hip().linear(x, w), ref, 6e-3)                       # bf16 output rounding
+    close(hip().linear(x, w, torch.float32), ref, 2e-5)        # float32 output: accumulation error only
+    parts = hip().linear(x, w, None, allow_partials=True)      # may be split over K
+    close(parts.sum(0) if parts.dim() == 3 else parts, ref, 6e-3 if parts.dim() == 2 else 2e-5)
+
+
+def test_linear_partials_are_used_where_tiles_are_few():
+    x = torch.randn(8, 3072, device=DEV).bfloat16()
+    w = torch.randn(1024, 3072, device=DEV).bfloat16()
+    assert hip().linear(x, w, None, allow_partials=True).dim() == 3
+    assert hip().linear(x, torch.randn(9000, 3072, device=DEV).bfloat16(), None, allow_partials=True).dim() == 2
+
+
+@pytest.mark.parametrize("M,N,K", [(200, 384, 80), (2048, 1024, 1024), (65, 100, 200), (70, 96, 44)])
+def test_linear_large_and_odd_bf16(M, N, K):
+    """Above the skinny range the library product runs; K not a multiple of 8 takes the FMA kernel."""
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    ref = x.double() @ w.double().t()
+    close(hip().linear(x, w), ref, 6e-3)
+    close(hip().linear(x, w, torch.float32), ref, 2e-5)
+    xs = torch.randn(M, K + 8, device=DEV).bfloat16()[:, :K]   # a row stride that is not K
+    close(hip().linear(xs, w), xs.double() @ w.double().t(), 6e-3)
+
+
+# ------------------------------------------------------------------------------- sampling
+
+def test_sample_greedy_and_noise():
+    S, V = 9, 1531
+    logits = torch.randn(S, V, device=DEV) * 3
+    keys = torch.randint(-2 ** 31, 2 ** 31 - 1, (S, 2), device=DEV, dtype=torch.int32)
+    zero = torch.zeros(S, device=DEV)
+    assert hip().sample(logits, zero, keys).tolist() == logits.argmax(-1).tolist()
+    tie = torch.zeros(2, 50, device=DEV); tie[:, [7, 30]] = 5.0
+    assert hip().sample(tie, zero[:2], keys[:2]).tolist() == [7, 7]           # first of equal maxima
+    temps = torch.tensor([0.0, 0.5, 1.0, 2.0, 0.8, 0.0, 1.5, 0.1, 1.0], device=DEV)
+    got = hip().sample(logits, temps, keys)
+    scores = twin.sample_scores(logits, temps, keys)
+    picked = scores.gather(1, got.long()[:, None])[:, 0]
+    assert torch.all(picked >= scores.max(-1).values - 1e-4)                  # the twin's argmax up to float noise
+    assert hip().sample(logits, temps, keys).tolist() == got.tolist()         # same keys, same tokens
+    other = hip().sample(logits, temps, keys.flip(1))
+    assert other[temps > 0.4].tolist() != got[temps > 0.4].tolist()
+
+
+def test_sample_frequencies_follow_softmax():
+    """Over many keys the exponential race picks token i with probability softmax(z/T)_i."""
+    V, n, T = 12, 20000, 0.7
+    z = torch.randn(V, device=DEV)
+    keys = torch.stack((torch.arange(n, device=DEV, dtype=torch.int32), torch.full((n,), 12345, device=DEV, dtype=torch.int32)), 1)
+    got = hip().sample(z.expand(n, V).contiguous(), torch.full((n,), T, device=DEV), keys)
+    freq = torch.bincount(got.long(), minlength=V).double().cpu() / n
+    p = torch.softmax(z.double().cpu() / T, 0)
+    chi2 = float((n * (freq - p) ** 2 / p).sum())
+    assert chi2 < 40.0, f"chi-square {chi2:.1f} with 11 degrees of freedom"   # p < 1e-4 under the null
+
+
+def test_kernels_refuse_what_they_cannot_do():
+    with pytest.raises(ops.KernelError, match="dtype"):
+        hip().silu_and_mul(torch.zeros(2, 4, device=DEV, dtype=torch.float16))
+    with pytest.raises(ops.KernelError):
+        hip().linear(torch.zeros(2, 8, device=DEV), torch.zeros(4, 8, device=DEV).bfloat16())
+    with pytest.raises(ops.KernelError, match="head_dim"):
+        hip().qk_norm_rope_store(torch.zeros(1, 3 * 600, device=DEV), None, None, 0.0, None,
+                                 torch.zeros(1, device=DEV, dtype=torch.int32), torch.zeros(1, device=DEV, dtype=torch.int32),
+                                 torch.zeros(1, 1, 4, 600, device=DEV), torch.zeros(1, 1, 600, 4, device=DEV), 1, 1, 600, 4, True)
