@@ -1,0 +1,207 @@
+"""Decode and prefill throughput of the engine on one MI355X, with the fraction of the roofline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model-size 0.6b] [--batch 8] [--context 2048]
+
+The default run has the layer sizes of Qwen3-0.6B (28 layers, hidden 1024, 16 query / 8 key heads
+of 128, intermediate 3072, vocabulary 151936, tied head) with seeded random weights, bfloat16, a
+batch of 8 requests each holding a 2,048-token context. A "step" is one decode step of the whole
+batch: the engine's own step function, cache manager and sampler (greedy), from token ids to the
+next token ids on the host. One JSON line is printed:
+  value        decoded tokens per second at the default batch
+  prefill      one 2,048-token prompt in one step: tokens/s, ms, fraction of the bf16 MFMA peak
+  roofline     bytes the decode step must read (every weight once + the live requests' cache) / time
+  points       decode tokens/s at batch 1 and 64
+Peaks: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s (MI355X, published).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+SIZES = {
+    # name: (layers, hidden, q heads, kv heads, head_dim, intermediate, vocab, tied)
+    "tinyA": (2, 64, 4, 2, 16, 128, 256, True),
+    "0.6b": (28, 1024, 16, 8, 128, 3072, 151936, True),
+    "8b": (36, 4096, 32, 8, 128, 12288, 151936, False),
+    "32b": (64, 5120, 64, 8, 128, 25600, 151936, False),
+}
+
+
+def model_config(size: str, layers: int | None):
+    from mini_engine_amd.config.model_config import Qwen3Config
+    L, h, Hq, Hkv, D, I, V, tied = SIZES[size]
+    return Qwen3Config.from_dict(dict(
+        architectures=["Qwen3ForCausalLM"], vocab_size=V, hidden_size=h, intermediate_size=I,
+        num_hidden_layers=layers or L, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D,
+        rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=tied, max_position_embeddings=40960)), L
+
+
+def linear_params_per_layer(cfg) -> int:
+    qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim * cfg.hidden_size
+    o = cfg.num_attention_heads * cfg.head_dim * cfg.hidden_size
+    return qkv + o + 3 * cfg.intermediate_size * cfg.hidden_size
+
+
+def decode_bytes(cfg, item: int, contexts: list) -> int:
+    """Bytes one decode step has to read: every weight it uses once, and the cache of the live requests."""
+    weights = cfg.num_hidden_layers * linear_params_per_layer(cfg) + cfg.vocab_size * cfg.hidden_size   # head (tied or not)
+    norms = cfg.num_hidden_layers * (2 * cfg.hidden_size + 2 * cfg.head_dim) + cfg.hidden_size
+    kv = sum(contexts) * 2 * cfg.num_key_value_heads * cfg.head_dim * cfg.num_hidden_layers
+    return weights * item + norms * 4 + kv * item
+
+
+def prefill_flops(cfg, T: int) -> float:
+    lin = 2.0 * T * cfg.num_hidden_layers * linear_params_per_layer(cfg)
+    attn = 4.0 * cfg.num_attention_heads * cfg.head_dim * T * (T + 1) / 2 * cfg.num_hidden_layers
+    head = 2.0 * cfg.vocab_size * cfg.hidden_size
+    return lin + attn + head
+
+
+class Bench:
+    def __init__(self, cfg, dtype: str, page: int, max_batch: int, context: int, gen: int, seed: int = 0):
+        import torch
+        from mini_engine_amd.cache.manager import CacheManager
+        from mini_engine_amd.engine.runner import ModelRunner
+        from mini_engine_amd.registry import build_model
+        from mini_engine_amd.weights.random_init import fill_random
+
+        self.torch = torch
+        self.cfg, self.page, self.context, self.gen = cfg, page, context, gen
+        self.dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
+        self.max_len = context + gen + 64
+        t0 = time.time()
+        self.model = fill_random(build_model(cfg), seed, "cuda", self.dtype, self.max_len)
+        print(f"[bench] random weights ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+        pages = max_batch * -(-self.max_len // page)
+        self.manager = CacheManager(pages, page, ModelRunner.windows_of(self.model), enable_prefix_caching=False)
+        self.runner = ModelRunner(self.model, self.manager, self.dtype, "cuda", self.max_len)
+        self.gen_ids = torch.Generator().manual_seed(seed)
+
+    def _ids(self, n):
+        return self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen_ids).tolist()
+
+    def prefill(self, rid, n, want_last=True):
+        from mini_engine_amd.engine.runner import StepEntry
+        assert self.manager.allocate(rid, 0, n)
+        return self.runner.step([StepEntry(rid, self._ids(n), 0, [n - 1] if want_last else [])])
+
+    def time_prefill(self, T: int, reps: int = 3):
+        torch = self.torch
+        best = None
+        for i in range(reps + 1):                          # the first run warms up
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            self.prefill(("p", i), T)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            self.manager.free(("p", i))
+            if i and (best is None or dt < best):
+                best = dt
+        return best
+
+    def time_decode(self, batch: int, steps: int, warmup: int):
+        """`batch` requests with `context` tokens each in the cache, then warmup + steps decode steps."""
+        from mini_engine_amd.engine.runner import StepEntry
+        torch = self.torch
+        reqs = [("d", batch, i) for i in range(batch)]
+        last = []
+        for r in reqs:                                     # real prefill, one request per step
+            logits = self.prefill(r, self.context)
+            last.append(int(self.runner.sample(logits, [0.0], [(0, 0)])[0]))
+        pos = self.context
+        temps, keys = [0.0] * batch, [(0, 0)] * batch
+
+        def one():
+            nonlocal last, pos
+            entries = []
+            for r, tok in zip(reqs, last):
+                assert self.manager.allocate(r, pos, 1)
+                entries.append(StepEntry(r, [tok], pos, [0]))
+            logits = self.runner.step(entries)
+            last = self.runner.sample(logits, temps, keys)  # token ids on the host: the step is complete
+            pos += 1
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ctx_mid = pos - steps / 2.0                        # mean context length over the timed steps
+        for r in reqs:
+            self.manager.free(r)
+        return dt / steps, ctx_mid
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--model-size", default="0.6b", choices=sorted(SIZES))
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the size has (both numbers are reported)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--gen", type=int, default=256)
+    ap.add_argument("--page", type=int, default=16)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--points", default="1,64", help="extra decode batch sizes, comma separated ('' for none)")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
+        return 2
+    if args.steps + args.warmup > args.gen:
+        args.gen = args.steps + args.warmup
+
+    import torch
+    cfg, full_layers = model_config(args.model_size, args.layers)
+    points = [int(p) for p in args.points.split(",") if p]
+    bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed)
+    item = 2 if args.dtype == "bfloat16" else 4
+
+    T = args.prefill_tokens
+    pre = bench.time_prefill(T)
+    prefill = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
+               "frac": round(prefill_flops(cfg, T) / pre / FLOP_PEAK[args.dtype], 4)}
+    print(f"[bench] prefill {T} tokens: {pre * 1e3:.2f} ms", file=sys.stderr, flush=True)
+
+    step_s, ctx_mid = bench.time_decode(args.batch, args.steps, args.warmup)
+    need = decode_bytes(cfg, item, [ctx_mid] * args.batch)
+    roofline = {"bound": "hbm", "achieved": round(need / step_s / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": round(need / step_s / HBM_PEAK, 4)}
+    print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    pts = {}
+    for b in points:
+        s, _ = bench.time_decode(b, min(args.steps, 64), min(args.warmup, 8))
+        pts[f"decode_b{b}"] = round(b / s, 1)
+        print(f"[bench] decode batch {b}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+
+    line = {
+        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens; % roofline",
+        "value": round(args.batch / step_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded random token ids, seeded random weights",
+        "config": {"model": f"Qwen3-{args.model_size} sizes", "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+                   "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "tied": bool(cfg.tie_word_embeddings), "page": args.page, "global_batch": args.batch,
+                   "seq_len": args.context, "gen": args.gen, "parallelism": "single GPU",
+                   "gpu": torch.cuda.get_device_name(0)},
+        "prefill": prefill, "roofline": roofline, "points": pts,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
