@@ -63,7 +63,8 @@ def prefill_flops(cfg, T: int) -> float:
 
 
 class Bench:
-    def __init__(self, cfg, dtype: str, page: int, max_batch: int, context: int, gen: int, seed: int = 0):
+    def __init__(self, cfg, dtype: str, page: int, max_batch: int, context: int, gen: int, seed: int = 0,
+                 graphs: bool = True):
         import torch
         from mini_engine_amd.cache.manager import CacheManager
         from mini_engine_amd.engine.runner import ModelRunner
@@ -79,7 +80,7 @@ class Bench:
         print(f"[bench] random weights ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
         pages = max_batch * -(-self.max_len // page)
         self.manager = CacheManager(pages, page, ModelRunner.windows_of(self.model), enable_prefix_caching=False)
-        self.runner = ModelRunner(self.model, self.manager, self.dtype, "cuda", self.max_len)
+        self.runner = ModelRunner(self.model, self.manager, self.dtype, "cuda", self.max_len, use_graphs=graphs)
         self.gen_ids = torch.Generator().manual_seed(seed)
 
     def _ids(self, n):
@@ -155,6 +156,7 @@ def main(argv=None) -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="extra decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -165,7 +167,7 @@ def main(argv=None) -> int:
     import torch
     cfg, full_layers = model_config(args.model_size, args.layers)
     points = [int(p) for p in args.points.split(",") if p]
-    bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed)
+    bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed, graphs=not args.no_graphs)
     item = 2 if args.dtype == "bfloat16" else 4
 
     T = args.prefill_tokens
@@ -196,7 +198,7 @@ def main(argv=None) -> int:
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "tied": bool(cfg.tie_word_embeddings), "page": args.page, "global_batch": args.batch,
                    "seq_len": args.context, "gen": args.gen, "parallelism": "single GPU",
-                   "gpu": torch.cuda.get_device_name(0)},
+                   "hip_graphs": not args.no_graphs},
         "prefill": prefill, "roofline": roofline, "points": pts,
     }
     print(json.dumps(line), flush=True)

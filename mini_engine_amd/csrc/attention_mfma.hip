@@ -82,11 +82,12 @@ __device__ __forceinline__ void attend32(const AttnArgs& a, const int32_t* __res
                                          f32x4 (&acc)[DT], int n, int g) {
   // ---- scores: two 16-key tiles, rows permuted as described above
   const int kgrp = t0 + 8 * (n >> 2);
-  const bool kgrp_ok = kgrp < L && kgrp + 7 >= lo_min;
+  bool kgrp_ok = kgrp < L && kgrp + 7 >= lo_min;
   int kpi = 0, kpage = 0;
   if (kgrp_ok) {
     kpi = page_index(kgrp, a.page, a.page_shift);
     kpage = bt[kpi];
+    kgrp_ok = kpage >= 0;  // a page that is not held is never dereferenced
   }
   const int koff = kgrp - kpi * a.page + (n & 3);
   f32x4 st[2];
@@ -106,11 +107,12 @@ __device__ __forceinline__ void attend32(const AttnArgs& a, const int32_t* __res
 
   // ---- V^T operands (issued before the softmax arithmetic so the loads overlap it)
   const int vgrp = t0 + 8 * g;
-  const bool vgrp_ok = vgrp < L && vgrp + 7 >= lo_min;
+  bool vgrp_ok = vgrp < L && vgrp + 7 >= lo_min;
   int vpi = 0, vpage = 0;
   if (vgrp_ok) {
     vpi = page_index(vgrp, a.page, a.page_shift);
     vpage = bt[vpi];
+    vgrp_ok = vpage >= 0;
   }
   const bf16_t* vp = a.v_cache + (((int64_t)vpage * a.Hkv + kvh) * HD + n) * a.page + (vgrp - vpi * a.page);
   bf16x8 va[DT];

@@ -20,7 +20,8 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
                    const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                    const int32_t* __restrict__ block_tables, int bt_stride,
                    const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
-                   int Hq, int Hkv, int D, int page, float scale, int window) {
+                   const int32_t* __restrict__ context_lens, int Hq, int Hkv, int D, int page, float scale,
+                   int window) {
   extern __shared__ float lds[];
   float* qs = lds;                 // D
   float* sc = lds + D;             // AS_THREADS scores / probabilities
@@ -38,7 +39,9 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
   for (int d = tid; d < D; d += AS_THREADS) qs[d] = to_f32<T>(q[t * q_stride + (int64_t)h * D + d]);
   __syncthreads();
 
-  const int hi = pos + 1;                                   // keys [lo, hi)
+  // keys [lo, hi): up to the query's own position, never past the request's context (a padding
+  // row has context 0 and sees nothing)
+  const int hi = min(pos + 1, context_lens[b]);
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   float m = -INFINITY, l = 0.f;
   // thread d < D owns output channel d (two channels per thread when D > AS_THREADS)
@@ -47,13 +50,17 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
   for (int c0 = (lo / AS_THREADS) * AS_THREADS; c0 < hi; c0 += AS_THREADS) {
     const int j = c0 + tid;
     float s = -INFINITY;
-    if (j >= lo && j < hi) {
+    bool keep = j >= lo && j < hi;
+    if (keep) {
       const int64_t pg = bt[j / page];
-      const int off = j % page;
-      const T* kr = k_cache + ((pg * Hkv + kvh) * (int64_t)page + off) * D;
-      float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot += qs[d] * to_f32<T>(kr[d]);
-      s = dot * scale;
+      keep = pg >= 0;                        // a page that is not held is never dereferenced
+      if (keep) {
+        const int off = j % page;
+        const T* kr = k_cache + ((pg * Hkv + kvh) * (int64_t)page + off) * D;
+        float dot = 0.f;
+        for (int d = 0; d < D; ++d) dot += qs[d] * to_f32<T>(kr[d]);
+        s = dot * scale;
+      }
     }
     // chunk max
     float cm = wave_max(s);
@@ -62,8 +69,8 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
     __syncthreads();
     cm = red[0];
     for (int w = 1; w < AS_THREADS / 64; ++w) cm = fmaxf(cm, red[w]);
-    const float m_new = fmaxf(m, cm);            // finite: every chunk holds at least one kept key
-    const float p = (j >= lo && j < hi) ? expf(s - m_new) : 0.f;
+    const float m_new = fmaxf(m, cm);
+    const float p = (keep && m_new > -INFINITY) ? expf(s - m_new) : 0.f;
     sc[tid] = p;
     float ps = wave_sum(p);
     __syncthreads();
@@ -71,7 +78,7 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
     __syncthreads();
     ps = 0.f;
     for (int w = 0; w < AS_THREADS / 64; ++w) ps += red[8 + w];
-    const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+    const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);   // m finite implies m_new finite
     l = l * alpha + ps;
     m = m_new;
     acc0 *= alpha;
@@ -83,6 +90,7 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
         float a = 0.f;
         for (int jj = jb; jj < je; ++jj) {
           const int64_t pg = bt[jj / page];
+          if (pg < 0) continue;                // its probability is 0
           const int off = jj % page;
           a += sc[jj - c0] * to_f32<T>(v_cache[((pg * Hkv + kvh) * (int64_t)D + d) * page + off]);
         }
@@ -100,7 +108,7 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
 extern "C" int me_attn_simple(const void* q, int64_t q_stride, void* out, int64_t out_stride, int dtype,
                               const void* k_cache, const void* v_cache, const int32_t* block_tables,
                               int bt_stride, const int32_t* seq_of_token, const int32_t* positions,
-                              int64_t num_tokens, int Hq, int Hkv, int D, int page, float scale, int window,
+                              const int32_t* context_lens, int64_t num_tokens, int Hq, int Hkv, int D, int page, float scale, int window,
                               hipStream_t stream) {
   if (num_tokens == 0) return 0;
   ME_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
@@ -111,11 +119,11 @@ extern "C" int me_attn_simple(const void* q, int64_t q_stride, void* out, int64_
   if (dtype == ME_F32)
     attn_simple_kernel<float><<<grid, block, lds, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_cache, (const float*)v_cache,
-        block_tables, bt_stride, seq_of_token, positions, Hq, Hkv, D, page, scale, window);
+        block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window);
   else if (dtype == ME_BF16)
     attn_simple_kernel<bf16_t><<<grid, block, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
-        block_tables, bt_stride, seq_of_token, positions, Hq, Hkv, D, page, scale, window);
+        block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window);
   else
     ME_CHECK(false, "attention: bad dtype code %d", dtype);
   ME_LAUNCH_CHECK();

@@ -1,0 +1,177 @@
+"""Decode steps as HIP graphs.
+
+A decode step of a small model is a few hundred short kernels; launched one by one their
+launch cost exceeds their run time. For steps in which every request brings exactly one
+token, the whole forward pass is captured once per (batch bucket, context cap) and replayed:
+the step's metadata lives in one device array of fixed layout that is rewritten before each
+replay. Rows beyond the real batch are padding: context length 0, slot -1 (nothing is
+written to the cache), token 0.
+
+The captured work is the same model code and kernels as the eager step; only the launch
+mechanism differs. Nothing is cleared with memset nodes inside the graph.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .context import GroupStep, StepContext
+
+BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+CONTEXT_STEP = 1024      # the context cap of a captured graph is a multiple of this
+
+
+def _pad4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class _Captured:
+    def __init__(self, runner, bucket: int, ctx_cap: int):
+        self.bucket, self.ctx_cap = bucket, ctx_cap
+        ps = runner.manager.page_size
+        self.G = runner.manager.num_groups
+        self.MB = -(-ctx_cap // ps)
+        B = bucket
+        self.seg, n = {}, 0
+        for name, size in (("tokens", B), ("positions", B), ("seq_of_token", B), ("context_lens", B), ("cu", B + 1),
+                           ("state_slots", B), ("first_chunk", B), ("rows", B)):
+            self.seg[name] = (n, size)
+            n += _pad4(size)
+        for g in range(self.G):
+            self.seg[f"slots{g}"] = (n, B); n += _pad4(B)
+            self.seg[f"bt{g}"] = (n, B * self.MB); n += _pad4(B * self.MB)
+        self.n = n
+        self.master = np.zeros(n, dtype=np.int32)            # host copy kept between steps
+        self.put("seq_of_token", np.arange(B))
+        self.put("cu", np.arange(B + 1))
+        self.put("rows", np.arange(B))
+        self.put("state_slots", -1)
+        for g in range(self.G):
+            self.put(f"bt{g}", -1)
+        self.row_req = [None] * B                            # which request's table a row holds
+        self.row_len = [[0] * B for _ in range(self.G)]      # how many of its entries are written
+        self.on_gpu = runner.device.type == "cuda"
+        self.pinned = [torch.empty(n, dtype=torch.int32, pin_memory=self.on_gpu) for _ in range(2)]
+        self.events = [None, None]
+        self.flip = 0
+        self.dev = torch.zeros(n, dtype=torch.int32, device=runner.device)
+        self.graph = None
+        self.logits = None
+
+    def put(self, name, values):
+        o, size = self.seg[name]
+        self.master[o:o + size] = values
+
+    def view(self, name):
+        o, size = self.seg[name]
+        return self.dev[o:o + size]
+
+    def context(self) -> StepContext:
+        B = self.bucket
+        return StepContext(
+            num_tokens=B, num_seqs=B, num_decodes=B, positions=self.view("positions"),
+            seq_of_token=self.view("seq_of_token"), context_lens=self.view("context_lens"),
+            cu_seqlens=self.view("cu"), prefill_cu=None, max_decode_context=self.ctx_cap,
+            groups=[GroupStep(self.view(f"bt{g}").view(B, self.MB), self.view(f"slots{g}")) for g in range(self.G)],
+            state_slots=self.view("state_slots"), first_chunk=self.view("first_chunk"),
+            q_lens=[1] * B, starts=[0] * B)
+
+    def upload(self):
+        i = self.flip
+        self.flip ^= 1
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        self.pinned[i].numpy()[:] = self.master
+        self.dev.copy_(self.pinned[i], non_blocking=True)
+        if self.on_gpu:
+            ev = torch.cuda.Event()
+            ev.record()
+            self.events[i] = ev
+
+
+class DecodeGraphs:
+    def __init__(self, runner, max_bucket: int = 256, capture: bool = True):
+        """capture=False runs the padded, fixed-layout step eagerly every time (no graph): the same
+        metadata path without the capture, for machines without a GPU."""
+        self.runner = runner
+        self.max_bucket = max_bucket
+        self.capture = capture
+        self.captured: dict = {}
+        self.replays = 0
+
+    def eligible(self, entries) -> bool:
+        r = self.runner
+        return ((r.device.type == "cuda" or not self.capture) and not r.pool.has_state and bool(r.plan.group_needs)
+                and len(entries) <= self.max_bucket and all(len(e.tokens) == 1 for e in entries))
+
+    def step(self, entries: list):
+        """Logits [len(entries), vocab] for a step in which every request brings one token."""
+        r = self.runner
+        B = len(entries)
+        bucket = next(b for b in BUCKETS if b >= B)
+        need_ctx = max(e.start for e in entries) + 1
+        ctx_cap = min(-(-need_ctx // CONTEXT_STEP) * CONTEXT_STEP, -(-r.max_positions // 8) * 8)
+        key = (bucket, ctx_cap)
+        cap = self.captured.get(key)
+        if cap is None:
+            cap = self.captured[key] = _Captured(r, bucket, ctx_cap)
+        ps = r.manager.page_size
+        tok = np.zeros(bucket, dtype=np.int64)
+        pos = np.zeros(bucket, dtype=np.int64)
+        ctx = np.zeros(bucket, dtype=np.int64)
+        tok[:B] = [e.tokens[0] for e in entries]
+        pos[:B] = [e.start for e in entries]
+        ctx[:B] = pos[:B] + 1
+        if r.vocab_size is not None and (tok.min() < 0 or tok.max() >= r.vocab_size):
+            raise ValueError(f"token id outside 0..{r.vocab_size - 1}")
+        cap.put("tokens", tok); cap.put("positions", pos); cap.put("context_lens", ctx)
+        cap.put("first_chunk", (pos == 0) & (ctx > 0))
+        for g in range(cap.G):
+            o, _ = cap.seg[f"bt{g}"]
+            bt = cap.master[o:o + bucket * cap.MB].reshape(bucket, cap.MB)
+            slots = np.full(bucket, -1, dtype=np.int64)
+            windowed = r.manager.groups[g].window is not None
+            for j, e in enumerate(entries):
+                t = r.manager.block_table(e.req, g)
+                if cap.row_req[j] != e.req or cap.row_len[g][j] > len(t) or windowed:
+                    bt[j, :] = -1
+                    cap.row_len[g][j] = 0
+                k = cap.row_len[g][j]
+                if len(t) > k:
+                    bt[j, k:len(t)] = t[k:]
+                    cap.row_len[g][j] = len(t)
+                page = t[e.start // ps] if e.start // ps < len(t) else -1
+                if page < 0:
+                    raise RuntimeError(f"request {e.req!r} has no page for position {e.start} (group {g}); "
+                                       f"allocate before stepping")
+                slots[j] = page * ps + e.start % ps
+            for j in range(B, bucket):
+                if cap.row_req[j] is not None:
+                    bt[j, :] = -1
+                    cap.row_len[g][j] = 0
+            cap.put(f"slots{g}", slots)
+        for j in range(bucket):
+            cap.row_req[j] = entries[j].req if j < B else None
+        cap.upload()
+        self.replays += 1
+        if not self.capture:
+            return self._forward(cap)[:B]
+        if cap.graph is None:
+            self._capture(cap)
+        cap.graph.replay()
+        return cap.logits[:B]
+
+    def _forward(self, cap: _Captured):
+        r = self.runner
+        h, residual = r.model.forward(cap.view("tokens"), cap.context(), r.pool.views, r.pool.states)
+        return r.model.logits(h, residual, cap.view("rows"))
+
+    def _capture(self, cap: _Captured) -> None:
+        # one eager run first: libraries load, scratch buffers get their size, the caching allocator warms up
+        # (it rewrites this step's cache entries with the same values the replay will write)
+        self._forward(cap)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            cap.logits = self._forward(cap)
+        cap.graph = graph

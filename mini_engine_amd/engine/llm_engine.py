@@ -49,7 +49,8 @@ class LLMEngine:
                                     num_state_slots=config.max_num_seqs if has_state else 0,
                                     enable_prefix_caching=config.enable_prefix_caching)
         self.runner = ModelRunner(self.model, self.manager, self.dtype, self.device, config.max_model_len,
-                                  poison_cache=bool(kwargs.get("poison_cache", False)))
+                                  poison_cache=bool(kwargs.get("poison_cache", False)),
+                                  use_graphs=config.use_graphs)
         self.tokenizer = _load_tokenizer(config.model)
         self.scheduler = Scheduler(config, self.manager)
         self.sampler = Sampler(self.runner, config.seed)

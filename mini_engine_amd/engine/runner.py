@@ -37,7 +37,7 @@ def _pad4(n: int) -> int:
 
 class ModelRunner:
     def __init__(self, model, manager: CacheManager, dtype: torch.dtype, device, max_positions: int,
-                 poison_cache: bool = False):
+                 poison_cache: bool = False, use_graphs: bool = False):
         self.model = model
         self.manager = manager
         self.dtype = dtype
@@ -52,6 +52,10 @@ class ModelRunner:
         if self.pool.has_state and manager.num_state_slots < 1:
             raise ValueError("the model keeps per-request state but the cache manager has no state slots")
         self.vocab_size = model.embedding.vocab_size if hasattr(model.embedding, "vocab_size") else None
+        self.graphs = None
+        if use_graphs:
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self, capture=self.device.type == "cuda")
         self._host = [None, None]
         self._events = [None, None]
         self._dev = None
@@ -107,6 +111,14 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
                     raise ValueError(f"request {e.req!r}: wanted place {w} outside its {len(e.tokens)} tokens")
+        if self.graphs is not None and self.graphs.eligible(entries):
+            logits = self.graphs.step(entries)
+            wanted = [i for i, e in enumerate(entries) if e.want]
+            if not wanted:
+                return None
+            if len(wanted) == len(entries):
+                return logits
+            return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
         # decodes (one new token) first, the others after, each kept in the caller's order
         order = [i for i, e in enumerate(entries) if len(e.tokens) == 1] + \
                 [i for i, e in enumerate(entries) if len(e.tokens) != 1]

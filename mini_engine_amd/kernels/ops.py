@@ -59,7 +59,7 @@ _CORE_PROTOS = {
     "me_silu_and_mul": [P, P, I, L, I, P],
     "me_qk_norm_rope_store": [P, I, L, L, P, P, F, P, L, P, P, P, P, I, I, I, I, I, P],
     "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
-    "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, L, I, I, I, I, F, I, P],
+    "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, I, I, P],
@@ -243,7 +243,8 @@ class HipBackend:
         if not mfma:
             core().call("me_attn_simple", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _code(q.dtype),
                         k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
-                        seq_of_token.data_ptr(), positions.data_ptr(), T, Hq, Hkv, D, page, float(scale), win, _stream())
+                        seq_of_token.data_ptr(), positions.data_ptr(), context_lens.data_ptr(), T, Hq, Hkv, D, page,
+                        float(scale), win, _stream())
             return out
         lib = attn_lib(D)
         es = q.element_size()
@@ -323,12 +324,15 @@ class HipBackend:
 SKINNY_MAX_M = 64
 _TARGET_WORKGROUPS = 512
 _scratch_buf: dict = {}
+_scratch_retired: list = []      # outgrown buffers stay alive: a captured graph may still write to them
 
 
 def _scratch(num_floats: int, device) -> torch.Tensor:
     buf = _scratch_buf.get(device)
     if buf is None or buf.numel() < num_floats:
-        buf = torch.empty((max(num_floats, 1 << 20),), dtype=torch.float32, device=device)
+        if buf is not None:
+            _scratch_retired.append(buf)
+        buf = torch.empty((max(2 * num_floats, 1 << 22),), dtype=torch.float32, device=device)
         _scratch_buf[device] = buf
     return buf
 

@@ -83,7 +83,11 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
         b = int(seq_of_token[t])
         pos = int(positions[t])
         lo = max(0, pos - window + 1) if window else 0
-        js = torch.arange(lo, pos + 1, device=q.device)
+        hi = min(pos + 1, int(context_lens[b]))            # a padding row (context 0) sees nothing
+        if hi <= lo:
+            out[t] = 0
+            continue
+        js = torch.arange(lo, hi, device=q.device)
         pages = block_tables[b, (js // page).long()].long()
         assert (pages >= 0).all(), "attention would read a page the request does not hold"
         offs = js % page

@@ -150,3 +150,32 @@ def test_replay_program_on_cpu(folders, plain_backend, tmp_path, monkeypatch, ca
     assert helpers.rel_err(rd(1), ra[20:21]) <= helpers.TOL_F32
     assert helpers.rel_err(rd(2), rb[[7, 11]]) <= helpers.TOL_F32
     assert helpers.rel_err(rd(3), ra[21:]) <= helpers.TOL_F32
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_padded_decode_layout_without_capture(folders, plain_backend, name):
+    """The fixed-layout decode step that HIP graphs replay (batch padded to a bucket, block tables
+    kept between steps and patched, rows changing owner), run eagerly on the CPU."""
+    V, page, folder = helpers.CONFIGS[name]["vocab_size"], helpers.PAGE[name], folders(name)
+    model = load_model(folder, "cpu", torch.float32, 512)
+    manager = CacheManager(80, page, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, torch.float32, "cpu", 512, poison_cache=True, use_graphs=True)
+    lens = {"a": 70, "b": 9, "c": 33, "d": 130, "e": 17}
+    ids = {r: helpers.random_ids(n + 24, V, 70 + i) for i, (r, n) in enumerate(lens.items())}
+    d = helpers.Driver(runner, manager)
+    d.step({r: ids[r][:lens[r]] for r in ("a", "b", "c")})
+    pos, live = dict(lens), ["a", "b", "c"]
+    for t in range(24):
+        if t == 5:
+            d.step({"d": ids["d"][:lens["d"]]}); live.append("d")
+        if t == 9:
+            live.remove("b"); manager.free("b"); d.fed.pop("b")
+        if t == 12:
+            d.step({"e": ids["e"][:lens["e"]]}); live.insert(0, "e")
+        d.step({r: ids[r][pos[r]:pos[r] + 1] for r in live})
+        for r in live:
+            pos[r] += 1
+    assert runner.graphs.replays == 24
+    for r in lens:
+        got = d.result(r)
+        assert helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]])) <= helpers.TOL_F32, r

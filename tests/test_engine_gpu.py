@@ -128,3 +128,40 @@ def test_pool_sizing_from_free_memory(folders):
     assert llm.config.num_kvcache_blocks == 4 * 8          # capped by what max_num_seqs requests can hold
     out = llm.generate([[1, 2, 3]], SamplingParams(temperature=0, max_tokens=3), use_tqdm=False)
     assert len(out[0]["token_ids"]) == 3
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_decode_graphs_replay_like_eager_steps(folders, dtype, name):
+    """Decode steps replayed from HIP graphs give the eager step's logits, on every replay, with
+    eager work (prefill of other requests, frees, reused pages) between the replays, batches that
+    change size and rows that change owner."""
+    env = Env(folders, dtype)
+    tol = env.tol
+    V = helpers.CONFIGS[name]["vocab_size"]
+    page = helpers.PAGE[name]
+    folder = folders(name)
+    model = load_model(folder, "cuda", dtype, 512)
+    manager = CacheManager(80, page, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, dtype, "cuda", 512, poison_cache=True, use_graphs=True)
+    lens = {"a": 70, "b": 9, "c": 33, "d": 130, "e": 17}
+    ids = {r: helpers.random_ids(n + 24, V, 70 + i) for i, (r, n) in enumerate(lens.items())}
+    d = helpers.Driver(runner, manager)
+    d.step({r: ids[r][:lens[r]] for r in ("a", "b", "c")})             # eager prefill
+    pos = dict(lens)
+    live = ["a", "b", "c"]
+    for t in range(24):
+        if t == 5:
+            d.step({"d": ids["d"][:lens["d"]]}); live.append("d")       # eager work between replays; bucket 3 -> 4
+        if t == 9:
+            live.remove("b"); manager.free("b"); d.fed.pop("b")         # rows change owner; bucket 4 -> 3
+        if t == 12:
+            d.step({"e": ids["e"][:lens["e"]]}); live.insert(0, "e")    # e reuses b's pages
+        d.step({r: ids[r][pos[r]:pos[r] + 1] for r in live})
+        for r in live:
+            pos[r] += 1
+    assert runner.graphs.replays >= 24
+    for r in lens:
+        got = d.result(r)
+        err = helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]]))
+        assert err <= tol, f"{name} {r}: {err:.3g}"
