@@ -48,7 +48,36 @@ extern "C" int me_gather_rows(const void* src, const int32_t* idx, void* out, in
 // y = w * r * rsqrt(mean(r^2) + eps)
 // x may be `num_partials` stacked float32 partial sums [P, T, n] (a split-K product whose
 // partial results are added here, in a fixed order) or one tensor of the compute dtype.
-template <typename TX, typename TY>
+// One workgroup per row; a thread owns groups of 4 consecutive elements, and all the loads of a
+// group (every partial, the residual) are issued before any is used.
+#define RN_MAX_PARTIALS 8
+
+template <typename TX> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Vec4<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = static_cast<float>(t[i]);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    bf16x4 t;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = static_cast<bf16_t>(v[i]);
+    *reinterpret_cast<bf16x4*>(p) = t;
+  }
+};
+
+// VEC: n % 4 == 0 and all pointers 16-byte aligned (rows then stay aligned); else scalar.
+template <typename TX, typename TY, bool VEC>
 __global__ void rms_norm_kernel(const TX* __restrict__ x, int num_partials, int64_t partial_stride,
                                 const float* __restrict__ res_in, float* __restrict__ res_out,
                                 const float* __restrict__ w, TY* __restrict__ y, int n, float eps) {
@@ -57,17 +86,54 @@ __global__ void rms_norm_kernel(const TX* __restrict__ x, int num_partials, int6
   const int64_t t = blockIdx.x;
   const TX* xr = x + t * n;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    float v = to_f32<TX>(xr[i]);
-    for (int p = 1; p < num_partials; ++p) v += to_f32<TX>(xr[p * partial_stride + i]);
-    if (res_in) v += res_in[t * n + i];
-    if (res_out) res_out[t * n + i] = v;
-    row[i] = v;
-    ss += v * v;
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
+      float part[RN_MAX_PARTIALS][4];
+#pragma unroll
+      for (int p = 0; p < RN_MAX_PARTIALS; ++p)
+        if (p < num_partials) Vec4<TX>::load(xr + p * partial_stride + i, part[p]);
+      float r[4] = {0.f, 0.f, 0.f, 0.f};
+      if (res_in) Vec4<float>::load(res_in + t * n + i, r);
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = part[0][e];
+#pragma unroll
+      for (int p = 1; p < RN_MAX_PARTIALS; ++p)
+        if (p < num_partials) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += part[p][e];
+        }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] += r[e];
+        ss += v[e] * v[e];
+        row[i + e] = v[e];
+      }
+      if (res_out) Vec4<float>::store(res_out + t * n + i, v);
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      float v = to_f32<TX>(xr[i]);
+      for (int p = 1; p < num_partials; ++p) v += to_f32<TX>(xr[p * partial_stride + i]);
+      if (res_in) v += res_in[t * n + i];
+      if (res_out) res_out[t * n + i] = v;
+      row[i] = v;
+      ss += v * v;
+    }
   }
   const float total = block_sum(ss, scratch);
   const float inv = rsqrtf(total / (float)n + eps);
-  for (int i = threadIdx.x; i < n; i += blockDim.x) y[t * n + i] = from_f32<TY>(w[i] * (row[i] * inv));
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
+      float wv[4], o[4];
+      Vec4<float>::load(w + i, wv);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = wv[e] * (row[i + e] * inv);
+      Vec4<TY>::store(y + t * n + i, o);
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) y[t * n + i] = from_f32<TY>(w[i] * (row[i] * inv));
+  }
 }
 
 extern "C" int me_rms_norm(const void* x, int x_dtype, int num_partials, int64_t partial_stride,
@@ -75,15 +141,26 @@ extern "C" int me_rms_norm(const void* x, int x_dtype, int num_partials, int64_t
                            int64_t num_rows, int n, float eps, hipStream_t stream) {
   if (num_rows == 0) return 0;
   ME_CHECK(n > 0 && n <= 36864, "rms_norm: width %d outside 1..36864", n);
-  ME_CHECK(num_partials >= 1, "rms_norm: num_partials must be >= 1");
+  ME_CHECK(num_partials >= 1 && num_partials <= RN_MAX_PARTIALS, "rms_norm: %d partial sums outside 1..%d",
+           num_partials, RN_MAX_PARTIALS);
   ME_CHECK(num_partials == 1 || x_dtype == ME_F32, "rms_norm: partial sums must be float32");
-  int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : (n >= 128 ? 128 : 64));
+  auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = n % 4 == 0 && al(x) && al(res_in) && al(res_out) && al(w) && al(y) &&
+                   (num_partials == 1 || partial_stride % 4 == 0);
+  int threads = vec ? (n / 4 >= 1024 ? 1024 : ((n / 4 + 63) / 64) * 64) : (n >= 512 ? 256 : (n >= 128 ? 128 : 64));
+  if (threads < 64) threads = 64;
   size_t lds = (size_t)n * sizeof(float);
   dim3 grid(num_rows), block(threads);
-#define LAUNCH(TX, TY)                                                                       \
-  rms_norm_kernel<TX, TY><<<grid, block, lds, stream>>>((const TX*)x, num_partials,          \
-                                                        partial_stride, res_in, res_out, w, \
-                                                        (TY*)y, n, eps)
+#define LAUNCH(TX, TY)                                                                                    \
+  do {                                                                                                    \
+    if (vec)                                                                                              \
+      rms_norm_kernel<TX, TY, true><<<grid, block, lds, stream>>>((const TX*)x, num_partials, partial_stride, \
+                                                                  res_in, res_out, w, (TY*)y, n, eps);   \
+    else                                                                                                  \
+      rms_norm_kernel<TX, TY, false><<<grid, block, lds, stream>>>((const TX*)x, num_partials,            \
+                                                                   partial_stride, res_in, res_out, w,   \
+                                                                   (TY*)y, n, eps);                      \
+  } while (0)
   if (x_dtype == ME_BF16 && y_dtype == ME_BF16) LAUNCH(bf16_t, bf16_t);
   else if (x_dtype == ME_F32 && y_dtype == ME_BF16) LAUNCH(float, bf16_t);
   else if (x_dtype == ME_F32 && y_dtype == ME_F32) LAUNCH(float, float);

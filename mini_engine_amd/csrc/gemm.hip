@@ -87,7 +87,19 @@ __device__ __forceinline__ bf16x8 gz8() {
 // MT: 16-token tiles per workgroup. Grid (ceil(N/16), ceil(M/(16*MT)), ksplit).
 // k-slot mapping of MFMA j (0..3) inside a 128-wide macro step s: lane group g supplies
 // k = 128 s + 32 g + 8 j + 0..7 for both operands, so a lane's four loads are 64 contiguous bytes.
-template <int MT, typename TO>
+// GATED: x is [M, 2K] and the B operand is silu(x[:, k]) * x[:, K + k], formed in float32 and
+// rounded once to bfloat16 (the SiLU-gating of the feed-forward fused into its down product).
+__device__ __forceinline__ bf16x8 silu_mul8(const bf16x8 g, const bf16x8 u) {
+  bf16x8 r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float gf = static_cast<float>(g[i]), uf = static_cast<float>(u[i]);
+    r[i] = static_cast<bf16_t>(gf / (1.f + expf(-gf)) * uf);
+  }
+  return r;
+}
+
+template <int MT, typename TO, bool GATED>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                    TO* __restrict__ y, int64_t ldy, float* __restrict__ partials, int M, int N, int K,
@@ -128,7 +140,11 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int k = kb + 8 * j;
-        const bf16x8 b = (xrow_ok[mt] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[mt] + k) : gz8();
+        bf16x8 b = (xrow_ok[mt] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[mt] + k) : gz8();
+        if (GATED) {
+          const bf16x8 u = (xrow_ok[mt] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[mt] + K + k) : gz8();
+          b = silu_mul8(b, u);
+        }
         acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b, acc[mt], 0, 0, 0);
       }
     }
@@ -153,7 +169,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
 // y: bf16 or float32 [M, N]; or, when ksplit > 1, `partials` float32 [ksplit, M, N] (y unused).
 extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y,
                                    int64_t ldy, int out_dtype, float* partials, int ksplit, int M, int N,
-                                   int K, hipStream_t stream) {
+                                   int K, int gated, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   ME_CHECK(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
            "skinny gemm: K=%d and the row strides must be multiples of 8", K);
@@ -166,9 +182,18 @@ extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, in
   const int mt = M > 32 ? 4 : (M > 16 ? 2 : 1);
   dim3 grid((N + 15) / 16, (M + 16 * mt - 1) / (16 * mt), ksplit), block(256);
   ME_CHECK(grid.y <= 65535, "skinny gemm: too many rows (%d)", M);
-#define LAUNCH(MTV, TO) \
-  gemm_skinny_kernel<MTV, TO><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, \
-                                                           (TO*)y, ldy, partials, M, N, K, steps_per_split)
+  ME_CHECK(!gated || ldx >= 2 * (int64_t)K, "skinny gemm: gated input rows must hold 2K values");
+#define LAUNCH(MTV, TO)                                                                                      \
+  do {                                                                                                       \
+    if (gated)                                                                                               \
+      gemm_skinny_kernel<MTV, TO, true><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, \
+                                                                    ldw, (TO*)y, ldy, partials, M, N, K,    \
+                                                                    steps_per_split);                       \
+    else                                                                                                     \
+      gemm_skinny_kernel<MTV, TO, false><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, \
+                                                                     ldw, (TO*)y, ldy, partials, M, N, K,   \
+                                                                     steps_per_split);                      \
+  } while (0)
   if (out_dtype == ME_F32 || partials) {
     if (mt == 4) LAUNCH(4, float); else if (mt == 2) LAUNCH(2, float); else LAUNCH(1, float);
   } else if (out_dtype == ME_BF16) {

@@ -19,45 +19,83 @@ __device__ __forceinline__ float exp_noise(uint32_t key0, uint32_t key1, uint32_
   return -logf(u);
 }
 
-__global__ void __launch_bounds__(1024)
-sample_kernel(const float* __restrict__ logits, int64_t ld, const float* __restrict__ temperatures,
-              const uint32_t* __restrict__ keys, int32_t* __restrict__ out, int V) {
-  __shared__ float bv[16];
-  __shared__ int bi[16];
-  const int row = blockIdx.x;
+// Stage 1: grid (chunks, rows). Each workgroup scans its share of the vocabulary and leaves its
+// best (score, index). Stage 2: one wave per row takes the best of the chunks. Ties go to the
+// lowest index at every stage, so the result does not depend on the number of chunks.
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+__global__ void __launch_bounds__(256)
+sample_scan_kernel(const float* __restrict__ logits, int64_t ld, const float* __restrict__ temperatures,
+                   const uint32_t* __restrict__ keys, float* __restrict__ part_v, int32_t* __restrict__ part_i,
+                   int V, int chunk) {
+  __shared__ float bv[4];
+  __shared__ int bi[4];
+  const int row = blockIdx.y, c = blockIdx.x;
   const float* z = logits + (int64_t)row * ld;
   const float T = temperatures[row];
   const uint32_t k0 = keys[2 * row], k1 = keys[2 * row + 1];
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int v = threadIdx.x; v < V; v += blockDim.x) {
+  const int end = min(V, (c + 1) * chunk);
+  for (int v = c * chunk + threadIdx.x; v < end; v += 256) {
     float s = z[v];
     if (T > 0.f) s = s / T - logf(exp_noise(k0, k1, (uint32_t)v));
-    if (s > best || (s == best && v < best_i)) { best = s; best_i = v; }
+    if (better(s, v, best, best_i)) { best = s; best_i = v; }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const float ov = __shfl_xor(best, off, ME_WAVE);
     const int oi = __shfl_xor(best_i, off, ME_WAVE);
-    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    if (better(ov, oi, best, best_i)) { best = ov; best_i = oi; }
   }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = (blockDim.x + 63) >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) { bv[wave] = best; bi[wave] = best_i; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < nwaves; ++w)
-      if (bv[w] > best || (bv[w] == best && bi[w] < best_i)) { best = bv[w]; best_i = bi[w]; }
-    out[row] = best_i == 0x7fffffff ? 0 : best_i;
+    for (int w = 1; w < 4; ++w)
+      if (better(bv[w], bi[w], best, best_i)) { best = bv[w]; best_i = bi[w]; }
+    part_v[(int64_t)row * gridDim.x + c] = best;
+    part_i[(int64_t)row * gridDim.x + c] = best_i;
   }
 }
 
-// keys: [S, 2] uint32 per row; temperatures: [S] float32 (0 = greedy); out: [S] int32.
+__global__ void __launch_bounds__(64)
+sample_merge_kernel(const float* __restrict__ part_v, const int32_t* __restrict__ part_i, int32_t* __restrict__ out,
+                    int chunks) {
+  const int row = blockIdx.x;
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    const float v = part_v[(int64_t)row * chunks + c];
+    const int i = part_i[(int64_t)row * chunks + c];
+    if (better(v, i, best, best_i)) { best = v; best_i = i; }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, ME_WAVE);
+    const int oi = __shfl_xor(best_i, off, ME_WAVE);
+    if (better(ov, oi, best, best_i)) { best = ov; best_i = oi; }
+  }
+  if (threadIdx.x == 0) out[row] = best_i == 0x7fffffff ? 0 : best_i;
+}
+
+// Scratch floats needed for S rows: (value, index) per chunk.
+extern "C" int me_sample_chunks(int V) { return V >= 16384 ? 32 : (V >= 2048 ? 4 : 1); }
+
+// keys: [S, 2] uint32 per row; temperatures: [S] float32 (0 = greedy); out: [S] int32;
+// scratch: 2 * S * me_sample_chunks(V) 4-byte words.
 extern "C" int me_sample(const float* logits, int64_t ld, const float* temperatures, const uint32_t* keys,
-                         int32_t* out, int S, int V, hipStream_t stream) {
+                         int32_t* out, void* scratch, int S, int V, hipStream_t stream) {
   if (S == 0) return 0;
   ME_CHECK(V >= 1 && ld >= V, "sample: bad vocabulary size or row stride");
-  const int threads = V >= 4096 ? 1024 : (V >= 512 ? 256 : 64);
-  sample_kernel<<<dim3(S), dim3(threads), 0, stream>>>(logits, ld, temperatures, keys, out, V);
+  ME_CHECK(S <= 65535, "sample: too many rows (%d)", S);
+  const int chunks = me_sample_chunks(V);
+  const int chunk = (V + chunks - 1) / chunks;
+  float* pv = (float*)scratch;
+  int32_t* pi = (int32_t*)scratch + (int64_t)S * chunks;
+  sample_scan_kernel<<<dim3(chunks, S), dim3(256), 0, stream>>>(logits, ld, temperatures, keys, pv, pi, V, chunk);
+  ME_LAUNCH_CHECK();
+  sample_merge_kernel<<<dim3(S), dim3(64), 0, stream>>>(pv, pi, out, chunks);
   ME_LAUNCH_CHECK();
   return 0;
 }

@@ -61,8 +61,8 @@ _CORE_PROTOS = {
     "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
-    "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
-    "me_sample": [P, L, P, P, P, I, I, P],
+    "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
+    "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
     "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, P],
@@ -297,13 +297,37 @@ class HipBackend:
             if ksplit > 1:
                 parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
                 core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
-                            ME_F32, parts.data_ptr(), ksplit, M, N, K, _stream())
+                            ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, _stream())
                 return parts
             y = torch.empty((M, N), dtype=out_dtype, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
-                        _code(out_dtype), None, 1, M, N, K, _stream())
+                        _code(out_dtype), None, 1, M, N, K, 0, _stream())
             return y
         return torch.matmul(x, w.t())
+
+    def silu_mul_linear(self, gu: torch.Tensor, w: torch.Tensor, allow_partials: bool = False):
+        """(silu(gu[:, :I]) * gu[:, I:]) . w[N, I]^T: the gating fused into the product for few
+        rows (bfloat16, M <= 16, where the product is a weight stream and the gating is free);
+        otherwise the two kernels one after the other (reference models/qwen3.py:50-51)."""
+        M, two_i = gu.shape
+        inter = two_i // 2
+        _check(w.shape[1] == inter and two_i == 2 * inter, f"silu_mul_linear: {tuple(gu.shape)} against {tuple(w.shape)}")
+        fused = (gu.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and M <= GATED_MAX_M and inter % 8 == 0
+                 and gu.is_contiguous() and w.stride(1) == 1 and w.stride(0) % 8 == 0
+                 and gu.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+        if not fused:
+            return self.linear(self.silu_and_mul(gu), w, None, allow_partials)
+        N = w.shape[0]
+        ksplit = choose_ksplit(M, N, inter) if allow_partials else 1
+        if ksplit > 1:
+            parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=gu.device)
+            core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), None, N,
+                        ME_F32, parts.data_ptr(), ksplit, M, N, inter, 1, _stream())
+            return parts
+        y = torch.empty((M, N), dtype=gu.dtype, device=gu.device)
+        core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
+                    ME_BF16, None, 1, M, N, inter, 1, _stream())
+        return y
 
     # -- sampling ------------------------------------------------------------------------
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:
@@ -316,13 +340,16 @@ class HipBackend:
                "sample: temperatures must be float32 [S]")
         _check(keys.dtype == torch.int32 and keys.shape == (S, 2) and keys.is_contiguous(), "sample: keys must be int32 [S, 2]")
         out = torch.empty((S,), dtype=torch.int32, device=logits.device)
+        scratch = torch.empty((2 * S * 32,), dtype=torch.int32, device=logits.device)
         core().call("me_sample", logits.data_ptr(), logits.stride(0), temperatures.data_ptr(), keys.data_ptr(),
-                    out.data_ptr(), S, V, _stream())
+                    out.data_ptr(), scratch.data_ptr(), S, V, _stream())
         return out
 
 
 SKINNY_MAX_M = 64
+GATED_MAX_M = 16
 _TARGET_WORKGROUPS = 512
+_DECODE_WORKGROUPS = 4096
 _scratch_buf: dict = {}
 _scratch_retired: list = []      # outgrown buffers stay alive: a captured graph may still write to them
 
@@ -347,15 +374,19 @@ def choose_ksplit(M: int, N: int, K: int) -> int:
 
 
 def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int) -> tuple:
-    """(keys per partition, number of partitions) for the split decode kernel: enough workgroups
-    to fill the GPU's compute units, partitions of at least 128 keys (the reference's rule is
-    layers/ops.py:44-51: split when sequences x kv heads cannot fill the SMs, 256-key partitions)."""
+    """(keys per partition, number of partitions) for the split decode kernel.
+
+    A workgroup's 4 waves take 32 keys each per round, so a partition of 128 keys is one round
+    with every load in flight at once; partitions grow beyond that only when (sequences x kv
+    heads x partitions) already gives several workgroups per compute unit, or to keep the
+    number of partitions to merge at 64 or less. (The reference's rule: layers/ops.py:44-51,
+    split when sequences x kv heads cannot fill the SMs, 256-key partitions.)"""
     col_tiles = (Hq // Hkv + 15) // 16
     base = max(1, num_seqs * Hkv * col_tiles)
-    want = max(1, -(-_TARGET_WORKGROUPS // base))
-    part = max(128, -(-max(1, max_context) // want))
-    part = -(-part // 128) * 128
-    parts = max(1, -(-max(1, max_context) // part))
+    ctx = max(1, max_context)
+    want = max(1, min(64, -(-_DECODE_WORKGROUPS // base)))
+    part = max(128, -(-(-(-ctx // want)) // 128) * 128)
+    parts = max(1, -(-ctx // part))
     return part, parts
 
 
@@ -385,4 +416,5 @@ def qk_norm_rope_store(*a, **k): return backend().qk_norm_rope_store(*a, **k)
 def store_kv(*a, **k): return backend().store_kv(*a, **k)
 def paged_attention(*a, **k): return backend().paged_attention(*a, **k)
 def linear(*a, **k): return backend().linear(*a, **k)
+def silu_mul_linear(*a, **k): return backend().silu_mul_linear(*a, **k)
 def sample(*a, **k): return backend().sample(*a, **k)

@@ -21,5 +21,4 @@ class SwiGLU(FeedForward):
 
     def forward(self, x):
         gu = self.gate_up.forward(x)
-        act = ops.silu_and_mul(gu)
-        return self.down.forward(act, allow_partials=True)
+        return ops.silu_mul_linear(gu, self.down.weight, allow_partials=True)

@@ -45,5 +45,6 @@ class RotaryEmbedding(PositionEncoding):
         half = self.head_dim // 2
         for x in (q, k):
             x1, x2 = x[..., :half].float(), x[..., half:].float()
-            x[..., :half] = (x1 * c - x2 * s).to(x.dtype)
-            x[..., half:] = (x2 * c + x1 * s).to(x.dtype)
+            lo, hi = x1 * c - x2 * s, x2 * c + x1 * s      # both halves before either is overwritten
+            x[..., :half] = lo.to(x.dtype)
+            x[..., half:] = hi.to(x.dtype)

@@ -106,6 +106,10 @@ def linear(x, w, out_dtype=None, allow_partials=False):
     return (x.float() @ w.float().t()).to(out_dtype or x.dtype)
 
 
+def silu_mul_linear(gu, w, allow_partials=False):
+    return linear(silu_and_mul(gu), w)
+
+
 def _fmix32(h):
     m = 0xFFFFFFFF
     h = h & m
@@ -146,4 +150,5 @@ class PlainBackend:
     store_kv = staticmethod(store_kv)
     paged_attention = staticmethod(paged_attention)
     linear = staticmethod(linear)
+    silu_mul_linear = staticmethod(silu_mul_linear)
     sample = staticmethod(sample)

@@ -247,6 +247,18 @@ def test_linear_skinny_bf16(M, N, K):
     close(parts.sum(0) if parts.dim() == 3 else parts, ref, 6e-3 if parts.dim() == 2 else 2e-5)
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40])
+@pytest.mark.parametrize("N,I", [(1024, 3072), (80, 224), (72, 200)])
+def test_silu_mul_linear(M, N, I):
+    """Gating fused into the down product (few rows) and the two-kernel form give the twin's result."""
+    gu = (torch.randn(M, 2 * I, device=DEV) * 2).bfloat16()
+    w = (torch.randn(N, I, device=DEV) * 0.05).bfloat16()
+    ref = twin.silu_and_mul(gu).double() @ w.double().t()        # the gated values rounded to bf16 once, as the kernel does
+    got = hip().silu_mul_linear(gu, w, allow_partials=True)
+    close(got.sum(0) if got.dim() == 3 else got, ref, 6e-3 if got.dim() == 2 else 3e-5)
+    close(hip().silu_mul_linear(gu, w), ref, 6e-3)
+
+
 def test_linear_partials_are_used_where_tiles_are_few():
     x = torch.randn(8, 3072, device=DEV).bfloat16()
     w = torch.randn(1024, 3072, device=DEV).bfloat16()

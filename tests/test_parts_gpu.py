@@ -62,7 +62,7 @@ def test_rotary_part_matches_plain_tables_and_unfused_apply():
     assert torch.allclose(rot.table[..., 1].double().cpu(), sin[:, :16], atol=3e-5)
     q, k = torch.randn(7, 3, 32, device=DEV), torch.randn(7, 1, 32, device=DEV)
     pos = torch.tensor([0, 5, 9, 100, 255, 1, 2], device=DEV, dtype=torch.int32)
-    qr = P.apply_rope(q.double().cpu(), cos, sin, pos.long().cpu())
+    qr = P.apply_rope(q.double().cpu(), cos32.double(), sin32.double(), pos.long().cpu())   # float32 angles, as above
     rot.apply(q, k, pos)
     assert torch.allclose(q.double().cpu(), qr, atol=1e-5)
 
