@@ -67,118 +67,205 @@ __device__ __forceinline__ bf16x8 zero8() {
 }
 __device__ __forceinline__ bf16x8 ld8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
+// Max / sum over the four lanes n, n+16, n+32, n+48 that share a column, left in all four.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of
+// its second, v_permlane32_swap the upper half of the first with the lower half of the second;
+// with both operands equal, the two results hold the two partners of every lane.
+__device__ __forceinline__ float max_over_groups(float v) {
+  unsigned u = __float_as_uint(v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  u = __float_as_uint(v);
+  auto r2 = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r2[0]), __uint_as_float(r2[1]));
+}
+__device__ __forceinline__ float sum_over_groups(float v) {
+  unsigned u = __float_as_uint(v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  u = __float_as_uint(v);
+  auto r2 = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r2[0]) + __uint_as_float(r2[1]);
+}
+
 __device__ __forceinline__ int page_index(int tok, int page, int shift) {
   return shift >= 0 ? (tok >> shift) : (tok / page);
 }
 
-// One 32-key block [t0, t0+32) against this wave's 16 columns.
-//   n = lane & 15 (column for B operands / row for A operands), g = lane >> 4.
-//   col_hi: last key position this lane's column may see (-1: column unused);
-//   col_lo: first key position it may see. lo_min: smallest col_lo of the whole call site, a
-//   bound below which pages may already have been given back (never loaded).
-__device__ __forceinline__ void attend32(const AttnArgs& a, const int32_t* __restrict__ bt, int kvh,
-                                         int t0, int L, int lo_min, const bf16x8 (&qb)[KS],
-                                         int col_lo, int col_hi, float& m, float& l,
-                                         f32x4 (&acc)[DT], int n, int g) {
-  // ---- scores: two 16-key tiles, rows permuted as described above
+// -------------------------------------------------------------------------------------
+// A 32-key block [t0, t0+32) of one kv head, as the operands of the two products.
+//   n = lane & 15 (row of an A operand), g = lane >> 4 (its 8-wide k-slot group).
+// Loads are unconditional: a lane whose keys are not to be read (at or past the context
+// length L, in a page behind a window that was given back, or in a table entry that holds no
+// page) reads from page 0 instead, which is always mapped, and its values are replaced by
+// zeros when they are used. So no load hides behind a branch and all of a block's loads are
+// in flight together; callers fetch the next block while they compute on the current one.
+// lo_min: a bound below which pages may already have been given back (never loaded).
+// -------------------------------------------------------------------------------------
+struct KVBlock {
+  bf16x8 k[2][KS];
+  bf16x8 v[DT];
+  bool kok[2];
+  uint32_t vmask[4];  // per 32-bit pair of this lane's 8 keys: which halves lie before L in a held page
+};
+
+// Page ids of a block, looked up one block before its keys and values are fetched, so that the
+// table read and the reads it addresses are not one chain of two latencies.
+struct BlockPages {
+  int kpage, koff, vpage, voff;  // kpage/vpage: table entries as loaded, not yet looked at
+  bool kgrp_ok, vgrp_ok;
+};
+
+// Only issues the two table reads; nothing here depends on what they return, so no wait is
+// placed behind them (a wait would also stall on every key/value load issued before).
+__device__ __forceinline__ void lookup_pages(const AttnArgs& a, const int32_t* __restrict__ bt, int t0, int L,
+                                             int lo_min, int n, int g, BlockPages& pg) {
   const int kgrp = t0 + 8 * (n >> 2);
-  bool kgrp_ok = kgrp < L && kgrp + 7 >= lo_min;
-  int kpi = 0, kpage = 0;
-  if (kgrp_ok) {
-    kpi = page_index(kgrp, a.page, a.page_shift);
-    kpage = bt[kpi];
-    kgrp_ok = kpage >= 0;  // a page that is not held is never dereferenced
+  pg.kgrp_ok = kgrp < L && kgrp + 7 >= lo_min;
+  const int kpi = pg.kgrp_ok ? page_index(kgrp, a.page, a.page_shift) : 0;
+  pg.kpage = bt[kpi];
+  pg.koff = pg.kgrp_ok ? kgrp - kpi * a.page + (n & 3) : (n & 3);
+  const int vgrp = t0 + 8 * g;
+  pg.vgrp_ok = vgrp < L && vgrp + 7 >= lo_min;
+  const int vpi = pg.vgrp_ok ? page_index(vgrp, a.page, a.page_shift) : 0;
+  pg.vpage = bt[vpi];
+  pg.voff = pg.vgrp_ok ? vgrp - vpi * a.page : 0;
+}
+
+__device__ __forceinline__ void load_kv(const AttnArgs& a, const BlockPages& pg, int kvh, int t0, int L, int n,
+                                        int g, KVBlock& blk) {
+  // a table entry that holds no page (-1) is treated like a key past the context: page 0, zeros
+  const bool kgrp_ok = pg.kgrp_ok && pg.kpage >= 0;
+  const int kpage = kgrp_ok ? pg.kpage : 0;
+  const int koff = kgrp_ok ? pg.koff : (n & 3);
+  // K rows: tile tt holds keys t0 + 8*(n/4) + 4*tt + (n%4)
+  const int kgrp = t0 + 8 * (n >> 2);
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    blk.kok[tt] = kgrp_ok && (kgrp + (n & 3) + 4 * tt) < L;
+    const bf16_t* kp = a.k_cache + (((int64_t)kpage * a.Hkv + kvh) * a.page + koff + 4 * tt) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = 32 * ks + 8 * g;
+      blk.k[tt][ks] = ld8(kp + ((HD % 32 == 0 || d0 < HD) ? d0 : 0));
+    }
   }
-  const int koff = kgrp - kpi * a.page + (n & 3);
+  // V^T rows: channel 16*dt + n, keys t0 + 8g .. t0 + 8g + 7
+  const bool vgrp_ok = pg.vgrp_ok && pg.vpage >= 0;
+  const int vpage = vgrp_ok ? pg.vpage : 0;
+  const int voff = vgrp_ok ? pg.voff : 0;
+  const bf16_t* vp = a.v_cache + (((int64_t)vpage * a.Hkv + kvh) * HD + n) * a.page + voff;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) blk.v[dt] = ld8(vp + (int64_t)dt * 16 * a.page);
+  // keys at or past L hold foreign or unwritten data (possibly NaN): their bits are cleared
+  const int nv = vgrp_ok ? L - (t0 + 8 * g) : 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    blk.vmask[j] = (2 * j < nv ? 0x0000ffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
+}
+
+__device__ __forceinline__ void load_block(const AttnArgs& a, const int32_t* __restrict__ bt, int kvh, int t0,
+                                           int L, int lo_min, int n, int g, KVBlock& blk) {
+  BlockPages pg;
+  lookup_pages(a, bt, t0, L, lo_min, n, g, pg);
+  load_kv(a, pg, kvh, t0, L, n, g, blk);
+}
+
+// Scores of the block against one 16-column tile, online-softmax update, and P.V.
+//   col_lo..col_hi: key positions this lane's column may see (col_hi = -1: column unused).
+//   The running max m is kept in the log2 domain: m = max(score) * c, c = scale * log2(e), so a
+//   probability is exp2(score * c - m): one fused multiply-add and one v_exp per score.
+//   FULL: every key of the block is visible to every column of the wave and lies before L in a
+//   held page, so nothing is masked or zeroed. Otherwise scores outside [col_lo, col_hi] are
+//   replaced, K rows and V keys that must not be read are zeroed.
+//   The accumulators are rescaled only when some column's max has risen (a wave-wide test).
+template <bool FULL>
+__device__ __forceinline__ void attend_block(const AttnArgs& a, const KVBlock& blk, int t0,
+                                             const bf16x8 (&qb)[KS], int col_lo, int col_hi, float& m, float& l,
+                                             f32x4 (&acc)[DT], int g) {
+  const bf16x8 z = zero8();
+  const float c = a.scale * 1.4426950408889634f;
   f32x4 st[2];
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt) {
-    const int tok = kgrp + (n & 3) + 4 * tt;
-    const bool ok = kgrp_ok && tok < L;
-    const bf16_t* kp = a.k_cache + (((int64_t)kpage * a.Hkv + kvh) * a.page + koff + 4 * tt) * HD + 8 * g;
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const bf16x8 ka = (ok && (32 * ks + 8 * g) < HD) ? ld8(kp + 32 * ks) : zero8();
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[ks], s, 0, 0, 0);
+      const bool dok = HD % 32 == 0 || (32 * ks + 8 * g) < HD;
+      const bf16x8 ka = ((FULL || blk.kok[tt]) && dok) ? blk.k[tt][ks] : z;
+      sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[ks], sacc, 0, 0, 0);
     }
-    st[tt] = s;
+    st[tt] = sacc;
   }
-
-  // ---- V^T operands (issued before the softmax arithmetic so the loads overlap it)
-  const int vgrp = t0 + 8 * g;
-  bool vgrp_ok = vgrp < L && vgrp + 7 >= lo_min;
-  int vpi = 0, vpage = 0;
-  if (vgrp_ok) {
-    vpi = page_index(vgrp, a.page, a.page_shift);
-    vpage = bt[vpi];
-    vgrp_ok = vpage >= 0;
-  }
-  const bf16_t* vp = a.v_cache + (((int64_t)vpage * a.Hkv + kvh) * HD + n) * a.page + (vgrp - vpi * a.page);
-  bf16x8 va[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) va[dt] = vgrp_ok ? ld8(vp + (int64_t)dt * 16 * a.page) : zero8();
-  if (vgrp_ok && vgrp + 8 > L) {  // tail: keys at or past L hold foreign or unwritten data
-    const int nv = L - vgrp;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (i >= nv) va[dt][i] = static_cast<bf16_t>(0.f);
-  }
-
-  // ---- mask, running max, probabilities (this lane: keys t0+8g+0..7 of column n)
-  float s[8];
-  bool keep[8];
+  // this lane: keys t0+8g+0..7 of its column
+  float sv[8];
   float bm = NEG;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int j = t0 + 8 * g + i;
-    keep[i] = j <= col_hi && j >= col_lo;
-    s[i] = keep[i] ? st[i >> 2][i & 3] * a.scale : NEG;
-    bm = fmaxf(bm, s[i]);
+    sv[i] = st[i >> 2][i & 3];
+    if (!FULL) {
+      const int j = t0 + 8 * g + i;
+      sv[i] = (j <= col_hi && j >= col_lo) ? sv[i] : NEG;
+    }
+    bm = fmaxf(bm, sv[i]);
   }
-  bm = fmaxf(bm, __shfl_xor(bm, 16, ME_WAVE));
-  bm = fmaxf(bm, __shfl_xor(bm, 32, ME_WAVE));
-  const float m_new = fmaxf(m, bm);
-  const float alpha = __expf(m - m_new);
+  bm = max_over_groups(bm);
+  const float m_new = fmaxf(m, bm > 0.5f * NEG ? bm * c : NEG);
+  const bool rose = m_new > m;
   float psum = 0.f;
   bf16x8 pb;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float p = keep[i] ? __expf(s[i] - m_new) : 0.f;
+    float p = __builtin_amdgcn_exp2f(fmaf(sv[i], c, -m_new));
+    if (!FULL) p = sv[i] > 0.5f * NEG ? p : 0.f;
     psum += p;
     pb[i] = static_cast<bf16_t>(p);
   }
-  l = l * alpha + psum;  // this lane's share of the column's sum; the 4 shares are added at the end
-  m = m_new;
+  if (__any(rose)) {
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    l *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      acc[dt][0] *= alpha; acc[dt][1] *= alpha; acc[dt][2] *= alpha; acc[dt][3] *= alpha;
+    }
+    m = m_new;
+  }
+  l += psum;  // this lane's share of the column's sum; the 4 shares are added at the end
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
-    f32x4 o = acc[dt];
-    o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt], pb, o, 0, 0, 0);
+    bf16x8 va = blk.v[dt];
+    if (!FULL) {
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      u32x4 vb = __builtin_bit_cast(u32x4, va);
+      vb[0] &= blk.vmask[0]; vb[1] &= blk.vmask[1]; vb[2] &= blk.vmask[2]; vb[3] &= blk.vmask[3];
+      va = __builtin_bit_cast(bf16x8, vb);
+    }
+    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, acc[dt], 0, 0, 0);
   }
 }
 
 __device__ __forceinline__ void load_q(const bf16_t* qrow, bool valid, int g, bf16x8 (&qb)[KS]) {
+  const bf16x8 z = zero8();
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    qb[ks] = (valid && (32 * ks + 8 * g) < HD) ? ld8(qrow + 32 * ks + 8 * g) : zero8();
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = 32 * ks + 8 * g;
+    const bool dok = HD % 32 == 0 || d0 < HD;
+    const bf16x8 v = ld8(qrow + (dok ? d0 : 0));
+    qb[ks] = (valid && dok) ? v : z;
+  }
 }
 
-__device__ __forceinline__ float column_sum(float l) {
-  l += __shfl_xor(l, 16, ME_WAVE);
-  l += __shfl_xor(l, 32, ME_WAVE);
-  return l;
-}
+__device__ __forceinline__ float column_sum(float l) { return sum_over_groups(l); }
 
 // =====================================================================================
-// Prefill / chunk kernel: each wave owns 16 columns of a (tok_tile tokens x G heads) tile of
-// one sequence and one kv head, and walks the keys [lo, hi) its columns may see.
+// Prefill / chunk kernel: each wave owns CT tiles of 16 columns of a (tok_tile tokens x G heads)
+// tile of one sequence and one kv head, and walks the keys [lo, hi) its columns may see, the next
+// block being fetched while the current one is used. Every K/V register serves CT products.
 // Grid: (floor(T / tok_tile) + num_seqs, Hkv). The first tile of sequence b is
 // floor(cu[b] / tok_tile) + b, an upper bound of the tiles before it; surplus tiles exit.
 // =====================================================================================
-__global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
+template <int CT>
+__global__ void __launch_bounds__(256, CT == 1 ? 2 : 1) attn_prefill_kernel(AttnArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int kvh = blockIdx.y;
@@ -201,38 +288,85 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   const int ncols = tile_tokens * a.G;
   const int tile_lo = a.window > 0 ? max(0, start + tok0 - a.window + 1) : 0;
 
-  for (int ct = wave; ct * 16 < ncols; ct += 4) {
-    const int c = ct * 16 + n;
-    const bool valid = c < ncols;
-    const int tl = valid ? c / a.G : 0;
-    const int hh = c - tl * a.G;
-    const int64_t t = q0 + tok0 + tl;
-    const int head = kvh * a.G + hh;
-    const int pos = start + tok0 + tl;
-    const int col_hi = valid ? pos : -1;
-    const int col_lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-    bf16x8 qb[KS];
-    load_q(a.q + t * a.q_stride + (int64_t)head * HD, valid, g, qb);
+  for (int c0 = wave * 16 * CT; c0 < ncols; c0 += 4 * 16 * CT) {
+    bf16x8 qb[CT][KS];
+    int col_lo[CT], col_hi[CT];
+    int64_t tq[CT];
+    int head[CT];
+    bool valid[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int c = c0 + 16 * ct + n;
+      valid[ct] = c < ncols;
+      const int tl = valid[ct] ? c / a.G : 0;
+      const int hh = valid[ct] ? c - tl * a.G : 0;
+      tq[ct] = q0 + tok0 + tl;
+      head[ct] = kvh * a.G + hh;
+      const int pos = start + tok0 + tl;
+      col_hi[ct] = valid[ct] ? pos : -1;
+      col_lo[ct] = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+      load_q(a.q + tq[ct] * a.q_stride + (int64_t)head[ct] * HD, valid[ct], g, qb[ct]);
+    }
     // keys this wave needs: from the window start of its first column to its last column's position
-    const int c_first = ct * 16, c_last = min(ncols, ct * 16 + 16) - 1;
-    const int pos_first = start + tok0 + c_first / a.G, pos_last = start + tok0 + c_last / a.G;
+    const int c_last = min(ncols, c0 + 16 * CT) - 1;
+    const int pos_first = start + tok0 + c0 / a.G, pos_last = start + tok0 + c_last / a.G;
     const int w_lo = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
-    float m = NEG, l = 0.f;
-    f32x4 acc[DT];
+    float m[CT], l[CT];
+    f32x4 acc[CT][DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int t0 = w_lo & ~31; t0 <= pos_last; t0 += 32)
-      attend32(a, bt, kvh, t0, L, tile_lo, qb, col_lo, col_hi, m, l, acc, n, g);
-    l = column_sum(l);
-    if (valid) {
-      const float inv = l > 0.f ? 1.f / l : 0.f;
-      bf16_t* o = a.out + t * a.out_stride + (int64_t)head * HD + 4 * g;
+    for (int ct = 0; ct < CT; ++ct) {
+      m[ct] = NEG; l[ct] = 0.f;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        bf16x4 r;
+      for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    // pipeline: page ids two blocks ahead, keys and values one block ahead of the products. The
+    // fetches are unconditional, also past the last block (they then read page 0 and are not used):
+    // a fetch behind a branch would make the waits of both paths merge into waits on the newest loads.
+    // a block all of whose keys every column of this wave sees (below the first column's position,
+    // above the last column's window start) takes the path without masks
+    const int full_hi = pos_first - 31;                                   // t0 <= full_hi: all 32 keys visible
+    const int full_lo = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;  // t0 >= full_lo: none behind a window
+#define ATTEND(BLK)                                                                                          \
+  do {                                                                                                       \
+    if (t0 <= full_hi && t0 >= full_lo) {                                                                    \
+      _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                      \
+          attend_block<true>(a, BLK, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);          \
+    } else {                                                                                                 \
+      _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                      \
+          attend_block<false>(a, BLK, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);         \
+    }                                                                                                        \
+  } while (0)
+    KVBlock A, B;
+    BlockPages pn;
+    int t0 = w_lo & ~31;
+    load_block(a, bt, kvh, t0, L, tile_lo, n, g, A);
+    lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
+    while (true) {
+      load_kv(a, pn, kvh, t0 + 32, L, n, g, B);
+      lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
+      ATTEND(A);
+      t0 += 32;
+      if (t0 > pos_last) break;
+      load_kv(a, pn, kvh, t0 + 32, L, n, g, A);
+      lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
+      ATTEND(B);
+      t0 += 32;
+      if (t0 > pos_last) break;
+    }
+#undef ATTEND
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r[i] = static_cast<bf16_t>(acc[dt][i] * inv);
-        *reinterpret_cast<bf16x4*>(o + 16 * dt) = r;
+    for (int ct = 0; ct < CT; ++ct) {
+      const float ls = column_sum(l[ct]);
+      if (valid[ct]) {
+        const float inv = ls > 0.f ? 1.f / ls : 0.f;
+        bf16_t* o = a.out + tq[ct] * a.out_stride + (int64_t)head[ct] * HD + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          bf16x4 r;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) r[i] = static_cast<bf16_t>(acc[ct][dt][i] * inv);
+          *reinterpret_cast<bf16x4*>(o + 16 * dt) = r;
+        }
       }
     }
   }
@@ -244,8 +378,8 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
 // through LDS. With one partition the result is written directly; otherwise the partition's
 // (max, sum, unnormalised output) go to scratch for the reduce kernel.
 // =====================================================================================
-__global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs a) {
-  extern __shared__ float lds[];  // [4 waves][16 cols][HD + 2]
+__global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
+  extern __shared__ float lds[];  // [4 waves][cols][HD + 2]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int b = blockIdx.x;
@@ -256,46 +390,58 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs a) {
   const int pos = L - 1;
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int32_t* bt = a.block_tables + (int64_t)b * a.bt_stride;
-  const int hh = ctile * 16 + n;
-  const bool valid = hh < a.G;
-  const int head = kvh * a.G + (valid ? hh : 0);
+  const int ncols = min(16, a.G - ctile * 16);
+  const bool valid = n < ncols;
+  const int head = kvh * a.G + ctile * 16 + (valid ? n : 0);
   const int64_t t = b;  // decode rows come first in the batch: token index == sequence index
 
-  bf16x8 qb[KS];
-  load_q(a.q + t * a.q_stride + (int64_t)head * HD, valid, g, qb);
+  const int p_lo = max(part * a.part_size, lo & ~31);
+  const int p_hi = min((part + 1) * a.part_size, L);
   float m = NEG, l = 0.f;
   f32x4 acc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  const int p_lo = max(part * a.part_size, lo & ~31);
-  const int p_hi = min((part + 1) * a.part_size, L);
-  for (int t0 = p_lo + 32 * wave; t0 < p_hi; t0 += 128)
-    attend32(a, bt, kvh, t0, L, lo, qb, lo, valid ? pos : -1, m, l, acc, n, g);
+  // One block buffer only: the registers saved let several workgroups share a compute unit,
+  // and it is their interleaving that hides the load latency here (partitions are short).
+  int t0 = p_lo + 32 * wave;
+  if (t0 < p_hi) {
+    KVBlock A;
+    load_block(a, bt, kvh, t0, L, lo, n, g, A);
+    bf16x8 qb[KS];
+    load_q(a.q + t * a.q_stride + (int64_t)head * HD, valid, g, qb);
+    const int col_hi = valid ? pos : -1;
+    while (true) {
+      if (t0 + 32 <= L && t0 >= lo) attend_block<true>(a, A, t0, qb, lo, col_hi, m, l, acc, g);
+      else attend_block<false>(a, A, t0, qb, lo, col_hi, m, l, acc, g);
+      t0 += 128;
+      if (t0 >= p_hi) break;
+      load_block(a, bt, kvh, t0, L, lo, n, g, A);
+    }
+  }
   l = column_sum(l);
 
-  // ---- merge the 4 waves
+  // ---- merge the 4 waves: only the columns in use pass through LDS
   const int stride = HD + 2;
-  float* mine = lds + ((wave * 16 + n) * stride);
-  if (g == 0) { mine[HD] = m; mine[HD + 1] = l; }
+  if (valid) {
+    float* mine = lds + ((wave * ncols + n) * stride);
+    if (g == 0) { mine[HD] = m; mine[HD + 1] = l; }
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) mine[16 * dt + 4 * g + i] = acc[dt][i];
+      for (int i = 0; i < 4; ++i) mine[16 * dt + 4 * g + i] = acc[dt][i];
+  }
   __syncthreads();
-  // thread -> (column, channel) pairs
-  const int ncols = min(16, a.G - ctile * 16);
   for (int e = threadIdx.x; e < ncols * HD; e += 256) {
     const int c = e / HD, d = e - c * HD;
     float M = NEG;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, lds[(w * 16 + c) * stride + HD]);
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, lds[(w * ncols + c) * stride + HD]);
     float o = 0.f, ls = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const float f = __expf(lds[(w * 16 + c) * stride + HD] - M);
-      o += f * lds[(w * 16 + c) * stride + d];
-      ls += f * lds[(w * 16 + c) * stride + HD + 1];
+      const float f = exp2f(lds[(w * ncols + c) * stride + HD] - M);
+      o += f * lds[(w * ncols + c) * stride + d];
+      ls += f * lds[(w * ncols + c) * stride + HD + 1];
     }
     const int hq = kvh * a.G + ctile * 16 + c;
     if (a.num_parts == 1) {
@@ -308,18 +454,31 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs a) {
   }
 }
 
-// Reduce over partitions: out = sum_p e^{m_p - M} o_p / sum_p e^{m_p - M} l_p. Grid (num_seqs, Hq).
-__global__ void attn_reduce_kernel(AttnArgs a) {
+// Reduce over partitions: out = sum_p e^{m_p - M} o_p / sum_p e^{m_p - M} l_p. Grid (num_seqs, Hq);
+// the weights of the partitions are formed once, in LDS, then every thread sums its channel.
+#define RED_MAX_PARTS 64
+__global__ void __launch_bounds__(128) attn_reduce_kernel(AttnArgs a) {
+  __shared__ float wgt[RED_MAX_PARTS];
+  __shared__ float inv_s;
   const int b = blockIdx.x, hq = blockIdx.y;
   const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_parts;
-  float M = NEG;
-  for (int p = 0; p < a.num_parts; ++p) M = fmaxf(M, a.tmp_m[row0 + p]);
-  float ls = 0.f;
-  for (int p = 0; p < a.num_parts; ++p) ls += __expf(a.tmp_m[row0 + p] - M) * a.tmp_l[row0 + p];
-  const float inv = ls > 0.f ? 1.f / ls : 0.f;
+  const int P = a.num_parts;
+  if (threadIdx.x < 64) {
+    const int p = threadIdx.x;
+    const float mp = p < P ? a.tmp_m[row0 + p] : NEG;
+    const float lp = p < P ? a.tmp_l[row0 + p] : 0.f;
+    const float M = wave_max(mp);
+    const float f = p < P ? exp2f(mp - M) : 0.f;
+    const float ls = wave_sum(f * lp);
+    wgt[p] = f;
+    if (p == 0) inv_s = ls > 0.f ? 1.f / ls : 0.f;
+  }
+  __syncthreads();
+  const float inv = inv_s;
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
     float o = 0.f;
-    for (int p = 0; p < a.num_parts; ++p) o += __expf(a.tmp_m[row0 + p] - M) * a.tmp_out[(row0 + p) * HD + d];
+#pragma unroll 8
+    for (int p = 0; p < P; ++p) o += wgt[p] * a.tmp_out[(row0 + p) * HD + d];
     a.out[(int64_t)b * a.out_stride + (int64_t)hq * HD + d] = static_cast<bf16_t>(o * inv);
   }
 }
@@ -342,6 +501,7 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
                (reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) && (reinterpret_cast<uintptr_t>(v_cache) % 16 == 0),
            "attention: q, out and cache pointers must be 16-byte aligned");
   ME_CHECK(window >= 0 && bt_stride >= 1, "attention: bad window or block-table stride");
+  ME_CHECK(scale > 0.f, "attention: the score scale must be positive");
   a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
   a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
   a.block_tables = block_tables; a.bt_stride = bt_stride; a.context_lens = context_lens;
@@ -359,16 +519,21 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                                const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                int bt_stride, const int32_t* context_lens, const int32_t* cu_seqlens,
                                int num_seqs, int64_t num_tokens, int Hq, int Hkv, int page, float scale,
-                               int window, hipStream_t stream) {
+                               int window, int col_tiles_per_wave, hipStream_t stream) {
   if (num_seqs == 0 || num_tokens == 0) return 0;
   AttnArgs a;
   if (fill_common(a, q, q_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
                   num_seqs, Hq, Hkv, page, scale, window)) return -1;
   a.cu_seqlens = cu_seqlens;
-  a.tok_tile = a.G >= 64 ? 1 : 64 / a.G;
+  // column tiles per wave: 2 when the step has enough tokens to fill the GPU with the larger tiles
+  const int ct = (col_tiles_per_wave == 1 || col_tiles_per_wave == 2) ? col_tiles_per_wave
+                 : ((num_tokens * Hq >= 32768 && HD <= 128) ? 2 : 1);
+  const int cols = 64 * ct;
+  a.tok_tile = a.G >= cols ? 1 : cols / a.G;
   const int64_t tiles = num_tokens / a.tok_tile + num_seqs;
   ME_CHECK(tiles < (1ll << 31), "attention: too many tiles");
-  attn_prefill_kernel<<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  if (ct == 2) attn_prefill_kernel<2><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  else attn_prefill_kernel<1><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
   ME_LAUNCH_CHECK();
   return 0;
 }
@@ -387,7 +552,7 @@ extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_
   AttnArgs a;
   if (fill_common(a, q, q_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
                   num_seqs, Hq, Hkv, page, scale, window)) return -1;
-  ME_CHECK(num_parts >= 1 && num_parts <= 65535, "attention: %d partitions outside 1..65535", num_parts);
+  ME_CHECK(num_parts >= 1 && num_parts <= RED_MAX_PARTS, "attention: %d partitions outside 1..%d", num_parts, RED_MAX_PARTS);
   ME_CHECK(num_parts == 1 || (part_size >= 32 && part_size % 32 == 0),
            "attention: partition size %d must be a multiple of 32", part_size);
   ME_CHECK(num_parts == 1 || scratch != nullptr, "attention: split decode needs scratch");
@@ -399,7 +564,7 @@ extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_
   }
   const int col_tiles = (a.G + 15) / 16;
   ME_CHECK((int64_t)Hkv * col_tiles <= 65535, "attention: too many heads for one launch");
-  const size_t lds = (size_t)4 * 16 * (HD + 2) * sizeof(float);
+  const size_t lds = (size_t)4 * (a.G < 16 ? a.G : 16) * (HD + 2) * sizeof(float);
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)attn_decode_kernel,
@@ -410,7 +575,7 @@ extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_
   attn_decode_kernel<<<dim3(num_seqs, Hkv * col_tiles, num_parts), dim3(256), lds, stream>>>(a);
   ME_LAUNCH_CHECK();
   if (num_parts > 1) {
-    attn_reduce_kernel<<<dim3(num_seqs, Hq), dim3(HD >= 128 ? 128 : 64), 0, stream>>>(a);
+    attn_reduce_kernel<<<dim3(num_seqs, Hq), dim3(128), 0, stream>>>(a);
     ME_LAUNCH_CHECK();
   }
   return 0;

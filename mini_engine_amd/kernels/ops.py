@@ -62,10 +62,11 @@ _CORE_PROTOS = {
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
+    "me_gemm_wide_bf16": [P, L, P, L, P, L, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
-    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, P],
+    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, P],
     "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, P],
 }
 
@@ -260,7 +261,7 @@ class HipBackend:
                      out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
                      block_tables.stride(0), context_lens.data_ptr() + num_decodes * 4, prefill_cu.data_ptr(),
-                     B - num_decodes, T - num_decodes, Hq, Hkv, page, float(scale), win, _stream())
+                     B - num_decodes, T - num_decodes, Hq, Hkv, page, float(scale), win, PREFILL_COL_TILES, _stream())
         return out
 
     # -- matrix products -----------------------------------------------------------------
@@ -291,6 +292,12 @@ class HipBackend:
             y = torch.empty((M, N), dtype=out_dtype, device=x.device)
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
+            return y
+        if (M <= SKINNY_MAX_M or out_dtype == torch.float32) and N >= WIDE_MIN_N:
+            # a very wide output (the head over the vocabulary): one wave per feature tile, whole K
+            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            core().call("me_gemm_wide_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
+                        _code(out_dtype), M, N, K, _stream())
             return y
         if M <= SKINNY_MAX_M or out_dtype == torch.float32:
             ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= SKINNY_MAX_M) else 1
@@ -347,6 +354,8 @@ class HipBackend:
 
 
 SKINNY_MAX_M = 64
+WIDE_MIN_N = 32768
+PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 GATED_MAX_M = 16
 _TARGET_WORKGROUPS = 512
 _DECODE_WORKGROUPS = 4096

@@ -255,7 +255,9 @@ def test_silu_mul_linear(M, N, I):
     w = (torch.randn(N, I, device=DEV) * 0.05).bfloat16()
     ref = twin.silu_and_mul(gu).double() @ w.double().t()        # the gated values rounded to bf16 once, as the kernel does
     got = hip().silu_mul_linear(gu, w, allow_partials=True)
-    close(got.sum(0) if got.dim() == 3 else got, ref, 6e-3 if got.dim() == 2 else 3e-5)
+    # float32 partial sums: what remains is that a gated value next to a rounding boundary may round to
+    # the other bf16 neighbour than the twin's (expf against sigmoid): 2^-8 on a few percent of the terms
+    close(got.sum(0) if got.dim() == 3 else got, ref, 6e-3 if got.dim() == 2 else 1e-3)
     close(hip().silu_mul_linear(gu, w), ref, 6e-3)
 
 
