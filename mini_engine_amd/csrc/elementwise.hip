@@ -173,16 +173,31 @@ extern "C" int me_rms_norm(const void* x, int x_dtype, int num_partials, int64_t
 
 // ------------------------------------------------------------------ SiLU(gate) * up
 // gu: [T, 2I] with gate = first I columns (reference layers/activation.py:6); out: [T, I].
-template <typename T>
+// VEC: a thread takes 16 bytes of gate and of up at a time (I a multiple of the vector length).
+template <typename T, bool VEC>
 __global__ void silu_and_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t rows, int inter) {
-  const int64_t total = rows * (int64_t)inter;
+  constexpr int W = VEC ? 16 / sizeof(T) : 1;
+  const int per_row = inter / W;
+  const int64_t total = rows * (int64_t)per_row;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
        e += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t t = e / inter;
-    const int i = (int)(e - t * inter);
-    const float g = to_f32<T>(gu[t * 2 * inter + i]);
-    const float u = to_f32<T>(gu[t * 2 * inter + inter + i]);
-    out[e] = from_f32<T>(g / (1.f + expf(-g)) * u);
+    const int64_t t = e / per_row;
+    const int i = (int)(e - t * per_row) * W;
+    alignas(16) T g[W], u[W], o[W];
+    if (VEC) {
+      *reinterpret_cast<uint4*>(g) = *reinterpret_cast<const uint4*>(gu + t * 2 * inter + i);
+      *reinterpret_cast<uint4*>(u) = *reinterpret_cast<const uint4*>(gu + t * 2 * inter + inter + i);
+    } else {
+      g[0] = gu[t * 2 * inter + i];
+      u[0] = gu[t * 2 * inter + inter + i];
+    }
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      const float gf = to_f32<T>(g[j]);
+      o[j] = from_f32<T>(gf / (1.f + expf(-gf)) * to_f32<T>(u[j]));
+    }
+    if (VEC) *reinterpret_cast<uint4*>(out + t * inter + i) = *reinterpret_cast<const uint4*>(o);
+    else out[t * inter + i] = o[0];
   }
 }
 
@@ -190,15 +205,20 @@ extern "C" int me_silu_and_mul(const void* gu, void* out, int dtype, int64_t row
                                hipStream_t stream) {
   if (rows == 0) return 0;
   ME_CHECK(inter > 0, "silu_and_mul: intermediate size must be positive");
-  const int64_t total = rows * (int64_t)inter;
+  ME_CHECK(dtype == ME_BF16 || dtype == ME_F32, "silu_and_mul: bad dtype code %d", dtype);
+  const int w = dtype == ME_BF16 ? 8 : 4;
+  const bool vec = inter % w == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int64_t total = rows * (int64_t)(vec ? inter / w : inter);
   int64_t blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
-  if (dtype == ME_BF16)
-    silu_and_mul_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, rows, inter);
-  else if (dtype == ME_F32)
-    silu_and_mul_kernel<float><<<dim3(blocks), dim3(256), 0, stream>>>((const float*)gu, (float*)out, rows, inter);
-  else
-    ME_CHECK(false, "silu_and_mul: bad dtype code %d", dtype);
+  dim3 grid(blocks), block(256);
+  if (dtype == ME_BF16) {
+    if (vec) silu_and_mul_kernel<bf16_t, true><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, rows, inter);
+    else silu_and_mul_kernel<bf16_t, false><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, rows, inter);
+  } else {
+    if (vec) silu_and_mul_kernel<float, true><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, rows, inter);
+    else silu_and_mul_kernel<float, false><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, rows, inter);
+  }
   ME_LAUNCH_CHECK();
   return 0;
 }

@@ -15,6 +15,42 @@
 
 #define ME_MAX_PAIRS 4  // pairs per lane: head_dim <= 2 * 64 * ME_MAX_PAIRS
 
+// A value head of token t into its transposed page.
+// Tokens are taken 8 at a time (by the workgroup of the group's first token): when their slots
+// are 8 consecutive places of one page, a channel's 8 values are one 16-byte store; a lane
+// reads them with 8 loads that are each contiguous across the lanes.
+template <typename T>
+__device__ void store_value_head(const T* row, int64_t row_stride, int64_t t, int64_t num_tokens,
+                                 const int32_t* slots, T* v_cache, int Hkv, int kvh, int D, int page, int lane) {
+  if (t & 7) return;
+  const int cnt = (int)min((int64_t)8, num_tokens - t);
+  const int s0 = slots[t];
+  bool run = cnt == 8 && s0 >= 0 && (s0 & 7) == 0 && page % 8 == 0;
+  if (run) {
+#pragma unroll
+    for (int i = 1; i < 8; ++i) run = run && slots[t + i] == s0 + i;
+  }
+  if (run) {
+    const int64_t pg = s0 / page, off = s0 - pg * page;
+    T* dst = v_cache + ((pg * Hkv + kvh) * (int64_t)D) * page + off;
+    for (int d = lane; d < D; d += 64) {
+      alignas(16) T vals[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) vals[i] = row[i * row_stride + d];
+      *reinterpret_cast<uint4*>(dst + (int64_t)d * page) = *reinterpret_cast<const uint4*>(vals);
+      if (sizeof(T) == 4) *reinterpret_cast<uint4*>(dst + (int64_t)d * page + 4) = *reinterpret_cast<const uint4*>(vals + 4);
+    }
+    return;
+  }
+  for (int i = 0; i < cnt; ++i) {
+    const int slot = slots[t + i];
+    if (slot < 0) continue;
+    const int64_t pg = slot / page, off = slot - pg * page;
+    T* dst = v_cache + ((pg * Hkv + kvh) * (int64_t)D) * page + off;
+    for (int d = lane; d < D; d += 64) dst[(int64_t)d * page] = row[i * row_stride + d];
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_store_kernel(T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ q_w,
@@ -22,7 +58,7 @@ qk_norm_rope_store_kernel(T* __restrict__ qkv, int64_t row_stride, const float* 
                           const float* __restrict__ table,  // [P, D/2, 2] cos,sin or null
                           const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
                           T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq, int Hkv, int D,
-                          int page, int store) {
+                          int page, int store, int64_t num_tokens) {
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -34,12 +70,7 @@ qk_norm_rope_store_kernel(T* __restrict__ qkv, int64_t row_stride, const float* 
   const int half = D >> 1;
 
   if (head >= Hq + Hkv) {  // a value head: copy into the transposed page
-    const int kvh = head - Hq - Hkv;
-    const int slot = slots[t];
-    if (slot < 0) return;
-    const int64_t pg = slot / page, off = slot - pg * page;
-    T* dst = v_cache + ((pg * Hkv + kvh) * (int64_t)D) * page + off;
-    for (int d = lane; d < D; d += 64) dst[(int64_t)d * page] = row[d];
+    store_value_head<T>(row, row_stride, t, num_tokens, slots, v_cache, Hkv, head - Hq - Hkv, D, page, lane);
     return;
   }
 
@@ -93,6 +124,103 @@ qk_norm_rope_store_kernel(T* __restrict__ qkv, int64_t row_stride, const float* 
   }
 }
 
+// ------------------------------------------------------------------ vectorised q/k form
+// The same arithmetic with 4 pairs per lane: LPH = D/8 lanes share a head (a power of two), a wave
+// takes 64/LPH heads, a lane reads x[4l..4l+3] and x[D/2+4l..], their 4 (cos, sin) and writes both
+// quadruples back. blockIdx.y < qk_blocks: q and k heads; the rest: value heads (one per wave).
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Quad<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = static_cast<float>(t[i]);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    bf16x4 t;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = static_cast<bf16_t>(v[i]);
+    *reinterpret_cast<bf16x4*>(p) = t;
+  }
+};
+
+template <typename T, int LPH>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ q_w,
+                              const float* __restrict__ k_w, float eps, const float* __restrict__ table,
+                              const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+                              T* __restrict__ k_cache, T* __restrict__ v_cache, int Hq, int Hkv, int D, int page,
+                              int store, int64_t num_tokens, int qk_blocks) {
+  constexpr int HPW = 64 / LPH;
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int half = D >> 1;
+  if ((int)blockIdx.y >= qk_blocks) {
+    const int kvh = ((int)blockIdx.y - qk_blocks) * 4 + wave;
+    if (kvh < Hkv) store_value_head<T>(qkv + t * row_stride + (int64_t)(Hq + Hkv + kvh) * D, row_stride, t, num_tokens,
+                                       slots, v_cache, Hkv, kvh, D, page, lane);
+    return;
+  }
+  const int head = (blockIdx.y * 4 + wave) * HPW + lane / LPH;
+  const int l = lane % LPH;
+  const bool active = head < Hq + Hkv;
+  const bool is_q = head < Hq;
+  T* row = qkv + t * row_stride + (int64_t)(active ? head : 0) * D;
+  float x1[4], x2[4];
+  Quad<T>::load(row + 4 * l, x1);
+  Quad<T>::load(row + half + 4 * l, x2);
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) ss += x1[i] * x1[i] + x2[i] * x2[i];
+  const float* w = is_q ? q_w : k_w;
+  float inv = 1.f;
+  if (w) {
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, ME_WAVE);
+    inv = rsqrtf(ss / (float)D + eps);
+  }
+  float o1[4], o2[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { o1[i] = x1[i] * inv; o2[i] = x2[i] * inv; }
+  if (w) {
+    float w1[4], w2[4];
+    Quad<float>::load(w + 4 * l, w1);
+    Quad<float>::load(w + half + 4 * l, w2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { o1[i] *= w1[i]; o2[i] *= w2[i]; }
+  }
+  if (table) {
+    const float* cs = table + ((int64_t)positions[t] * half + 4 * l) * 2;   // (cos, sin) of 4 pairs: 8 floats
+    float c0[4], c1[4];
+    Quad<float>::load(cs, c0);
+    Quad<float>::load(cs + 4, c1);
+    const float c[4] = {c0[0], c0[2], c1[0], c1[2]}, sn[4] = {c0[1], c0[3], c1[1], c1[3]};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a = o1[i], b = o2[i];
+      o1[i] = a * c[i] - b * sn[i];
+      o2[i] = b * c[i] + a * sn[i];
+    }
+  }
+  if (!active) return;
+  T* dst = row;
+  if (!is_q && store) {
+    const int slot = slots[t];
+    if (slot < 0) return;
+    const int64_t pg = slot / page, off = slot - pg * page;
+    dst = k_cache + ((pg * Hkv + (head - Hq)) * (int64_t)page + off) * D;
+  }
+  Quad<T>::store(dst + 4 * l, o1);
+  Quad<T>::store(dst + half + 4 * l, o2);
+}
+
 extern "C" int me_qk_norm_rope_store(void* qkv, int dtype, int64_t num_tokens, int64_t row_stride,
                                      const float* q_w, const float* k_w, float eps,
                                      const float* table, int64_t table_positions,
@@ -107,17 +235,43 @@ extern "C" int me_qk_norm_rope_store(void* qkv, int dtype, int64_t num_tokens, i
   ME_CHECK(row_stride >= (int64_t)(Hq + (store ? 2 * Hkv : Hkv)) * D, "qk_norm_rope_store: row stride too small");
   ME_CHECK(!table || table_positions > 0, "qk_norm_rope_store: empty rotary table");
   const int heads = Hq + (store ? 2 * Hkv : Hkv);
+  ME_CHECK(dtype == ME_BF16 || dtype == ME_F32, "qk_norm_rope_store: bad dtype code %d", dtype);
+  // vectorised form: D/8 lanes per head must be a power of two, rows and caches 16-byte aligned
+  const int lph = D / 8;
+  const int esz = dtype == ME_BF16 ? 2 : 4;
+  const bool vec = D % 8 == 0 && lph >= 1 && lph <= 32 && (lph & (lph - 1)) == 0 && (row_stride * esz) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(q_w) % 16 == 0 && reinterpret_cast<uintptr_t>(k_w) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(table) % 16 == 0;
+  if (vec) {
+    const int hpw = 64 / lph;
+    const int qk_blocks = (Hq + Hkv + 4 * hpw - 1) / (4 * hpw);
+    const int v_blocks = store ? (Hkv + 3) / 4 : 0;
+    dim3 grid(num_tokens, qk_blocks + v_blocks), block(256);
+#define LAUNCH(TT, L)                                                                                       \
+  qk_norm_rope_store_vec_kernel<TT, L><<<grid, block, 0, stream>>>((TT*)qkv, row_stride, q_w, k_w, eps, table, \
+                                                                   positions, slots, (TT*)k_cache, (TT*)v_cache, \
+                                                                   Hq, Hkv, D, page, store, num_tokens, qk_blocks)
+#define PICK(TT)                                                                                            \
+  do {                                                                                                      \
+    if (lph == 1) LAUNCH(TT, 1); else if (lph == 2) LAUNCH(TT, 2); else if (lph == 4) LAUNCH(TT, 4);        \
+    else if (lph == 8) LAUNCH(TT, 8); else if (lph == 16) LAUNCH(TT, 16); else LAUNCH(TT, 32);              \
+  } while (0)
+    if (dtype == ME_BF16) PICK(bf16_t); else PICK(float);
+#undef PICK
+#undef LAUNCH
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid(num_tokens, (heads + 3) / 4), block(256);
   if (dtype == ME_BF16)
     qk_norm_rope_store_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (bf16_t*)qkv, row_stride, q_w, k_w, eps, table, positions, slots, (bf16_t*)k_cache,
-        (bf16_t*)v_cache, Hq, Hkv, D, page, store);
-  else if (dtype == ME_F32)
+        (bf16_t*)v_cache, Hq, Hkv, D, page, store, num_tokens);
+  else
     qk_norm_rope_store_kernel<float><<<grid, block, 0, stream>>>(
         (float*)qkv, row_stride, q_w, k_w, eps, table, positions, slots, (float*)k_cache,
-        (float*)v_cache, Hq, Hkv, D, page, store);
-  else
-    ME_CHECK(false, "qk_norm_rope_store: bad dtype code %d", dtype);
+        (float*)v_cache, Hq, Hkv, D, page, store, num_tokens);
   ME_LAUNCH_CHECK();
   return 0;
 }
