@@ -1,0 +1,106 @@
+"""Offline throughput from the command line, in the manner of the reference's bench.py:8-90.
+
+    python -m mini_engine_amd.cli --model DIR [--num-seqs 256] [--chunked 1] [--budget 16384]
+                                  [--threshold 0] [--out results/bench.jsonl] [--label NAME]
+    python -m mini_engine_amd.cli --random-weights 0.6b ...      (no model folder at hand)
+
+Options the reference has keep its names and meanings: --model, --num-seqs, --out, --label,
+--chunked (1 = chunked prefill, 0 = prefill-first), --budget (max_num_batched_tokens),
+--threshold (long_prefill_token_threshold). The workload is the reference's (bench.py:38-48,60-66):
+`random.seed(0)`, prompts of 100-1024 random ids below 10000, max_tokens 100-1024, temperature 0.6,
+ignore_eos, max_num_seqs 256, max_model_len 2048, one warm-up generate; the figure is the sum of
+max_tokens over the wall time. One JSON row is printed and appended to --out.
+Not taken over: --engine (other engines), --attn unified (this engine has one attention path),
+--expect-gpu.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+from datetime import datetime
+from random import randint, seed
+
+
+def main(argv=None) -> int:
+    p = argparse.ArgumentParser(prog="python -m mini_engine_amd.cli", description=__doc__,
+                                formatter_class=argparse.RawDescriptionHelpFormatter)
+    p.add_argument("--model", default=None, help="folder with config.json and *.safetensors")
+    p.add_argument("--random-weights", default=None, metavar="SIZE",
+                   help="write a model folder of this size (tinyA, 0.6b, 8b, 32b) with seeded random weights and use it")
+    p.add_argument("--num-seqs", type=int, default=256)
+    p.add_argument("--out", default="results/bench.jsonl")
+    p.add_argument("--label", default="")
+    p.add_argument("--chunked", type=int, default=1)
+    p.add_argument("--budget", type=int, default=16384)
+    p.add_argument("--threshold", type=int, default=0)
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    p.add_argument("--seed", type=int, default=0, help="seed of the sampler's noise and of random weights")
+    p.add_argument("--max-model-len", type=int, default=2048)
+    p.add_argument("--max-num-seqs", type=int, default=256)
+    p.add_argument("--block-size", type=int, default=16, help="kvcache_block_size")
+    p.add_argument("--policy", default="fcfs", choices=["fcfs", "priority"])
+    p.add_argument("--max-prompt", type=int, default=1024)
+    p.add_argument("--max-output", type=int, default=1024)
+    args = p.parse_args(argv)
+    if (args.model is None) == (args.random_weights is None):
+        p.error("give exactly one of --model and --random-weights")
+
+    import torch
+    from . import LLM, SamplingParams
+
+    tmp = None
+    path = args.model
+    if args.random_weights:
+        sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+        from bench import SIZES, model_config          # the sizes the repository's benchmark names
+        from .weights.random_init import write_random_model
+        if args.random_weights not in SIZES:
+            p.error(f"--random-weights must be one of {sorted(SIZES)}")
+        tmp = tempfile.TemporaryDirectory()
+        cfg, _ = model_config(args.random_weights, None)
+        path = write_random_model(cfg, args.seed, tmp.name)
+    path = os.path.expanduser(path)
+
+    seed(0)
+    N = args.num_seqs
+    vocab_cap = 10000
+    prompt_token_ids = [[randint(0, vocab_cap) for _ in range(randint(min(100, args.max_prompt), args.max_prompt))] for _ in range(N)]
+    max_tokens = [randint(min(100, args.max_output), args.max_output) for _ in range(N)]
+
+    llm = LLM(path, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len, max_num_batched_tokens=args.budget,
+              enable_chunked_prefill=bool(args.chunked), long_prefill_token_threshold=args.threshold, dtype=args.dtype,
+              seed=args.seed, kvcache_block_size=args.block_size, scheduling_policy=args.policy)
+    vocab = llm.model.embedding.vocab_size
+    if vocab <= vocab_cap:
+        prompt_token_ids = [[t % vocab for t in ids] for ids in prompt_token_ids]
+    sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
+
+    llm.generate([[1, 2, 3]], SamplingParams(max_tokens=4), use_tqdm=False)      # warm-up
+    t = time.time()
+    llm.generate(prompt_token_ids, sps, use_tqdm=False)
+    t = time.time() - t
+
+    total = sum(max_tokens)
+    row = {
+        "engine": "mini_engine_amd", "label": args.label, "gpu": torch.cuda.get_device_name(0), "torch": torch.__version__,
+        "model": args.random_weights or path, "dtype": args.dtype, "num_seqs": N,
+        "input_tokens": sum(len(x) for x in prompt_token_ids), "output_tokens": total, "time_s": round(t, 2),
+        "throughput_tok_s": round(total / t, 1), "chunked": bool(args.chunked), "budget": args.budget,
+        "threshold": args.threshold, "preemptions": llm.scheduler.num_preemptions,
+        "kv_blocks": llm.config.num_kvcache_blocks, "time": datetime.now().isoformat(timespec="seconds"),
+    }
+    print(json.dumps(row))
+    os.makedirs(os.path.dirname(args.out) or ".", exist_ok=True)
+    with open(args.out, "a") as f:
+        f.write(json.dumps(row) + "\n")
+    if tmp is not None:
+        tmp.cleanup()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
