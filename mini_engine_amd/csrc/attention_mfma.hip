@@ -34,6 +34,10 @@ constexpr int HD = ME_HEAD_DIM;
 constexpr int KS = (HD + 31) / 32;  // 32-channel steps of the score product
 constexpr int DT = HD / 16;         // 16-channel tiles of the output
 constexpr float NEG = -1e30f;       // "no key yet": finite, so that differences never give NaN
+// log2 units by which the max must rise before the accumulators are rescaled. 0: follow the max exactly.
+// (A step of 8 rescales far less often but measured slower on MI355X, 97 us against 86 us for a 2,048-token
+// prefill at 16x128 heads, so it stays off.)
+constexpr float RESCALE_STEP = 0.f;
 
 struct AttnArgs {
   const bf16_t* q;
@@ -102,10 +106,16 @@ __device__ __forceinline__ int page_index(int tok, int page, int shift) {
 // in flight together; callers fetch the next block while they compute on the current one.
 // lo_min: a bound below which pages may already have been given back (never loaded).
 // -------------------------------------------------------------------------------------
-struct KVBlock {
+struct KVBlock {   // the keys of a block: fetched one block ahead of their use
   bf16x8 k[2][KS];
-  bf16x8 v[DT];
   bool kok[2];
+  // where the block's values are (looked up with the keys' pages, fetched when the block is used:
+  // they are needed only after the scores and the softmax, which cover their latency)
+  int vpage, voff;
+  bool vgrp_ok;
+};
+struct VBlock {
+  bf16x8 v[DT];
   uint32_t vmask[4];  // per 32-bit pair of this lane's 8 keys: which halves lie before L in a held page
 };
 
@@ -150,18 +160,22 @@ __device__ __forceinline__ void load_kv(const AttnArgs& a, const BlockPages& pg,
       blk.k[tt][ks] = ld8(kp + ((HD % 32 == 0 || d0 < HD) ? d0 : 0));
     }
   }
-  // V^T rows: channel 16*dt + n, keys t0 + 8g .. t0 + 8g + 7
-  const bool vgrp_ok = pg.vgrp_ok && pg.vpage >= 0;
-  const int vpage = vgrp_ok ? pg.vpage : 0;
-  const int voff = vgrp_ok ? pg.voff : 0;
-  const bf16_t* vp = a.v_cache + (((int64_t)vpage * a.Hkv + kvh) * HD + n) * a.page + voff;
+  blk.vgrp_ok = pg.vgrp_ok && pg.vpage >= 0;
+  blk.vpage = blk.vgrp_ok ? pg.vpage : 0;
+  blk.voff = blk.vgrp_ok ? pg.voff : 0;
+}
+
+// V^T rows: channel 16*dt + n, keys t0 + 8g .. t0 + 8g + 7
+__device__ __forceinline__ void load_v(const AttnArgs& a, const KVBlock& blk, int kvh, int t0, int L, int n, int g,
+                                       VBlock& vb) {
+  const bf16_t* vp = a.v_cache + (((int64_t)blk.vpage * a.Hkv + kvh) * HD + n) * a.page + blk.voff;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) blk.v[dt] = ld8(vp + (int64_t)dt * 16 * a.page);
+  for (int dt = 0; dt < DT; ++dt) vb.v[dt] = ld8(vp + (int64_t)dt * 16 * a.page);
   // keys at or past L hold foreign or unwritten data (possibly NaN): their bits are cleared
-  const int nv = vgrp_ok ? L - (t0 + 8 * g) : 0;
+  const int nv = blk.vgrp_ok ? L - (t0 + 8 * g) : 0;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
-    blk.vmask[j] = (2 * j < nv ? 0x0000ffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
+    vb.vmask[j] = (2 * j < nv ? 0x0000ffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
 }
 
 __device__ __forceinline__ void load_block(const AttnArgs& a, const int32_t* __restrict__ bt, int kvh, int t0,
@@ -180,7 +194,7 @@ __device__ __forceinline__ void load_block(const AttnArgs& a, const int32_t* __r
 //   replaced, K rows and V keys that must not be read are zeroed.
 //   The accumulators are rescaled only when some column's max has risen (a wave-wide test).
 template <bool FULL>
-__device__ __forceinline__ void attend_block(const AttnArgs& a, const KVBlock& blk, int t0,
+__device__ __forceinline__ void attend_block(const AttnArgs& a, const KVBlock& blk, const VBlock& vblk, int t0,
                                              const bf16x8 (&qb)[KS], int col_lo, int col_hi, float& m, float& l,
                                              f32x4 (&acc)[DT], int g) {
   const bf16x8 z = zero8();
@@ -210,18 +224,15 @@ __device__ __forceinline__ void attend_block(const AttnArgs& a, const KVBlock& b
     bm = fmaxf(bm, sv[i]);
   }
   bm = max_over_groups(bm);
-  const float m_new = fmaxf(m, bm > 0.5f * NEG ? bm * c : NEG);
-  const bool rose = m_new > m;
-  float psum = 0.f;
-  bf16x8 pb;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    float p = __builtin_amdgcn_exp2f(fmaf(sv[i], c, -m_new));
-    if (!FULL) p = sv[i] > 0.5f * NEG ? p : 0.f;
-    psum += p;
-    pb[i] = static_cast<bf16_t>(p);
-  }
+  // The reference point m of the exponentials follows the running max lazily: it moves only when
+  // the max has risen by more than RESCALE_STEP (in log2 units), so probabilities may reach
+  // 2^RESCALE_STEP instead of 1 (harmless in float32 sums and in bfloat16, whose precision is
+  // relative) and the accumulators are rescaled rarely. Sums and outputs share the same m, so the
+  // result is the same softmax.
+  const float m_blk = bm > 0.5f * NEG ? bm * c : NEG;
+  const bool rose = m_blk > m + RESCALE_STEP;
   if (__any(rose)) {
+    const float m_new = rose ? m_blk : m;
     const float alpha = __builtin_amdgcn_exp2f(m - m_new);
     l *= alpha;
 #pragma unroll
@@ -230,14 +241,23 @@ __device__ __forceinline__ void attend_block(const AttnArgs& a, const KVBlock& b
     }
     m = m_new;
   }
+  float psum = 0.f;
+  bf16x8 pb;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float p = __builtin_amdgcn_exp2f(fmaf(sv[i], c, -m));
+    if (!FULL) p = sv[i] > 0.5f * NEG ? p : 0.f;
+    psum += p;
+    pb[i] = static_cast<bf16_t>(p);
+  }
   l += psum;  // this lane's share of the column's sum; the 4 shares are added at the end
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
-    bf16x8 va = blk.v[dt];
+    bf16x8 va = vblk.v[dt];
     if (!FULL) {
       typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
       u32x4 vb = __builtin_bit_cast(u32x4, va);
-      vb[0] &= blk.vmask[0]; vb[1] &= blk.vmask[1]; vb[2] &= blk.vmask[2]; vb[3] &= blk.vmask[3];
+      vb[0] &= vblk.vmask[0]; vb[1] &= vblk.vmask[1]; vb[2] &= vblk.vmask[2]; vb[3] &= vblk.vmask[3];
       va = __builtin_bit_cast(bf16x8, vb);
     }
     acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, acc[dt], 0, 0, 0);
@@ -264,8 +284,8 @@ __device__ __forceinline__ float column_sum(float l) { return sum_over_groups(l)
 // Grid: (floor(T / tok_tile) + num_seqs, Hkv). The first tile of sequence b is
 // floor(cu[b] / tok_tile) + b, an upper bound of the tiles before it; surplus tiles exit.
 // =====================================================================================
-template <int CT>
-__global__ void __launch_bounds__(256, CT == 1 ? 2 : 1) attn_prefill_kernel(AttnArgs a) {
+template <int CT, bool PIPE>
+__global__ void __launch_bounds__(256, PIPE ? 1 : 2) attn_prefill_kernel(AttnArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int kvh = blockIdx.y;
@@ -326,32 +346,52 @@ __global__ void __launch_bounds__(256, CT == 1 ? 2 : 1) attn_prefill_kernel(Attn
     // above the last column's window start) takes the path without masks
     const int full_hi = pos_first - 31;                                   // t0 <= full_hi: all 32 keys visible
     const int full_lo = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;  // t0 >= full_lo: none behind a window
-#define ATTEND(BLK)                                                                                          \
+#define ATTEND(BLK, vb_)                                                                                     \
   do {                                                                                                       \
     if (t0 <= full_hi && t0 >= full_lo) {                                                                    \
       _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                      \
-          attend_block<true>(a, BLK, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);          \
+          attend_block<true>(a, BLK, vb_, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);     \
     } else {                                                                                                 \
       _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                      \
-          attend_block<false>(a, BLK, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);         \
+          attend_block<false>(a, BLK, vb_, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);    \
     }                                                                                                        \
   } while (0)
-    KVBlock A, B;
-    BlockPages pn;
     int t0 = w_lo & ~31;
-    load_block(a, bt, kvh, t0, L, tile_lo, n, g, A);
-    lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
-    while (true) {
-      load_kv(a, pn, kvh, t0 + 32, L, n, g, B);
-      lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
-      ATTEND(A);
-      t0 += 32;
-      if (t0 > pos_last) break;
-      load_kv(a, pn, kvh, t0 + 32, L, n, g, A);
-      lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
-      ATTEND(B);
-      t0 += 32;
-      if (t0 > pos_last) break;
+    if (PIPE) {
+      KVBlock A, B;
+      VBlock VA, VB;
+      BlockPages pn;
+      load_block(a, bt, kvh, t0, L, tile_lo, n, g, A);
+      load_v(a, A, kvh, t0, L, n, g, VA);
+      lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
+      while (true) {
+        load_kv(a, pn, kvh, t0 + 32, L, n, g, B);
+        load_v(a, B, kvh, t0 + 32, L, n, g, VB);
+        lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
+        ATTEND(A, VA);
+        t0 += 32;
+        if (t0 > pos_last) break;
+        load_kv(a, pn, kvh, t0 + 32, L, n, g, A);
+        load_v(a, A, kvh, t0 + 32, L, n, g, VA);
+        lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
+        ATTEND(B, VB);
+        t0 += 32;
+        if (t0 > pos_last) break;
+      }
+    } else {
+      // one block buffer, two waves per SIMD: the other wave's work covers this wave's loads
+      KVBlock A;
+      VBlock VA;
+      BlockPages pn;
+      lookup_pages(a, bt, t0, L, tile_lo, n, g, pn);
+      while (true) {
+        load_kv(a, pn, kvh, t0, L, n, g, A);
+        load_v(a, A, kvh, t0, L, n, g, VA);
+        lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
+        ATTEND(A, VA);
+        t0 += 32;
+        if (t0 > pos_last) break;
+      }
     }
 #undef ATTEND
 #pragma unroll
@@ -411,8 +451,10 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     load_q(a.q + t * a.q_stride + (int64_t)head * HD, valid, g, qb);
     const int col_hi = valid ? pos : -1;
     while (true) {
-      if (t0 + 32 <= L && t0 >= lo) attend_block<true>(a, A, t0, qb, lo, col_hi, m, l, acc, g);
-      else attend_block<false>(a, A, t0, qb, lo, col_hi, m, l, acc, g);
+      VBlock vb;
+      load_v(a, A, kvh, t0, L, n, g, vb);
+      if (t0 + 32 <= L && t0 >= lo) attend_block<true>(a, A, vb, t0, qb, lo, col_hi, m, l, acc, g);
+      else attend_block<false>(a, A, vb, t0, qb, lo, col_hi, m, l, acc, g);
       t0 += 128;
       if (t0 >= p_hi) break;
       load_block(a, bt, kvh, t0, L, lo, n, g, A);
@@ -526,14 +568,18 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                   num_seqs, Hq, Hkv, page, scale, window)) return -1;
   a.cu_seqlens = cu_seqlens;
   // column tiles per wave: 2 when the step has enough tokens to fill the GPU with the larger tiles
-  const int ct = (col_tiles_per_wave == 1 || col_tiles_per_wave == 2) ? col_tiles_per_wave
+  const int ctw = col_tiles_per_wave & 15;
+  const int ct = (ctw == 1 || ctw == 2) ? ctw
                  : ((num_tokens * Hq >= 32768 && HD <= 128) ? 2 : 1);
   const int cols = 64 * ct;
   a.tok_tile = a.G >= cols ? 1 : cols / a.G;
   const int64_t tiles = num_tokens / a.tok_tile + num_seqs;
   ME_CHECK(tiles < (1ll << 31), "attention: too many tiles");
-  if (ct == 2) attn_prefill_kernel<2><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
-  else attn_prefill_kernel<1><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  const bool pipe = col_tiles_per_wave < 16;   // +16: the single-buffer, two-waves-per-SIMD variant (tuning)
+  if (ct == 2 && pipe) attn_prefill_kernel<2, true><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  else if (ct == 2) attn_prefill_kernel<2, false><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  else if (pipe) attn_prefill_kernel<1, true><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  else attn_prefill_kernel<1, false><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
   ME_LAUNCH_CHECK();
   return 0;
 }

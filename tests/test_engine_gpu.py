@@ -165,3 +165,32 @@ def test_decode_graphs_replay_like_eager_steps(folders, dtype, name):
         got = d.result(r)
         err = helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]]))
         assert err <= tol, f"{name} {r}: {err:.3g}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_real_layer_sizes(tmp_path_factory, dtype):
+    """Qwen3-0.6B's layer sizes (hidden 1024, 16 query / 8 key heads of 128, intermediate 3072, page 16)
+    with 2 layers and a vocabulary that is no power of two: a long prompt in portions, then decoding,
+    beside a second request, against the plain implementation."""
+    from mini_engine_amd.config.model_config import Qwen3Config
+    from mini_engine_amd.weights.random_init import write_random_model
+    cfgd = dict(architectures=["Qwen3ForCausalLM"], vocab_size=20011, hidden_size=1024, intermediate_size=3072,
+                num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
+                rope_theta=1e6, tie_word_embeddings=True, max_position_embeddings=4096)
+    folder = write_random_model(Qwen3Config.from_dict(cfgd), 3, str(tmp_path_factory.mktemp("real")))
+    model = load_model(folder, "cuda", dtype, 1024)
+    manager = CacheManager(64, 16, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, dtype, "cuda", 1024, poison_cache=True, use_graphs=True)
+    a, b = helpers.random_ids(300, 20011, 1), helpers.random_ids(70, 20011, 2)
+    d = helpers.Driver(runner, manager)
+    d.step({"a": a[:200]})
+    d.step({"a": a[200:263], "b": b[:64]})
+    d.step({"a": a[263:290], "b": b[64:65]})
+    for t in range(5):
+        d.step({"a": a[290 + t:291 + t], "b": b[65 + t:66 + t]})
+    d.step({"a": a[295:]})
+    tol = helpers.TOL_F32 if dtype == torch.float32 else helpers.TOL_BF16
+    for ids, r in ((a, "a"), (b, "b")):
+        got = d.result(r)
+        err = helpers.rel_err(got, helpers.plain_logits(folder, ids)[: got.shape[0]])
+        assert err <= tol, f"{r}: {err:.3g}"
