@@ -64,7 +64,7 @@ def prefill_flops(cfg, T: int) -> float:
 
 class Bench:
     def __init__(self, cfg, dtype: str, page: int, max_batch: int, context: int, gen: int, seed: int = 0,
-                 graphs: bool = True):
+                 graphs: bool = True, min_pages: int = 0, max_len: int = 0):
         import torch
         from mini_engine_amd.cache.manager import CacheManager
         from mini_engine_amd.engine.runner import ModelRunner
@@ -74,11 +74,11 @@ class Bench:
         self.torch = torch
         self.cfg, self.page, self.context, self.gen = cfg, page, context, gen
         self.dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
-        self.max_len = context + gen + 64
+        self.max_len = max(context + gen + 64, max_len)
         t0 = time.time()
         self.model = fill_random(build_model(cfg), seed, "cuda", self.dtype, self.max_len)
         print(f"[bench] random weights ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
-        pages = max_batch * -(-self.max_len // page)
+        pages = max(max_batch * -(-self.max_len // page), min_pages)
         self.manager = CacheManager(pages, page, ModelRunner.windows_of(self.model), enable_prefix_caching=False)
         self.runner = ModelRunner(self.model, self.manager, self.dtype, "cuda", self.max_len, use_graphs=graphs)
         self.gen_ids = torch.Generator().manual_seed(seed)
@@ -141,6 +141,33 @@ class Bench:
         return dt / steps, ctx_mid
 
 
+    def offline(self, num_seqs: int, budget: int = 16384, max_model_len: int = 2048):
+        """The reference's offline workload (its bench.py:38-48,60-66): `random.seed(0)`, prompts of 100-1024
+        random ids below 10000, max_tokens 100-1024, temperature 0.6, ignore_eos, max_num_seqs 256,
+        max_model_len 2048, chunked prefill under a 16k budget. Returns (sum of max_tokens / seconds, record)."""
+        from random import randint, seed
+        from types import SimpleNamespace
+        from mini_engine_amd.engine.llm_engine import LLMEngine
+        from mini_engine_amd.sampling.sampling_params import SamplingParams
+        seed(0)
+        prompts = [[randint(0, 10000) % self.cfg.vocab_size for _ in range(randint(100, 1024))] for _ in range(num_seqs)]
+        max_tokens = [randint(100, 1024) for _ in range(num_seqs)]
+        conf = SimpleNamespace(max_num_seqs=256, max_num_batched_tokens=budget, long_prefill_token_threshold=0,
+                               enable_chunked_prefill=True, scheduling_policy="fcfs", eos=-1, max_model_len=max_model_len,
+                               seed=0)
+        llm = LLMEngine.from_parts(conf, self.model, self.manager, self.runner)
+        sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
+        llm.generate([[1, 2, 3]], SamplingParams(max_tokens=4), use_tqdm=False)
+        self.torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        llm.generate(prompts, sps, use_tqdm=False)
+        dt = time.perf_counter() - t0
+        total = sum(max_tokens)
+        return total / dt, {"value": round(total / dt, 1), "unit": "output tokens/s", "seconds": round(dt, 2),
+                            "requests": num_seqs, "input_tokens": sum(len(p) for p in prompts), "output_tokens": total,
+                            "preemptions": llm.scheduler.num_preemptions, "reference_a100_tok_s": 4205.0}
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -156,6 +183,8 @@ def main(argv=None) -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="extra decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--offline", type=int, default=256,
+                    help="also run the reference's offline workload with this many requests (0: skip)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     args = ap.parse_args(argv)
     if args.gpus != 1:
@@ -167,7 +196,9 @@ def main(argv=None) -> int:
     import torch
     cfg, full_layers = model_config(args.model_size, args.layers)
     points = [int(p) for p in args.points.split(",") if p]
-    bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed, graphs=not args.no_graphs)
+    off_pages = args.offline * -(-2048 // args.page) if args.offline else 0
+    bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed,
+                  graphs=not args.no_graphs, min_pages=off_pages, max_len=2048 if args.offline else 0)
     item = 2 if args.dtype == "bfloat16" else 4
 
     T = args.prefill_tokens
@@ -187,6 +218,11 @@ def main(argv=None) -> int:
         pts[f"decode_b{b}"] = round(b / s, 1)
         print(f"[bench] decode batch {b}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
 
+    offline = None
+    if args.offline:
+        _, offline = bench.offline(args.offline)
+        print(f"[bench] reference offline workload: {offline['value']} output tokens/s", file=sys.stderr, flush=True)
+
     line = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens; % roofline",
         "value": round(args.batch / step_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
@@ -201,6 +237,8 @@ def main(argv=None) -> int:
                    "hip_graphs": not args.no_graphs},
         "prefill": prefill, "roofline": roofline, "points": pts,
     }
+    if offline is not None:
+        line["offline"] = offline
     print(json.dumps(line), flush=True)
     return 0
 

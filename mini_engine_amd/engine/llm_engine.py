@@ -55,6 +55,17 @@ class LLMEngine:
         self.scheduler = Scheduler(config, self.manager)
         self.sampler = Sampler(self.runner, config.seed)
 
+    @classmethod
+    def from_parts(cls, config, model, manager, runner, tokenizer=None):
+        """An engine around an already loaded model and its runner (benchmarks that build random
+        weights in memory). `config` needs the scheduler's fields and `seed`."""
+        self = cls.__new__(cls)
+        self.config, self.model, self.manager, self.runner = config, model, manager, runner
+        self.device, self.dtype, self.tokenizer = runner.device, runner.dtype, tokenizer
+        self.scheduler = Scheduler(config, manager)
+        self.sampler = Sampler(runner, config.seed)
+        return self
+
     def _size_pool(self, plan) -> int:
         """Pages per group from the memory that is free now (reference engine/model_runner.py:69-80
         sizes from a measured warm-up peak; here the step's working set is estimated instead)."""
