@@ -6,7 +6,7 @@
 //    (no matrix-core, no reduced precision). Each output element is one thread's sequential sum
 //    over K, so a row's result does not depend on the other rows of the batch. This is the
 //    float32 path and the fallback for bf16 shapes the MFMA kernel refuses.
-//  * me_gemm_skinny_bf16: the decode product, M small. Pure weight streaming: each workgroup
+//  * me_gemm_skinny_bf16: the decode product, M <= 16 (up to 32 rows when K is split over workgroups). Pure weight streaming: each workgroup
 //    owns 16 output features, its 4 waves split K, every lane reads 64 contiguous bytes of a
 //    weight row per step (whole cache lines per row and wave), products on
 //    v_mfma_f32_16x16x32_bf16 with the tokens as the 16-wide B operand, waves merged through
@@ -200,121 +200,6 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
       else y[(int64_t)m * ldy + n] = from_f32<TO>(v);
     }
   }
-}
-
-// ------------------------------------------------------------------ wide bf16 product on MFMA
-// Many output features (the head over a vocabulary) or more than 16 rows: each wave owns NT tiles
-// of 16 features over the whole K, streams their weight rows once, and multiplies them with all
-// 16*MT rows of x; no split of K, so no LDS and no barrier. A workgroup's 4 waves read the same x.
-// Grid (ceil(N / (64*NT)), ceil(M / (16*MT))).
-template <int MT, int NT, typename TO>
-__global__ void __launch_bounds__(256)
-gemm_wide_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
-                 TO* __restrict__ y, int64_t ldy, int M, int N, int K) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = (blockIdx.x * 4 + wave) * 16 * NT, m0 = blockIdx.y * 16 * MT;
-  if (n0 >= N) return;
-  const bf16_t* wrow[NT];
-  bool wrow_ok[NT];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    const int n = n0 + 16 * nt + r;
-    wrow_ok[nt] = n < N;
-    wrow[nt] = w + (int64_t)(wrow_ok[nt] ? n : 0) * ldw;
-  }
-  const bf16_t* xrow[MT];
-  bool xrow_ok[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = m0 + 16 * mt + r;
-    xrow_ok[mt] = m < M;
-    xrow[mt] = x + (int64_t)(xrow_ok[mt] ? m : 0) * ldx;
-  }
-  f32x4 acc[NT][MT];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 z = gz8();
-  struct Ops { bf16x8 a[NT][4]; bf16x8 b[MT][4]; };
-  auto fetch = [&](int s, Ops& op) {
-    const int kb = 128 * s + 32 * g;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int k = kb + 8 * j;
-      const int ks = k < K ? k : 0;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) op.a[nt][j] = *reinterpret_cast<const bf16x8*>(wrow[nt] + ks);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) op.b[mt][j] = *reinterpret_cast<const bf16x8*>(xrow[mt] + ks);
-    }
-  };
-  auto product = [&](int s, const Ops& op) {
-    const int kb = 128 * s + 32 * g;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bool kok = kb + 8 * j < K;
-      bf16x8 b[MT];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) b[mt] = (xrow_ok[mt] && kok) ? op.b[mt][j] : z;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const bf16x8 a = (wrow_ok[nt] && kok) ? op.a[nt][j] : z;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[mt], acc[nt][mt], 0, 0, 0);
-      }
-    }
-  };
-  const int steps = (K + 127) / 128;
-  Ops A, B;
-  int s = 0;
-  fetch(0, A);
-  while (true) {
-    fetch(s + 1 < steps ? s + 1 : s, B);
-    product(s, A);
-    if (++s >= steps) break;
-    fetch(s + 1 < steps ? s + 1 : s, A);
-    product(s, B);
-    if (++s >= steps) break;
-  }
-  // accumulator: lane (token r, g) holds features 16*nt + 4g + i of its tile
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = m0 + 16 * mt + r;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + 16 * nt + 4 * g + i;
-        if (m < M && n < N) y[(int64_t)m * ldy + n] = from_f32<TO>(acc[nt][mt][i]);
-      }
-    }
-}
-
-extern "C" int me_gemm_wide_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
-                                 int out_dtype, int M, int N, int K, hipStream_t stream) {
-  if (M == 0 || N == 0) return 0;
-  ME_CHECK(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
-           "wide gemm: K=%d and the row strides must be multiples of 8", K);
-  ME_CHECK((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0),
-           "wide gemm: operands must be 16-byte aligned");
-  const int mt = M > 32 ? 4 : (M > 16 ? 2 : 1);
-  const int nt = mt == 4 ? 2 : 1;      // more features per wave where x is large: x is then read half as often
-  dim3 grid((N + 64 * nt - 1) / (64 * nt), (M + 16 * mt - 1) / (16 * mt)), block(256);
-  ME_CHECK(grid.y <= 65535, "wide gemm: too many rows (%d)", M);
-#define LAUNCH(MTV, NTV, TO) \
-  gemm_wide_kernel<MTV, NTV, TO><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, ldy, M, N, K)
-  if (out_dtype == ME_F32) {
-    if (mt == 4) LAUNCH(4, 2, float); else if (mt == 2) LAUNCH(2, 1, float); else LAUNCH(1, 1, float);
-  } else if (out_dtype == ME_BF16) {
-    if (mt == 4) LAUNCH(4, 2, bf16_t); else if (mt == 2) LAUNCH(2, 1, bf16_t); else LAUNCH(1, 1, bf16_t);
-  } else {
-    ME_CHECK(false, "wide gemm: bad output dtype code %d", out_dtype);
-  }
-#undef LAUNCH
-  ME_LAUNCH_CHECK();
-  return 0;
 }
 
 // y: bf16 or float32 [M, N]; or, when ksplit > 1, `partials` float32 [ksplit, M, N] (y unused).

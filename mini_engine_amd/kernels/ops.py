@@ -62,7 +62,6 @@ _CORE_PROTOS = {
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
-    "me_gemm_wide_bf16": [P, L, P, L, P, L, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
@@ -269,10 +268,10 @@ class HipBackend:
                allow_partials: bool = False):
         """x [M, K] . w[N, K]^T (reference layers/linear.py:25-26: F.linear, no bias).
 
-        float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for M <= 64 or float32 output,
-        the library product (hipBLASLt through torch) above that, the FMA kernel for shapes the
-        MFMA kernel refuses. With allow_partials a skinny product with few output features may
-        split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
+        float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 16 rows (32 when K is
+        split), the library product (hipBLASLt through torch) above that and for the head over a
+        large vocabulary, the FMA kernel for shapes the MFMA kernel refuses. With allow_partials a
+        skinny product with few output features may split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
         adds them."""
         _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: {tuple(x.shape)} x {tuple(w.shape)}^T")
         _check(x.dtype == w.dtype, f"linear: activation {x.dtype} and weight {w.dtype} differ")
@@ -293,23 +292,21 @@ class HipBackend:
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
             return y
-        if (M <= SKINNY_MAX_M or out_dtype == torch.float32) and N >= WIDE_MIN_N:
-            # a very wide output (the head over the vocabulary): one wave per feature tile, whole K
-            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
-            core().call("me_gemm_wide_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
-                        _code(out_dtype), M, N, K, _stream())
-            return y
-        if M <= SKINNY_MAX_M or out_dtype == torch.float32:
-            ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= SKINNY_MAX_M) else 1
-            if ksplit > 1:
-                parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
-                core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
-                            ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, _stream())
-                return parts
+        ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype) else 1
+        if ksplit > 1:
+            parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
+            core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
+                        ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, _stream())
+            return parts
+        if M <= SKINNY_MAX_M and N < LIBRARY_MIN_N:
             y = torch.empty((M, N), dtype=out_dtype, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), None, 1, M, N, K, 0, _stream())
             return y
+        # many rows, or the head over a large vocabulary: the library product (float32 accumulation; the
+        # float32 output form keeps the logits unrounded)
+        if out_dtype == torch.float32:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
         return torch.matmul(x, w.t())
 
     def silu_mul_linear(self, gu: torch.Tensor, w: torch.Tensor, allow_partials: bool = False):
@@ -325,7 +322,7 @@ class HipBackend:
         if not fused:
             return self.linear(self.silu_and_mul(gu), w, None, allow_partials)
         N = w.shape[0]
-        ksplit = choose_ksplit(M, N, inter) if allow_partials else 1
+        ksplit = choose_ksplit(M, N, inter) if allow_partials else 1      # fused only for M <= GATED_MAX_M <= PARTIALS_MAX_M
         if ksplit > 1:
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=gu.device)
             core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), None, N,
@@ -353,8 +350,9 @@ class HipBackend:
         return out
 
 
-SKINNY_MAX_M = 64
-WIDE_MIN_N = 32768
+SKINNY_MAX_M = 16        # rows up to which the skinny MFMA kernel beats the library product (measured)
+PARTIALS_MAX_M = 32      # rows up to which a product split over K (float32 partial sums) does
+LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go to the library at any M
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 GATED_MAX_M = 16
 _TARGET_WORKGROUPS = 512
