@@ -284,8 +284,8 @@ __device__ __forceinline__ float column_sum(float l) { return sum_over_groups(l)
 // Grid: (floor(T / tok_tile) + num_seqs, Hkv). The first tile of sequence b is
 // floor(cu[b] / tok_tile) + b, an upper bound of the tiles before it; surplus tiles exit.
 // =====================================================================================
-template <int CT, bool PIPE>
-__global__ void __launch_bounds__(256, PIPE ? 1 : 2) attn_prefill_kernel(AttnArgs a) {
+template <int CT>
+__global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int kvh = blockIdx.y;
@@ -339,9 +339,6 @@ __global__ void __launch_bounds__(256, PIPE ? 1 : 2) attn_prefill_kernel(AttnArg
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    // pipeline: page ids two blocks ahead, keys and values one block ahead of the products. The
-    // fetches are unconditional, also past the last block (they then read page 0 and are not used):
-    // a fetch behind a branch would make the waits of both paths merge into waits on the newest loads.
     // a block all of whose keys every column of this wave sees (below the first column's position,
     // above the last column's window start) takes the path without masks
     const int full_hi = pos_first - 31;                                   // t0 <= full_hi: all 32 keys visible
@@ -356,42 +353,29 @@ __global__ void __launch_bounds__(256, PIPE ? 1 : 2) attn_prefill_kernel(AttnArg
           attend_block<false>(a, BLK, vb_, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);    \
     }                                                                                                        \
   } while (0)
+    // pipeline: page ids two blocks ahead, keys and values one block ahead of the products. The
+    // fetches are unconditional, also past the last block (they then read page 0 and are not used):
+    // a fetch behind a branch would make the waits of both paths merge into waits on the newest loads.
     int t0 = w_lo & ~31;
-    if (PIPE) {
-      KVBlock A, B;
-      VBlock VA, VB;
-      BlockPages pn;
-      load_block(a, bt, kvh, t0, L, tile_lo, n, g, A);
-      load_v(a, A, kvh, t0, L, n, g, VA);
-      lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
-      while (true) {
-        load_kv(a, pn, kvh, t0 + 32, L, n, g, B);
-        load_v(a, B, kvh, t0 + 32, L, n, g, VB);
-        lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
-        ATTEND(A, VA);
-        t0 += 32;
-        if (t0 > pos_last) break;
-        load_kv(a, pn, kvh, t0 + 32, L, n, g, A);
-        load_v(a, A, kvh, t0 + 32, L, n, g, VA);
-        lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
-        ATTEND(B, VB);
-        t0 += 32;
-        if (t0 > pos_last) break;
-      }
-    } else {
-      // one block buffer, two waves per SIMD: the other wave's work covers this wave's loads
-      KVBlock A;
-      VBlock VA;
-      BlockPages pn;
-      lookup_pages(a, bt, t0, L, tile_lo, n, g, pn);
-      while (true) {
-        load_kv(a, pn, kvh, t0, L, n, g, A);
-        load_v(a, A, kvh, t0, L, n, g, VA);
-        lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
-        ATTEND(A, VA);
-        t0 += 32;
-        if (t0 > pos_last) break;
-      }
+    KVBlock A, B;
+    VBlock VA, VB;
+    BlockPages pn;
+    load_block(a, bt, kvh, t0, L, tile_lo, n, g, A);
+    load_v(a, A, kvh, t0, L, n, g, VA);
+    lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
+    while (true) {
+      load_kv(a, pn, kvh, t0 + 32, L, n, g, B);
+      load_v(a, B, kvh, t0 + 32, L, n, g, VB);
+      lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
+      ATTEND(A, VA);
+      t0 += 32;
+      if (t0 > pos_last) break;
+      load_kv(a, pn, kvh, t0 + 32, L, n, g, A);
+      load_v(a, A, kvh, t0 + 32, L, n, g, VA);
+      lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
+      ATTEND(B, VB);
+      t0 += 32;
+      if (t0 > pos_last) break;
     }
 #undef ATTEND
 #pragma unroll
@@ -568,18 +552,14 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                   num_seqs, Hq, Hkv, page, scale, window)) return -1;
   a.cu_seqlens = cu_seqlens;
   // column tiles per wave: 2 when the step has enough tokens to fill the GPU with the larger tiles
-  const int ctw = col_tiles_per_wave & 15;
-  const int ct = (ctw == 1 || ctw == 2) ? ctw
+  const int ct = (col_tiles_per_wave == 1 || col_tiles_per_wave == 2) ? col_tiles_per_wave
                  : ((num_tokens * Hq >= 32768 && HD <= 128) ? 2 : 1);
   const int cols = 64 * ct;
   a.tok_tile = a.G >= cols ? 1 : cols / a.G;
   const int64_t tiles = num_tokens / a.tok_tile + num_seqs;
   ME_CHECK(tiles < (1ll << 31), "attention: too many tiles");
-  const bool pipe = col_tiles_per_wave < 16;   // +16: the single-buffer, two-waves-per-SIMD variant (tuning)
-  if (ct == 2 && pipe) attn_prefill_kernel<2, true><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
-  else if (ct == 2) attn_prefill_kernel<2, false><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
-  else if (pipe) attn_prefill_kernel<1, true><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
-  else attn_prefill_kernel<1, false><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  if (ct == 2) attn_prefill_kernel<2><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  else attn_prefill_kernel<1><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
   ME_LAUNCH_CHECK();
   return 0;
 }

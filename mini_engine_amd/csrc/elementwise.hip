@@ -136,6 +136,48 @@ __global__ void rms_norm_kernel(const TX* __restrict__ x, int num_partials, int6
   }
 }
 
+// Many rows (prefill): one wave per row, the row held in registers (n <= 64 * 4 * RW_MAX_QUADS),
+// no LDS and no workgroup barrier; 4 rows per workgroup.
+#define RW_MAX_QUADS 4
+template <typename TX, typename TY>
+__global__ void __launch_bounds__(256)
+rms_norm_rows_kernel(const TX* __restrict__ x, const float* __restrict__ res_in, float* __restrict__ res_out,
+                     const float* __restrict__ w, TY* __restrict__ y, int64_t num_rows, int n, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= num_rows) return;
+  float v[RW_MAX_QUADS][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int q = 0; q < RW_MAX_QUADS; ++q) {
+    const int i = (q * 64 + lane) * 4;
+    if (i < n) {
+      Vec4<TX>::load(x + t * n + i, v[q]);
+      if (res_in) {
+        float r[4];
+        Vec4<float>::load(res_in + t * n + i, r);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[q][e] += r[e];
+      }
+      if (res_out) Vec4<float>::store(res_out + t * n + i, v[q]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += v[q][e] * v[q][e];
+    }
+  }
+  const float inv = rsqrtf(wave_sum(ss) / (float)n + eps);
+#pragma unroll
+  for (int q = 0; q < RW_MAX_QUADS; ++q) {
+    const int i = (q * 64 + lane) * 4;
+    if (i < n) {
+      float wv[4], o[4];
+      Vec4<float>::load(w + i, wv);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = wv[e] * (v[q][e] * inv);
+      Vec4<TY>::store(y + t * n + i, o);
+    }
+  }
+}
+
 extern "C" int me_rms_norm(const void* x, int x_dtype, int num_partials, int64_t partial_stride,
                            const float* res_in, float* res_out, const float* w, void* y, int y_dtype,
                            int64_t num_rows, int n, float eps, hipStream_t stream) {
@@ -147,6 +189,19 @@ extern "C" int me_rms_norm(const void* x, int x_dtype, int num_partials, int64_t
   auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
   const bool vec = n % 4 == 0 && al(x) && al(res_in) && al(res_out) && al(w) && al(y) &&
                    (num_partials == 1 || partial_stride % 4 == 0);
+  if (vec && num_partials == 1 && num_rows >= 256 && n <= 64 * 4 * RW_MAX_QUADS) {
+    dim3 grid((num_rows + 3) / 4), block(256);
+#define LAUNCH_ROWS(TX, TY) \
+  rms_norm_rows_kernel<TX, TY><<<grid, block, 0, stream>>>((const TX*)x, res_in, res_out, w, (TY*)y, num_rows, n, eps)
+    if (x_dtype == ME_BF16 && y_dtype == ME_BF16) LAUNCH_ROWS(bf16_t, bf16_t);
+    else if (x_dtype == ME_F32 && y_dtype == ME_BF16) LAUNCH_ROWS(float, bf16_t);
+    else if (x_dtype == ME_F32 && y_dtype == ME_F32) LAUNCH_ROWS(float, float);
+    else if (x_dtype == ME_BF16 && y_dtype == ME_F32) LAUNCH_ROWS(bf16_t, float);
+    else ME_CHECK(false, "rms_norm: bad dtype codes %d %d", x_dtype, y_dtype);
+#undef LAUNCH_ROWS
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   int threads = vec ? (n / 4 >= 1024 ? 1024 : ((n / 4 + 63) / 64) * 64) : (n >= 512 ? 256 : (n >= 128 ? 128 : 64));
   if (threads < 64) threads = 64;
   size_t lds = (size_t)n * sizeof(float);

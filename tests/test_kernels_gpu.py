@@ -32,7 +32,7 @@ def test_gather_rows(dtype, rows, width):
     assert torch.equal(hip().gather_rows(src, idx), twin.gather_rows(src, idx))
 
 
-@pytest.mark.parametrize("T,n", [(1, 80), (13, 1000), (64, 4096), (3, 5120)])
+@pytest.mark.parametrize("T,n", [(1, 80), (13, 1000), (64, 4096), (3, 5120), (300, 1024), (257, 72), (1000, 1028)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rms_norm(dtype, T, n):
     torch.manual_seed(T * n)
