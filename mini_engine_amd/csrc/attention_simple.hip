@@ -26,7 +26,6 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
   float* qs = lds;                 // D
   float* sc = lds + D;             // AS_THREADS scores / probabilities
   __shared__ float red[16];
-  __shared__ float bcast[2];
 
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
@@ -99,7 +98,6 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
     }
     __syncthreads();
   }
-  (void)bcast;
   const float inv = l > 0.f ? 1.f / l : 0.f;
   if (tid < D) out[t * out_stride + (int64_t)h * D + tid] = from_f32<T>(acc0 * inv);
   if (tid + AS_THREADS < D) out[t * out_stride + (int64_t)h * D + tid + AS_THREADS] = from_f32<T>(acc1 * inv);

@@ -6,11 +6,11 @@ parameter is stored in a checkpoint (`weight_sources`).
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import CacheNeed, CacheView, LayerCall, Part, StateNeed
+from ..parts.base import CacheNeed, LayerCall, Part, StateNeed
 from ..parts.block import norm_of
 
 

@@ -8,7 +8,7 @@ name; the step function hands each part the per-step metadata it may need.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Iterator
 
 import torch
@@ -21,8 +21,9 @@ class ParamSpec:
     ``init`` names the distribution used by the random-weights mode:
     ``"matrix"`` ~ N(0, 0.02) (linears, embeddings), ``"norm"`` ~ 1 + U(-0.1, 0.1).
     ``dtype`` is ``"compute"`` (the engine's dtype: bfloat16 or float32),
-    ``"float32"`` (always 32-bit: norm weights, exact for both stored forms) or
-    ``"int32"`` (integer tables).
+    ``"float32"`` (always 32-bit: norm weights, exact for both stored forms),
+    ``"int32"`` (integer tables) or ``"stored"`` (what the checkpoint holds: bfloat16
+    stays bfloat16, 32-bit stays 32-bit).
     """
 
     shape: tuple

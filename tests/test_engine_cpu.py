@@ -179,3 +179,10 @@ def test_padded_decode_layout_without_capture(folders, plain_backend, name):
     for r in lens:
         got = d.result(r)
         assert helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]])) <= helpers.TOL_F32, r
+
+
+def test_toy_architecture_on_cpu(plain_backend):
+    """A stateful mixer, a layer run twice, a call that reads another call's cache and an unfused
+    position encoding, registered from tests/toy_arch.py, stepped through the real runner."""
+    import toy_arch
+    toy_arch.run_toy("cpu", torch.float32, 1e-5)
