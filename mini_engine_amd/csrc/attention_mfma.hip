@@ -61,7 +61,32 @@ struct AttnArgs {
   float* tmp_out;               // [num_seqs, Hq, num_parts, HD] unnormalised
   float* tmp_m;                 // [num_seqs, Hq, num_parts]
   float* tmp_l;
+  // prefill: a tile whose keys span more than seg_keys is cut into segments handled by different
+  // workgroups (grid z); their partial results go to pf_scratch and are merged by a second kernel
+  int seg_keys;                 // 0: no cutting; else a multiple of 32
+  int max_segs;
+  float* pf_scratch;            // [tokens, Hq, max_segs, HD + 2]: unnormalised output, max (log2 domain), sum
+  const int32_t* seq_of_token;  // prefill: [tokens] index of the token's sequence among the prefill sequences + seq_base
+  int seq_base;
 };
+
+// Key range of the tile that holds new token `tl` (index within its sequence's new tokens) and the
+// number of segments it is cut into; shared by the prefill kernel and the merge kernel.
+struct TileRange {
+  int tok0, tile_tokens, tile_lo, tile_base, pos_last, nseg;
+};
+__device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tok0, int q_len, int L) {
+  TileRange r;
+  const int start = L - q_len;
+  r.tok0 = tok0;
+  r.tile_tokens = min(a.tok_tile, q_len - tok0);
+  r.tile_lo = a.window > 0 ? max(0, start + tok0 - a.window + 1) : 0;
+  r.tile_base = r.tile_lo & ~31;
+  r.pos_last = start + tok0 + r.tile_tokens - 1;
+  // never more than the scratch has room for: the last segment then runs to the tile's end
+  r.nseg = a.seg_keys > 0 ? min((r.pos_last + 1 - r.tile_base + a.seg_keys - 1) / a.seg_keys, a.max_segs) : 1;
+  return r;
+}
 
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
@@ -304,9 +329,14 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
   const int L = a.context_lens[b];
   const int start = L - q_len;  // position of the sequence's first new token
   const int32_t* bt = a.block_tables + (int64_t)b * a.bt_stride;
-  const int tile_tokens = min(a.tok_tile, q_len - tok0);
+  const TileRange tr = tile_range(a, tok0, q_len, L);
+  const int tile_tokens = tr.tile_tokens;
   const int ncols = tile_tokens * a.G;
-  const int tile_lo = a.window > 0 ? max(0, start + tok0 - a.window + 1) : 0;
+  const int tile_lo = tr.tile_lo;
+  const int seg = blockIdx.z;
+  if (seg >= tr.nseg) return;
+  const int seg_lo = a.seg_keys > 0 ? tr.tile_base + seg * a.seg_keys : 0;          // keys [seg_lo, seg_hi)
+  const int seg_hi = (a.seg_keys > 0 && seg + 1 < tr.nseg) ? seg_lo + a.seg_keys : (1 << 30);
 
   for (int c0 = wave * 16 * CT; c0 < ncols; c0 += 4 * 16 * CT) {
     bf16x8 qb[CT][KS];
@@ -356,7 +386,9 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
     // pipeline: page ids two blocks ahead, keys and values one block ahead of the products. The
     // fetches are unconditional, also past the last block (they then read page 0 and are not used):
     // a fetch behind a branch would make the waits of both paths merge into waits on the newest loads.
-    int t0 = w_lo & ~31;
+    int t0 = max(w_lo & ~31, seg_lo);
+    const int last = min(pos_last, seg_hi - 1);      // last key of this wave inside the segment
+    if (t0 <= last) {
     KVBlock A, B;
     VBlock VA, VB;
     BlockPages pn;
@@ -369,19 +401,26 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
       lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
       ATTEND(A, VA);
       t0 += 32;
-      if (t0 > pos_last) break;
+      if (t0 > last) break;
       load_kv(a, pn, kvh, t0 + 32, L, n, g, A);
       load_v(a, A, kvh, t0 + 32, L, n, g, VA);
       lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
       ATTEND(B, VB);
       t0 += 32;
-      if (t0 > pos_last) break;
+      if (t0 > last) break;
+    }
     }
 #undef ATTEND
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
       const float ls = column_sum(l[ct]);
-      if (valid[ct]) {
+      if (valid[ct] && tr.nseg > 1) {      // a segment's share: unnormalised, for the merge kernel
+        float* p = a.pf_scratch + (((int64_t)tq[ct] * a.Hq + head[ct]) * a.max_segs + seg) * (HD + 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          *reinterpret_cast<f32x4*>(p + 16 * dt + 4 * g) = acc[ct][dt];
+        if (g == 0) { p[HD] = m[ct]; p[HD + 1] = ls; }
+      } else if (valid[ct]) {
         const float inv = ls > 0.f ? 1.f / ls : 0.f;
         bf16_t* o = a.out + tq[ct] * a.out_stride + (int64_t)head[ct] * HD + 4 * g;
 #pragma unroll
@@ -393,6 +432,29 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(AttnArgs a) {
         }
       }
     }
+  }
+}
+
+// Merge of the segments of cut tiles: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s.
+// Grid (tokens, Hq); tokens of tiles that were not cut already hold their result and return.
+__global__ void __launch_bounds__(128) attn_prefill_merge_kernel(AttnArgs a) {
+  const int64_t t = blockIdx.x;
+  const int hq = blockIdx.y;
+  const int b = a.seq_of_token[t] - a.seq_base;
+  const int q0 = a.cu_seqlens[b], q_len = a.cu_seqlens[b + 1] - q0;
+  const int tok0 = ((int)(t - q0) / a.tok_tile) * a.tok_tile;
+  const TileRange tr = tile_range(a, tok0, q_len, a.context_lens[b]);
+  if (tr.nseg <= 1) return;
+  const float* p = a.pf_scratch + ((t * a.Hq + hq) * a.max_segs) * (HD + 2);
+  float M = NEG;
+  for (int s = 0; s < tr.nseg; ++s) M = fmaxf(M, p[s * (HD + 2) + HD]);
+  float ls = 0.f;
+  for (int s = 0; s < tr.nseg; ++s) ls += exp2f(p[s * (HD + 2) + HD] - M) * p[s * (HD + 2) + HD + 1];
+  const float inv = ls > 0.f ? 1.f / ls : 0.f;
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < tr.nseg; ++s) o += exp2f(p[s * (HD + 2) + HD] - M) * p[s * (HD + 2) + d];
+    a.out[t * a.out_stride + (int64_t)hq * HD + d] = static_cast<bf16_t>(o * inv);
   }
 }
 
@@ -536,6 +598,7 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
   for (int s = 0; s < 31; ++s) if ((1 << s) == page) a.page_shift = s;
   a.scale = scale; a.window = window; a.tok_tile = 1; a.part_size = 0; a.num_parts = 1;
   a.tmp_out = a.tmp_m = a.tmp_l = nullptr;
+  a.seg_keys = 0; a.max_segs = 1; a.pf_scratch = nullptr; a.seq_of_token = nullptr; a.seq_base = 0;
   return 0;
 }
 
@@ -545,7 +608,8 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                                const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                int bt_stride, const int32_t* context_lens, const int32_t* cu_seqlens,
                                int num_seqs, int64_t num_tokens, int Hq, int Hkv, int page, float scale,
-                               int window, int col_tiles_per_wave, hipStream_t stream) {
+                               int window, int col_tiles_per_wave, int seg_keys, int max_segs, float* pf_scratch,
+                               const int32_t* seq_of_token, int seq_base, hipStream_t stream) {
   if (num_seqs == 0 || num_tokens == 0) return 0;
   AttnArgs a;
   if (fill_common(a, q, q_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
@@ -558,9 +622,20 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   a.tok_tile = a.G >= cols ? 1 : cols / a.G;
   const int64_t tiles = num_tokens / a.tok_tile + num_seqs;
   ME_CHECK(tiles < (1ll << 31), "attention: too many tiles");
-  if (ct == 2) attn_prefill_kernel<2><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
-  else attn_prefill_kernel<1><<<dim3((unsigned)tiles, Hkv), dim3(256), 0, stream>>>(a);
+  if (seg_keys > 0 && max_segs > 1) {
+    ME_CHECK(seg_keys % 32 == 0 && max_segs <= 65535, "attention: bad segment size %d or count %d", seg_keys, max_segs);
+    ME_CHECK(pf_scratch && seq_of_token, "attention: cutting tiles into segments needs scratch and seq_of_token");
+    a.seg_keys = seg_keys; a.max_segs = max_segs; a.pf_scratch = pf_scratch;
+    a.seq_of_token = seq_of_token; a.seq_base = seq_base;
+  }
+  const dim3 grid((unsigned)tiles, Hkv, a.max_segs);
+  if (ct == 2) attn_prefill_kernel<2><<<grid, dim3(256), 0, stream>>>(a);
+  else attn_prefill_kernel<1><<<grid, dim3(256), 0, stream>>>(a);
   ME_LAUNCH_CHECK();
+  if (a.max_segs > 1) {
+    attn_prefill_merge_kernel<<<dim3((unsigned)num_tokens, Hq), dim3(128), 0, stream>>>(a);
+    ME_LAUNCH_CHECK();
+  }
   return 0;
 }
 

@@ -65,7 +65,7 @@ _CORE_PROTOS = {
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
-    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, P],
+    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, P, P, I, P],
     "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, P],
 }
 
@@ -219,13 +219,15 @@ class HipBackend:
     # -- attention -----------------------------------------------------------------------
     def paged_attention(self, q, k_cache, v_cache, page: int, block_tables, context_lens, seq_of_token,
                         positions, prefill_cu, num_decodes: int, max_decode_context: int, scale: float,
-                        window: int | None, Hq: int, Hkv: int, D: int, force_simple: bool = False):
+                        window: int | None, Hq: int, Hkv: int, D: int, force_simple: bool = False,
+                        max_prefill_context: int = 0):
         """Causal attention of this step's tokens over the paged keys of their requests.
 
         q: [T, Hq*D] (a strided view is fine). Rows are ordered decode requests first (one token
         each, `num_decodes` of them), then the others; `prefill_cu` int32 [B - num_decodes + 1]
         are prefix sums of the new-token counts of the others. `context_lens` int32 [B] counts keys
-        after this step's write; `block_tables` int32 [B, MB]. Returns [T, Hq*D].
+        after this step's write; `block_tables` int32 [B, MB]. `max_prefill_context`: the largest
+        context among the others (a hint for cutting long key ranges; 0 = unknown). Returns [T, Hq*D].
         (reference layers/attention.py:63-76: decode rows to the decode kernel, the rest to the
         prefill kernel; csrc/paged_decode.cu, csrc/paged_prefill.cu.)"""
         T = q.shape[0]
@@ -256,11 +258,15 @@ class HipBackend:
                      num_decodes, Hq, Hkv, page, float(scale), win, part_size, num_parts, _ptr(scratch), _stream())
         if T > num_decodes:
             _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
+            Tp = T - num_decodes
+            seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq)
+            pf = torch.empty((Tp * Hq * max_segs * (D + 2),), dtype=torch.float32, device=q.device) if max_segs > 1 else None
             lib.call("me_attn_prefill", q.data_ptr() + num_decodes * q.stride(0) * es, q.stride(0),
                      out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
                      block_tables.stride(0), context_lens.data_ptr() + num_decodes * 4, prefill_cu.data_ptr(),
-                     B - num_decodes, T - num_decodes, Hq, Hkv, page, float(scale), win, PREFILL_COL_TILES, _stream())
+                     B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, PREFILL_COL_TILES, seg_keys, max_segs,
+                     _ptr(pf), seq_of_token.data_ptr() + num_decodes * 4, num_decodes, _stream())
         return out
 
     # -- matrix products -----------------------------------------------------------------
@@ -353,6 +359,7 @@ class HipBackend:
 SKINNY_MAX_M = 16        # rows up to which the skinny MFMA kernel beats the library product (measured)
 PARTIALS_MAX_M = 32      # rows up to which a product split over K (float32 partial sums) does
 LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go to the library at any M
+PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 GATED_MAX_M = 16
 _TARGET_WORKGROUPS = 512
@@ -369,6 +376,27 @@ def _scratch(num_floats: int, device) -> torch.Tensor:
         buf = torch.empty((max(2 * num_floats, 1 << 22),), dtype=torch.float32, device=device)
         _scratch_buf[device] = buf
     return buf
+
+
+def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int) -> tuple:
+    """(keys per segment, most segments per tile) for the prefill kernel; (0, 1): no cutting.
+
+    A step with few new tokens over a long context (a late chunk of a long prompt) gives the
+    kernel few workgroups, each walking the whole context. Cutting the key range into segments
+    run by different workgroups fills the GPU; a second kernel merges the segments' results.
+    Measured at 16x128 heads: 256 tokens over 8,192 keys 355 -> 147 us. With enough workgroups
+    already, cutting only adds the merge: 2,048 tokens over 2,048 keys 89 -> 100 us, so it is
+    left whole. PREFILL_SEGMENT_KEYS forces a segment size."""
+    span = min(max_context, window + 256) if window else max_context
+    if PREFILL_SEGMENT_KEYS is not None:
+        seg = PREFILL_SEGMENT_KEYS
+        return (seg, -(-span // seg) + 1) if seg > 0 and span > seg else (0, 1)
+    workgroups = max(1, num_tokens * Hq // (128 if num_tokens * Hq >= 32768 else 64))
+    if workgroups >= 192 or span < 1024:
+        return 0, 1
+    segs = min(-(-512 // workgroups), span // 256)
+    seg = -(-(-(-span // segs)) // 32) * 32
+    return seg, -(-span // seg) + 1
 
 
 def choose_ksplit(M: int, N: int, K: int) -> int:

@@ -86,5 +86,6 @@ class Attention(Mixer):
         q = qkv[:, : self.q_size]
         o = ops.paged_attention(q, cache.k, cache.v, cache.page_size, grp.block_tables, step.context_lens,
                                 step.seq_of_token, step.positions, step.prefill_cu, step.num_decodes,
-                                step.max_decode_context, self.scale, self.window, Hq, Hkv, D)
+                                step.max_decode_context, self.scale, self.window, Hq, Hkv, D,
+                                max_prefill_context=step.max_prefill_context)
         return self.o.forward(o, allow_partials=True)

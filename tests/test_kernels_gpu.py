@@ -212,6 +212,29 @@ def test_attention_window_edges(dtype, window):
         close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
 
 
+@pytest.mark.parametrize("seg_keys", [32, 96, 256])
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 64, 16), (16, 8, 128, 16), (6, 2, 32, 8), (3, 1, 48, 32)])
+def test_attention_prefill_cut_into_segments(monkeypatch, seg_keys, Hq, Hkv, D, page):
+    """Long tiles cut into key segments run by different workgroups and merged: every segment
+    count from 1 up, a segment that holds none of a wave's keys, the peak in each segment, a
+    window, and a context bound that is too small (the last segment then takes the rest)."""
+    monkeypatch.setattr(ops, "PREFILL_SEGMENT_KEYS", seg_keys)
+    seqs = [(700, 700), (40, 40), (513, 130), (300, 2), (1000, 64)]
+    for peak, window, bound in ((None, None, 1000), (0, None, 1000), (450, None, 1000), (699, None, 1000),
+                                (None, 200, 1000), (600, 200, 1000), (333, None, 300), (None, None, 0)):
+        args = _attention_case(torch.bfloat16, Hq, Hkv, D, page, seqs, window=window, seed=seg_keys, peak=peak)
+        close(hip().paged_attention(*args, max_prefill_context=bound), twin.paged_attention(*args), 1.5e-2)
+
+
+def test_attention_prefill_segments_chosen_automatically():
+    """A short chunk at the end of a long context is cut by the engine's own rule."""
+    seqs = [(2500, 33), (1100, 2)]
+    assert ops.prefill_segments(2500, 0, 35, 4)[1] > 1 and ops.prefill_segments(2048, 0, 2048, 16) == (0, 1)
+    for peak in (None, 3, 1200, 2467):
+        args = _attention_case(torch.bfloat16, 4, 2, 64, 16, seqs, seed=5, peak=peak)
+        close(hip().paged_attention(*args, max_prefill_context=2500), twin.paged_attention(*args), 1.5e-2)
+
+
 def test_attention_generic_path_takes_odd_sizes():
     """Head size 24 and page 5 are outside the matrix-core kernel: the generic kernel takes them."""
     for dtype in (torch.float32, torch.bfloat16):
