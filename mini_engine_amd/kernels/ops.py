@@ -275,8 +275,9 @@ class HipBackend:
         """x [M, K] . w[N, K]^T (reference layers/linear.py:25-26: F.linear, no bias).
 
         float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 16 rows (32 when K is
-        split), the library product (hipBLASLt through torch) above that and for the head over a
-        large vocabulary, the FMA kernel for shapes the MFMA kernel refuses. With allow_partials a
+        split), the library product (hipBLASLt through torch) above that, for the head over a
+        large vocabulary and for large weights with 2 or more rows (LIBRARY_MIN_WEIGHT), the FMA
+        kernel for shapes the MFMA kernel refuses. With allow_partials a
         skinny product with few output features may split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
         adds them."""
         _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: {tuple(x.shape)} x {tuple(w.shape)}^T")
@@ -298,13 +299,14 @@ class HipBackend:
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
             return y
-        ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype) else 1
+        ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype
+                                            and not library_streams_better(M, N, K)) else 1
         if ksplit > 1:
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
                         ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, _stream())
             return parts
-        if M <= SKINNY_MAX_M and N < LIBRARY_MIN_N:
+        if M <= SKINNY_MAX_M and N < LIBRARY_MIN_N and not library_streams_better(M, N, K):
             y = torch.empty((M, N), dtype=out_dtype, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), None, 1, M, N, K, 0, _stream())
@@ -317,12 +319,14 @@ class HipBackend:
 
     def silu_mul_linear(self, gu: torch.Tensor, w: torch.Tensor, allow_partials: bool = False):
         """(silu(gu[:, :I]) * gu[:, I:]) . w[N, I]^T: the gating fused into the product for few
-        rows (bfloat16, M <= 16, where the product is a weight stream and the gating is free);
+        rows and a moderate width (bfloat16, M <= 16, I <= 4096, where the product is a weight stream
+        and the gating is free);
         otherwise the two kernels one after the other (reference models/qwen3.py:50-51)."""
         M, two_i = gu.shape
         inter = two_i // 2
         _check(w.shape[1] == inter and two_i == 2 * inter, f"silu_mul_linear: {tuple(gu.shape)} against {tuple(w.shape)}")
         fused = (gu.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and M <= GATED_MAX_M and inter % 8 == 0
+                 and inter <= GATED_MAX_K and not library_streams_better(M, w.shape[0], inter)
                  and gu.is_contiguous() and w.stride(1) == 1 and w.stride(0) % 8 == 0
                  and gu.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
         if not fused:
@@ -359,9 +363,24 @@ class HipBackend:
 SKINNY_MAX_M = 16        # rows up to which the skinny MFMA kernel beats the library product (measured)
 PARTIALS_MAX_M = 32      # rows up to which a product split over K (float32 partial sums) does
 LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go to the library at any M
+# Large weights with 2 or more rows go to the library: every workgroup of the skinny kernel reads
+# all of x, which at 8 to 16 rows is as much traffic as the weights themselves. Measured with 8
+# rows, weights streamed from HBM (us, skinny / library): at Qwen3-8B sizes qkv 6144x4096
+# 19.3 / 14.2, gate_up 24576x4096 59.8 / 45.4, down 4096x12288 28.0 / 22.1, and below the
+# threshold o 4096x4096 11.2 / 15.4; at Qwen3-32B sizes qkv 10240x5120 39.9 / 24.7, o 5120x8192
+# 34.6 / 20.5, gate_up 51200x5120 96.7 / 96.3, but down 5120x25600 113.8 / 136.0 (the library's
+# choice for a very long K is poor, hence LIBRARY_MAX_K). With one row the two are level on
+# average (the library wins on the 32B qkv and o, loses 2x on its down); all Qwen3-0.6B products
+# favour the skinny kernel.
+LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
+LIBRARY_MAX_K = 16384
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 PREFILL_PIPELINE = 0           # 0: chosen by the launcher; 1: two register sets (one wave per SIMD); 2: one set (two waves)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
+# The fused form evaluates the gate in every workgroup (N/16 of them), which is free while the
+# product waits for its weights but not over a long K: at 4096x12288, one row, fused 63 us against
+# 27 us for the plain product after a separate gating kernel (3 us).
+GATED_MAX_K = 4096
 GATED_MAX_M = 16
 _TARGET_WORKGROUPS = 512
 _DECODE_WORKGROUPS = 4096
@@ -398,6 +417,11 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int) ->
     segs = min(-(-512 // workgroups), span // 256)
     seg = -(-(-(-span // segs)) // 32) * 32
     return seg, -(-span // seg) + 1
+
+
+def library_streams_better(M: int, N: int, K: int) -> bool:
+    """Whether a product of few rows goes to the library rather than the skinny kernel."""
+    return M >= 2 and N * K >= LIBRARY_MIN_WEIGHT and K <= LIBRARY_MAX_K
 
 
 def choose_ksplit(M: int, N: int, K: int) -> int:

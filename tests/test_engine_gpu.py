@@ -106,6 +106,25 @@ def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(fold
         assert [o["token_ids"] for o in wide.generate(prompts, sp, use_tqdm=False)] == out_together
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefix_hits_give_the_same_tokens(folders, dtype):
+    """A request whose first pages were written by another request (prefix cache hit) starts its
+    prompt behind them: its tokens equal those of a run without the cache."""
+    from mini_engine_amd import SamplingParams
+    folder = folders("A")
+    shared = helpers.random_ids(40, 256, 990)
+    prompts = [shared + helpers.random_ids(5, 256, 991), shared + helpers.random_ids(9, 256, 992)]
+    sp = SamplingParams(temperature=0, max_tokens=6)
+    kw = dict(kvcache_block_size=16, num_kvcache_blocks=16, max_num_seqs=4, max_num_batched_tokens=256, max_model_len=128)
+    cold = _llm(folder, dtype, enable_prefix_caching=False, **kw)
+    want = [o["token_ids"] for o in cold.generate(prompts, sp, use_tqdm=False)]
+    warm = _llm(folder, dtype, **kw)
+    first = warm.generate(prompts[:1], sp, use_tqdm=False)[0]["token_ids"]
+    assert warm.manager.find_prefix_hit(prompts[1]).num_pages == 2          # 32 of the 40 shared tokens
+    second = warm.generate(prompts[1:], sp, use_tqdm=False)[0]["token_ids"]
+    assert [first, second] == want
+
+
 def test_float32_logits_do_not_depend_on_the_cut_bitwise(folders):
     """The float32 kernels fix the order of every sum per token, so cuts agree to the last bit."""
     env = Env(folders, torch.float32)

@@ -1,0 +1,35 @@
+"""The host-side rules that pick a kernel form (pure functions of the sizes), on the CPU."""
+from mini_engine_amd.kernels import ops
+
+
+def test_decode_partitions_cover_the_context():
+    for S, Hq, Hkv, ctx in ((1, 16, 8, 2048), (8, 16, 8, 2048), (64, 16, 8, 2304), (1, 32, 8, 100), (3, 6, 2, 130000),
+                            (256, 64, 8, 1), (1, 4, 4, 129)):
+        part, parts = ops.decode_partitions(S, Hq, Hkv, ctx)
+        assert part % 128 == 0 and parts <= 64 or part * 64 >= ctx
+        assert part * parts >= ctx and part * (parts - 1) < ctx
+
+
+def test_prefill_segments_cover_the_span_and_only_cut_small_launches():
+    assert ops.prefill_segments(2048, 0, 2048, 16) == (0, 1)          # enough workgroups: left whole
+    assert ops.prefill_segments(900, 0, 4, 16) == (0, 1)              # short span: left whole
+    for ctx, window, tokens, heads in ((8192, 0, 256, 16), (32768, 0, 64, 16), (40000, 0, 2, 32), (5000, 3000, 8, 4)):
+        seg, most = ops.prefill_segments(ctx, window, tokens, heads)
+        span = min(ctx, window + 256) if window else ctx
+        assert seg > 0 and seg % 32 == 0 and (most - 1) * seg >= span
+    assert ops.prefill_segments(8192, 512, 64, 16) == (0, 1)          # a window bounds the span
+
+
+def test_ksplit_keeps_256_of_k_per_split_and_fills_the_gpu():
+    assert ops.choose_ksplit(8, 4096, 1024) == 1                       # 256 feature tiles already
+    for M, N, K in ((8, 1024, 2048), (1, 1024, 3072), (16, 80, 224), (8, 1024, 256)):
+        ks = ops.choose_ksplit(M, N, K)
+        assert 1 <= ks <= 8 and (ks == 1 or K // ks >= 256)
+
+
+def test_large_weights_with_several_rows_go_to_the_library():
+    assert not ops.library_streams_better(1, 24576, 4096)              # one row: the skinny kernel
+    assert ops.library_streams_better(8, 24576, 4096)
+    assert not ops.library_streams_better(8, 4096, 4096)               # below the size threshold
+    assert not ops.library_streams_better(8, 5120, 25600)              # very long K: the library's choice is poor
+    assert not ops.library_streams_better(16, 6144, 1024)
