@@ -6,9 +6,10 @@
 //    (no matrix-core, no reduced precision). Each output element is one thread's sequential sum
 //    over K, so a row's result does not depend on the other rows of the batch. This is the
 //    float32 path and the fallback for bf16 shapes the MFMA kernel refuses.
-//  * me_gemm_skinny_bf16: the decode product, M <= 16 (up to 32 rows when K is split over workgroups). Pure weight streaming: each workgroup
-//    owns 16 output features, its 4 waves split K, every lane reads 64 contiguous bytes of a
-//    weight row per step (whole cache lines per row and wave), products on
+//  * me_gemm_skinny_bf16: the decode product, M <= 16 (up to 32 rows when K is split over
+//    workgroups). Pure weight streaming: each workgroup owns 16 output features, its 4 waves split
+//    K, every lane reads 64 contiguous bytes of a weight row per step (whole cache lines per row
+//    and wave), the fetches run two steps ahead of the products, products on
 //    v_mfma_f32_16x16x32_bf16 with the tokens as the 16-wide B operand, waves merged through
 //    LDS. Optional split of K over workgroups writes float32 partial sums [S, M, N] that the
 //    consumer (the fused residual + RMSNorm kernel) adds in a fixed order.
@@ -102,6 +103,15 @@ __device__ __forceinline__ bf16x8 silu_mul8(const bf16x8 g, const bf16x8 u) {
 // One macro step's operands. Loads are unconditional (a row or a k beyond the matrix is read from
 // row 0 / k 0 instead and zeroed afterwards), so they all go out together and the next step's
 // loads are in flight while this step's products run.
+// Keeps the loads issued so far where they are. A value that is loaded in one loop iteration and
+// first used in the next reaches its use through a phi, and the compiler rewrites "phi of loads"
+// into "load of a phi of addresses": the load then sits in front of its use and nothing is in
+// flight ahead. Something that may write memory between the load and the end of its block forbids
+// that rewrite; an empty statement that claims to do so costs no instruction and no wait.
+__device__ __forceinline__ void pin_loads() { asm volatile("" ::: "memory"); }
+
+#define SKINNY_DEPTH 3  // operand sets in the ring: fetches run SKINNY_DEPTH - 1 steps ahead
+
 template <int MT, bool GATED>
 struct SkinnyOperands {
   bf16x8 a[4];
@@ -109,7 +119,10 @@ struct SkinnyOperands {
   bf16x8 u[GATED ? MT : 1][4];
 };
 
-template <int MT, typename TO, bool GATED>
+// EXACT_K: K is a multiple of 128, so no k-slot of any step lies beyond K and nothing is zeroed.
+// Rows beyond N or M are read from row 0 and not zeroed either: an output element depends on its
+// own weight row and token row only, and the elements of such rows are never written.
+template <int MT, typename TO, bool GATED, bool EXACT_K>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                    TO* __restrict__ y, int64_t ldy, float* __restrict__ partials, int M, int N, int K,
@@ -123,15 +136,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
   const int total_steps = (K + 127) / 128;
   const int s_end = min(total_steps, s_begin + steps_per_split);
 
-  const bool wrow_ok = n0 + r < N;
-  const bf16_t* wrow = w + (int64_t)(wrow_ok ? n0 + r : 0) * ldw;
+  const bf16_t* wrow = w + (int64_t)(n0 + r < N ? n0 + r : 0) * ldw;
   const bf16_t* xrow[MT];
-  bool xrow_ok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = m0 + 16 * mt + r;
-    xrow_ok[mt] = m < M;
-    xrow[mt] = x + (int64_t)(xrow_ok[mt] ? m : 0) * ldx;
+    xrow[mt] = x + (int64_t)(m < M ? m : 0) * ldx;
   }
   f32x4 acc[MT];
 #pragma unroll
@@ -143,7 +153,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = kb + 8 * j;
-      const int ks = k < K ? k : 0;
+      const int ks = (EXACT_K || k < K) ? k : 0;
       op.a[j] = *reinterpret_cast<const bf16x8*>(wrow + ks);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
@@ -156,33 +166,45 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
     const int kb = 128 * s + 32 * g;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const bool kok = kb + 8 * j < K;
-      const bf16x8 a = (wrow_ok && kok) ? op.a[j] : z;
+      const bool kok = EXACT_K || kb + 8 * j < K;
+      const bf16x8 a = kok ? op.a[j] : z;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         bf16x8 b = op.b[mt][j];
         if (GATED) b = silu_mul8(b, op.u[mt][j]);
-        b = (xrow_ok[mt] && kok) ? b : z;
         acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
       }
     }
   };
 
-  // this wave's macro steps: s_begin + wave, + 4, ...; fetched one step ahead, also past the end
-  // (then from k = 0, unused), so that no fetch sits behind a branch
+  // This wave's macro steps are s_begin + wave, + 4, ... Up to two steps: both fetched at once.
+  // More: a ring of SKINNY_DEPTH operand sets keeps the fetches of the next SKINNY_DEPTH - 1 steps
+  // in flight while a step's products run; a fetch past the wave's last step re-reads the last
+  // step (no fetch sits behind a branch) and its products are skipped.
   int s = s_begin + wave;
   if (s < s_end) {
-    SkinnyOperands<MT, GATED> A, B;
-    fetch(s, A);
-    while (true) {
-      fetch(s + 4 < s_end ? s + 4 : s, B);
-      product(s, A);
-      s += 4;
-      if (s >= s_end) break;
-      fetch(s + 4 < s_end ? s + 4 : s, A);
-      product(s, B);
-      s += 4;
-      if (s >= s_end) break;
+    const int last = s + ((s_end - 1 - s) >> 2 << 2);   // this wave's last step
+    if (last <= s + 4) {
+      SkinnyOperands<MT, GATED> first, second;
+      fetch(s, first);
+      if (last > s) fetch(last, second);
+      pin_loads();
+      product(s, first);
+      if (last > s) product(last, second);
+    } else {
+      SkinnyOperands<MT, GATED> ring[SKINNY_DEPTH];
+#pragma unroll
+      for (int d = 0; d < SKINNY_DEPTH - 1; ++d) fetch(min(s + 4 * d, last), ring[d]);
+      pin_loads();
+      while (s <= last) {
+#pragma unroll
+        for (int u = 0; u < SKINNY_DEPTH; ++u) {
+          fetch(min(s + 4 * (SKINNY_DEPTH - 1), last), ring[(u + SKINNY_DEPTH - 1) % SKINNY_DEPTH]);
+          pin_loads();
+          if (s <= last) product(s, ring[u]);
+          s += 4;
+        }
+      }
     }
   }
   // accumulator: lane (token r, g) holds features n0 + 4g + i
@@ -219,25 +241,29 @@ extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, in
   dim3 grid((N + 15) / 16, (M + 16 * mt - 1) / (16 * mt), ksplit), block(256);
   ME_CHECK(grid.y <= 65535, "skinny gemm: too many rows (%d)", M);
   ME_CHECK(!gated || ldx >= 2 * (int64_t)K, "skinny gemm: gated input rows must hold 2K values");
+  const bool exact = K % 128 == 0;
+#define LAUNCH1(MTV, TO, G, E)                                                                               \
+  gemm_skinny_kernel<MTV, TO, G, E><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, \
+                                                                (TO*)y, ldy, partials, M, N, K, steps_per_split)
 #define LAUNCH(MTV, TO)                                                                                      \
   do {                                                                                                       \
-    if (gated)                                                                                               \
-      gemm_skinny_kernel<MTV, TO, true><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, \
-                                                                    ldw, (TO*)y, ldy, partials, M, N, K,    \
-                                                                    steps_per_split);                       \
-    else                                                                                                     \
-      gemm_skinny_kernel<MTV, TO, false><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, \
-                                                                     ldw, (TO*)y, ldy, partials, M, N, K,   \
-                                                                     steps_per_split);                      \
+    if (exact) LAUNCH1(MTV, TO, false, true); else LAUNCH1(MTV, TO, false, false);                           \
   } while (0)
+#define LAUNCH_GATED(TO)                                                                                     \
+  do {                                                                                                       \
+    if (exact) LAUNCH1(1, TO, true, true); else LAUNCH1(1, TO, true, false);                                 \
+  } while (0)
+  ME_CHECK(!gated || mt == 1, "skinny gemm: the gated form takes at most 16 rows (%d)", M);
   if (out_dtype == ME_F32 || partials) {
-    if (mt == 4) LAUNCH(4, float); else if (mt == 2) LAUNCH(2, float); else LAUNCH(1, float);
+    if (gated) LAUNCH_GATED(float); else if (mt == 4) LAUNCH(4, float); else if (mt == 2) LAUNCH(2, float); else LAUNCH(1, float);
   } else if (out_dtype == ME_BF16) {
-    if (mt == 4) LAUNCH(4, bf16_t); else if (mt == 2) LAUNCH(2, bf16_t); else LAUNCH(1, bf16_t);
+    if (gated) LAUNCH_GATED(bf16_t); else if (mt == 4) LAUNCH(4, bf16_t); else if (mt == 2) LAUNCH(2, bf16_t); else LAUNCH(1, bf16_t);
   } else {
     ME_CHECK(false, "skinny gemm: bad output dtype code %d", out_dtype);
   }
+#undef LAUNCH_GATED
 #undef LAUNCH
+#undef LAUNCH1
   ME_LAUNCH_CHECK();
   return 0;
 }

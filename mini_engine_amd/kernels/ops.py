@@ -276,7 +276,7 @@ class HipBackend:
 
         float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 16 rows (32 when K is
         split), the library product (hipBLASLt through torch) above that, for the head over a
-        large vocabulary and for large weights with 2 or more rows (LIBRARY_MIN_WEIGHT), the FMA
+        large vocabulary and for large weights with several rows (library_streams_better), the FMA
         kernel for shapes the MFMA kernel refuses. With allow_partials a
         skinny product with few output features may split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
         adds them."""
@@ -363,15 +363,19 @@ class HipBackend:
 SKINNY_MAX_M = 16        # rows up to which the skinny MFMA kernel beats the library product (measured)
 PARTIALS_MAX_M = 32      # rows up to which a product split over K (float32 partial sums) does
 LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go to the library at any M
-# Large weights with 2 or more rows go to the library: every workgroup of the skinny kernel reads
-# all of x, which at 8 to 16 rows is as much traffic as the weights themselves. Measured with 8
-# rows, weights streamed from HBM (us, skinny / library): at Qwen3-8B sizes qkv 6144x4096
-# 19.3 / 14.2, gate_up 24576x4096 59.8 / 45.4, down 4096x12288 28.0 / 22.1, and below the
-# threshold o 4096x4096 11.2 / 15.4; at Qwen3-32B sizes qkv 10240x5120 39.9 / 24.7, o 5120x8192
-# 34.6 / 20.5, gate_up 51200x5120 96.7 / 96.3, but down 5120x25600 113.8 / 136.0 (the library's
-# choice for a very long K is poor, hence LIBRARY_MAX_K). With one row the two are level on
-# average (the library wins on the 32B qkv and o, loses 2x on its down); all Qwen3-0.6B products
-# favour the skinny kernel.
+# Large weights with LIBRARY_MIN_ROWS or more rows go to the library: every workgroup of the skinny
+# kernel reads all of x, which at 8 to 16 rows is as much traffic as the weights themselves.
+# Measured with weights streamed from HBM (us, skinny / library), Qwen3-8B sizes:
+#   rows   qkv 6144x4096   o 4096x4096   gate_up 24576x4096   down 4096x12288
+#     1    15.7 / 14.3      9.5 / 15.4      45.0 / 45.5          22.0 / 22.4
+#     4    17.6 / 15.6     10.1 / 15.4      48.5 / 45.5          22.7 / 22.4
+#     8    18.9 / 14.3     10.8 / 15.6      54.3 / 45.4          25.0 / 22.4
+#    16    22.3 / 14.3     12.4 / 15.5      65.9 / 45.6          31.2 / 22.8
+# (o is below the size threshold.) At Qwen3-32B sizes, 8 rows: qkv 10240x5120 36.7 / 24.8,
+# o 5120x8192 33.4 / 20.5, gate_up 51200x5120 96.8 / 96.7, but down 5120x25600 85.3 / 136.4: the
+# library's choice for a very long K is poor, hence LIBRARY_MAX_K. All Qwen3-0.6B products favour
+# the skinny kernel (3.3-5.5 us against 7.4-12 us).
+LIBRARY_MIN_ROWS = 4
 LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
 LIBRARY_MAX_K = 16384
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
@@ -421,7 +425,7 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int) ->
 
 def library_streams_better(M: int, N: int, K: int) -> bool:
     """Whether a product of few rows goes to the library rather than the skinny kernel."""
-    return M >= 2 and N * K >= LIBRARY_MIN_WEIGHT and K <= LIBRARY_MAX_K
+    return M >= LIBRARY_MIN_ROWS and N * K >= LIBRARY_MIN_WEIGHT and K <= LIBRARY_MAX_K
 
 
 def choose_ksplit(M: int, N: int, K: int) -> int:

@@ -29,6 +29,7 @@ def test_ksplit_keeps_256_of_k_per_split_and_fills_the_gpu():
 
 def test_large_weights_with_several_rows_go_to_the_library():
     assert not ops.library_streams_better(1, 24576, 4096)              # one row: the skinny kernel
+    assert not ops.library_streams_better(2, 24576, 4096)              # two rows: still level
     assert ops.library_streams_better(8, 24576, 4096)
     assert not ops.library_streams_better(8, 4096, 4096)               # below the size threshold
     assert not ops.library_streams_better(8, 5120, 25600)              # very long K: the library's choice is poor
