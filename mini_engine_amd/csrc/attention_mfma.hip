@@ -137,7 +137,7 @@ struct KVBlock {   // the keys of a block: fetched one block ahead of their use
   // where the block's values are (looked up with the keys' pages, fetched when the block is used:
   // they are needed only after the scores and the softmax, which cover their latency)
   int vpage, voff;
-  bool vgrp_ok;
+  int vkeys;  // how many of this lane's 8 keys of the V operand may be used (0: none)
 };
 struct VBlock {
   bf16x8 v[DT];
@@ -185,9 +185,19 @@ __device__ __forceinline__ void load_kv(const AttnArgs& a, const BlockPages& pg,
       blk.k[tt][ks] = ld8(kp + ((HD % 32 == 0 || d0 < HD) ? d0 : 0));
     }
   }
-  blk.vgrp_ok = pg.vgrp_ok && pg.vpage >= 0;
-  blk.vpage = blk.vgrp_ok ? pg.vpage : 0;
-  blk.voff = blk.vgrp_ok ? pg.voff : 0;
+  const bool vgrp_ok = pg.vgrp_ok && pg.vpage >= 0;
+  blk.vpage = vgrp_ok ? pg.vpage : 0;
+  blk.voff = vgrp_ok ? pg.voff : 0;
+  blk.vkeys = vgrp_ok ? L - (t0 + 8 * g) : 0;
+}
+
+// Makes the block's value-page fields exist in registers of their own from here on. They are
+// selects on the table entry that lookup_pages fetched; left alone, the compiler forms them where
+// they are used (when the values are fetched, late in a loop iteration), keeps the raw entry alive
+// until then, and must copy the next lookup's result into its register at the end of the
+// iteration, which waits for every load in flight.
+__device__ __forceinline__ void settle_value_page(KVBlock& blk) {
+  asm volatile("" : "+v"(blk.vpage), "+v"(blk.voff), "+v"(blk.vkeys));
 }
 
 // V^T rows: channel 16*dt + n, keys t0 + 8g .. t0 + 8g + 7
@@ -197,7 +207,7 @@ __device__ __forceinline__ void load_v(const AttnArgs& a, const KVBlock& blk, in
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) vb.v[dt] = ld8(vp + (int64_t)dt * 16 * a.page);
   // keys at or past L hold foreign or unwritten data (possibly NaN): their bits are cleared
-  const int nv = blk.vgrp_ok ? L - (t0 + 8 * g) : 0;
+  const int nv = blk.vkeys;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
     vb.vmask[j] = (2 * j < nv ? 0x0000ffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
@@ -385,8 +395,8 @@ __device__ __forceinline__ float column_sum(float l) { return sum_over_groups(l)
 // Grid: (floor(T / tok_tile) + num_seqs) * Hkv. The first tile of sequence b is
 // floor(cu[b] / tok_tile) + b, an upper bound of the tiles before it; surplus tiles exit.
 // =====================================================================================
-template <int CT, bool DEEP>
-__global__ void __launch_bounds__(256, DEEP ? 1 : 2) attn_prefill_kernel(AttnArgs a) {
+template <int CT>
+__global__ void __launch_bounds__(256, 2) attn_prefill_kernel(AttnArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   // Workgroups go to the 8 XCDs in turn, each with an L2 of its own: consecutive ids take the kv
@@ -452,59 +462,28 @@ __global__ void __launch_bounds__(256, DEEP ? 1 : 2) attn_prefill_kernel(AttnArg
     // above the last column's window start) needs no masks
     const int full_hi = pos_first - 31;                                   // t0 <= full_hi: all 32 keys visible
     const int full_lo = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;  // t0 >= full_lo: none behind a window
-    // Two pipelines. DEEP: two sets of key and value registers, the next block fetched whole while
-    // this one is used; only one wave fits on a SIMD, but a wave alone on its SIMD is fastest this
-    // way, so it serves launches of about one workgroup per CU or fewer. Otherwise one set,
-    // refilled as soon as the products that read it are issued (the next keys arrive behind the
-    // softmax and the value product, the next values behind the score product and the softmax):
-    // two waves fit on a SIMD, and one wave's softmax (vector ALU) runs beside the other's products
-    // (matrix cores). Measured inside a 28-layer prefill: 2,048 tokens 6.56 ms deep against 6.92,
-    // 8,192 tokens 29.6 ms deep against 27.6. Page ids are looked up a block earlier still. The
-    // fetches are unconditional, also past the last block (they then read page 0 and are not used):
-    // a fetch behind a branch would make the waits of both paths merge into waits on the newest loads.
+    // One set of key registers and one of value registers, refilled as soon as the products that
+    // read them are issued: the next keys arrive behind the softmax and the value product, the next
+    // values behind the score product and the softmax. Page ids are looked up a block earlier
+    // still. The fetches are unconditional, also past the last block (they then read page 0 and are
+    // not used): a fetch behind a branch would make the waits of both paths merge into waits on the
+    // newest loads. With single sets two waves fit on a SIMD. (Two sets per wave, the next block
+    // fetched whole while this one is used, need more than 256 registers, leave one wave per
+    // SIMD, and measured slower at every size: 2,048 tokens 93 against 78 us, 8,192 tokens 689
+    // against 668 us.)
     int t0 = max(w_lo & ~31, seg_lo);
     const int last = min(pos_last, seg_hi - 1);      // last key of this wave inside the segment
-    if (DEEP) {
-      if (t0 <= last) {
-        KVBlock A, B;
-        VBlock VA, VB;
-        BlockPages pn;
-#define ATTEND(BLK, VBLK)                                                                                    \
-  do {                                                                                                       \
-    if (t0 <= full_hi && t0 >= full_lo) {                                                                    \
-      _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                      \
-          attend_block<true>(a, BLK, VBLK, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);    \
-    } else {                                                                                                 \
-      _Pragma("unroll") for (int ct = 0; ct < CT; ++ct)                                                      \
-          attend_block<false>(a, BLK, VBLK, t0, qb[ct], col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g);   \
-    }                                                                                                        \
-  } while (0)
-        load_block(a, bt, kvh, t0, L, tile_lo, n, g, A);
-        load_v(a, A, kvh, t0, L, n, g, VA);
-        lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
-        while (true) {
-          load_kv(a, pn, kvh, t0 + 32, L, n, g, B);
-          load_v(a, B, kvh, t0 + 32, L, n, g, VB);
-          lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
-          ATTEND(A, VA);
-          t0 += 32;
-          if (t0 > last) break;
-          load_kv(a, pn, kvh, t0 + 32, L, n, g, A);
-          load_v(a, A, kvh, t0 + 32, L, n, g, VA);
-          lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
-          ATTEND(B, VB);
-          t0 += 32;
-          if (t0 > last) break;
-        }
-#undef ATTEND
-      }
-    } else if (t0 <= last) {
+    if (t0 <= last) {
       KVBlock K;
       VBlock V;
       BlockPages pn;
+      // issued in the order of the loop (keys, page ids, values): the waits inside the loop are
+      // placed for the worse of the two ways into it, and a different order here would make every
+      // iteration wait as if the page ids had been fetched last
       load_block(a, bt, kvh, t0, L, tile_lo, n, g, K);
-      load_v(a, K, kvh, t0, L, n, g, V);
+      settle_value_page(K);
       lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
+      load_v(a, K, kvh, t0, L, n, g, V);
       while (true) {
         const bool full = t0 <= full_hi && t0 >= full_lo;
         if (!full) hide_keys(K);
@@ -512,6 +491,7 @@ __global__ void __launch_bounds__(256, DEEP ? 1 : 2) attn_prefill_kernel(AttnArg
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) block_scores(K, qb[ct], g, st[ct]);
         load_kv(a, pn, kvh, t0 + 32, L, n, g, K);
+        settle_value_page(K);
         lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
         bf16x8 pb[CT];
 #pragma unroll
@@ -740,7 +720,7 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                                const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                int bt_stride, const int32_t* context_lens, const int32_t* cu_seqlens,
                                int num_seqs, int64_t num_tokens, int Hq, int Hkv, int page, float scale,
-                               int window, int col_tiles_per_wave, int pipeline, int seg_keys, int max_segs, float* pf_scratch,
+                               int window, int col_tiles_per_wave, int seg_keys, int max_segs, float* pf_scratch,
                                const int32_t* seq_of_token, int seq_base, hipStream_t stream) {
   if (num_seqs == 0 || num_tokens == 0) return 0;
   AttnArgs a;
@@ -761,11 +741,8 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
     a.seq_of_token = seq_of_token; a.seq_base = seq_base;
   }
   const dim3 grid((unsigned)(tiles * Hkv), 1, a.max_segs);
-  const bool deep = pipeline == 1 || (pipeline != 2 && tiles * Hkv * a.max_segs <= 320);
-  if (ct == 2 && deep) attn_prefill_kernel<2, true><<<grid, dim3(256), 0, stream>>>(a);
-  else if (ct == 2) attn_prefill_kernel<2, false><<<grid, dim3(256), 0, stream>>>(a);
-  else if (deep) attn_prefill_kernel<1, true><<<grid, dim3(256), 0, stream>>>(a);
-  else attn_prefill_kernel<1, false><<<grid, dim3(256), 0, stream>>>(a);
+  if (ct == 2) attn_prefill_kernel<2><<<grid, dim3(256), 0, stream>>>(a);
+  else attn_prefill_kernel<1><<<grid, dim3(256), 0, stream>>>(a);
   ME_LAUNCH_CHECK();
   if (a.max_segs > 1) {
     const int64_t rows = num_tokens * Hq;
