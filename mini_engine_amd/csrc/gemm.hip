@@ -6,8 +6,8 @@
 //    (no matrix-core, no reduced precision). Each output element is one thread's sequential sum
 //    over K, so a row's result does not depend on the other rows of the batch. This is the
 //    float32 path and the fallback for bf16 shapes the MFMA kernel refuses.
-//  * me_gemm_skinny_bf16: the decode product, M <= 16 (up to 32 rows when K is split over
-//    workgroups). Pure weight streaming: each workgroup owns 16 output features, its 4 waves split
+//  * me_gemm_skinny_bf16: the decode product, up to 64 rows (the caller decides from which row
+//    count the library is faster). Pure weight streaming: each workgroup owns 16 output features, its 4 waves split
 //    K, every lane reads 64 contiguous bytes of a weight row per step (whole cache lines per row
 //    and wave), the fetches run two steps ahead of the products, products on
 //    v_mfma_f32_16x16x32_bf16 with the tokens as the 16-wide B operand, waves merged through

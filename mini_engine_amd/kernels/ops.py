@@ -274,8 +274,8 @@ class HipBackend:
                allow_partials: bool = False):
         """x [M, K] . w[N, K]^T (reference layers/linear.py:25-26: F.linear, no bias).
 
-        float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 16 rows (32 when K is
-        split), the library product (hipBLASLt through torch) above that, for the head over a
+        float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 32 rows (64 for
+        smaller weights or when K is split), the library product (hipBLASLt through torch) above that, for the head over a
         large vocabulary and for large weights with several rows (library_streams_better), the FMA
         kernel for shapes the MFMA kernel refuses. With allow_partials a
         skinny product with few output features may split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
@@ -306,7 +306,7 @@ class HipBackend:
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
                         ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, _stream())
             return parts
-        if M <= SKINNY_MAX_M and N < LIBRARY_MIN_N and not library_streams_better(M, N, K):
+        if skinny_takes(M, N, K):
             y = torch.empty((M, N), dtype=out_dtype, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), None, 1, M, N, K, 0, _stream())
@@ -360,8 +360,15 @@ class HipBackend:
         return out
 
 
-SKINNY_MAX_M = 16        # rows up to which the skinny MFMA kernel beats the library product (measured)
-PARTIALS_MAX_M = 32      # rows up to which a product split over K (float32 partial sums) does
+# Rows up to which the skinny MFMA kernel beats the library product. Measured at Qwen3-0.6B sizes
+# (us, skinny / library): 32 rows qkv 4096x1024 6.0 / 11.2, gate_up 6144x1024 8.8 / 11.5; 64 rows
+# qkv 8.1 / 11.6 but gate_up 14.3 / 11.8, hence the smaller limit for weights above
+# SKINNY_WIDE_MAX_WEIGHT elements. Split over K with the sum left to the norm kernel
+# (product + norm): 64 rows o 1024x2048 10.6 / 11.3, down 1024x3072 11.9 / 14.3.
+SKINNY_MAX_M = 32
+SKINNY_WIDE_MAX_M = 64
+SKINNY_WIDE_MAX_WEIGHT = 5 * 1024 * 1024
+PARTIALS_MAX_M = 64      # rows up to which a product split over K (float32 partial sums) pays
 LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go to the library at any M
 # Large weights with LIBRARY_MIN_ROWS or more rows go to the library: every workgroup of the skinny
 # kernel reads all of x, which at 8 to 16 rows is as much traffic as the weights themselves.
@@ -420,6 +427,12 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int) ->
     segs = min(-(-512 // workgroups), span // 256)
     seg = -(-(-(-span // segs)) // 32) * 32
     return seg, -(-span // seg) + 1
+
+
+def skinny_takes(M: int, N: int, K: int) -> bool:
+    """Whether the skinny kernel (without a split over K) takes an aligned bfloat16 product."""
+    rows_ok = M <= SKINNY_MAX_M or (M <= SKINNY_WIDE_MAX_M and N * K <= SKINNY_WIDE_MAX_WEIGHT)
+    return rows_ok and N < LIBRARY_MIN_N and not library_streams_better(M, N, K)
 
 
 def library_streams_better(M: int, N: int, K: int) -> bool:

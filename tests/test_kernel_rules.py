@@ -34,3 +34,10 @@ def test_large_weights_with_several_rows_go_to_the_library():
     assert not ops.library_streams_better(8, 4096, 4096)               # below the size threshold
     assert not ops.library_streams_better(8, 5120, 25600)              # very long K: the library's choice is poor
     assert not ops.library_streams_better(16, 6144, 1024)
+
+
+def test_skinny_kernel_takes_few_rows():
+    assert ops.skinny_takes(32, 6144, 1024) and not ops.skinny_takes(33, 6144, 1024)
+    assert ops.skinny_takes(64, 4096, 1024) and not ops.skinny_takes(65, 4096, 1024)
+    assert not ops.skinny_takes(1, 151936, 1024)                       # the head goes to the library
+    assert not ops.skinny_takes(8, 24576, 4096)
