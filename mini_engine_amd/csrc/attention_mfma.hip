@@ -52,7 +52,7 @@ struct AttnArgs {
   const int32_t* cu_seqlens;    // prefill: [num_seqs + 1] prefix sums of new tokens
   int num_seqs;
   int Hq, Hkv, G;
-  int page, page_shift;         // page_shift >= 0 iff page is a power of two
+  int page, page_shift;         // page = 1 << page_shift
   float scale;
   int window;                   // 0: all keys
   int tok_tile;                 // prefill: query tokens per workgroup
@@ -117,9 +117,6 @@ __device__ __forceinline__ float sum_over_groups(float v) {
   return __uint_as_float(r2[0]) + __uint_as_float(r2[1]);
 }
 
-__device__ __forceinline__ int page_index(int tok, int page, int shift) {
-  return shift >= 0 ? (tok >> shift) : (tok / page);
-}
 
 // -------------------------------------------------------------------------------------
 // A 32-key block [t0, t0+32) of one kv head, as the operands of the two products.
@@ -157,12 +154,12 @@ __device__ __forceinline__ void lookup_pages(const AttnArgs& a, const int32_t* _
                                              int lo_min, int n, int g, BlockPages& pg) {
   const int kgrp = t0 + 8 * (n >> 2);
   pg.kgrp_ok = kgrp < L && kgrp + 7 >= lo_min;
-  const int kpi = pg.kgrp_ok ? page_index(kgrp, a.page, a.page_shift) : 0;
+  const int kpi = pg.kgrp_ok ? (kgrp >> a.page_shift) : 0;
   pg.kpage = bt[kpi];
   pg.koff = pg.kgrp_ok ? kgrp - kpi * a.page + (n & 3) : (n & 3);
   const int vgrp = t0 + 8 * g;
   pg.vgrp_ok = vgrp < L && vgrp + 7 >= lo_min;
-  const int vpi = pg.vgrp_ok ? page_index(vgrp, a.page, a.page_shift) : 0;
+  const int vpi = pg.vgrp_ok ? (vgrp >> a.page_shift) : 0;
   pg.vpage = bt[vpi];
   pg.voff = pg.vgrp_ok ? vgrp - vpi * a.page : 0;
 }
@@ -333,13 +330,14 @@ __device__ __forceinline__ void block_scores(const KVBlock& blk, const bf16x8 (&
 // Online-softmax update of one 16-column tile from its block scores (as in attend_block):
 // rescales l and acc when some column's max has risen and returns the probabilities as the
 // operand of the value product.
-__device__ __forceinline__ void block_softmax(const AttnArgs& a, const f32x4 (&st)[2], bool full, int t0, int col_lo,
+template <bool FULL>
+__device__ __forceinline__ void block_softmax(const AttnArgs& a, const f32x4 (&st)[2], int t0, int col_lo,
                                               int col_hi, float& m, float& l, f32x4 (&acc)[DT], int g, bf16x8& pb) {
   const float c = a.scale * 1.4426950408889634f;
   float sv[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) sv[i] = st[i >> 2][i & 3];
-  if (!full) {
+  if (!FULL) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int j = t0 + 8 * g + i;
@@ -368,7 +366,7 @@ __device__ __forceinline__ void block_softmax(const AttnArgs& a, const f32x4 (&s
     // a masked score is NEG: while the column has seen no key m is NEG too, and exp2(NEG * c - NEG)
     // is not 0, hence the select
     float p = __builtin_amdgcn_exp2f(fmaf(sv[i], c, -m));
-    if (!full) p = sv[i] > 0.5f * NEG ? p : 0.f;
+    if (!FULL) p = sv[i] > 0.5f * NEG ? p : 0.f;
     psum += p;
     pb[i] = static_cast<bf16_t>(p);
   }
@@ -395,8 +393,10 @@ __device__ __forceinline__ float column_sum(float l) { return sum_over_groups(l)
 // Grid: (floor(T / tok_tile) + num_seqs) * Hkv. The first tile of sequence b is
 // floor(cu[b] / tok_tile) + b, an upper bound of the tiles before it; surplus tiles exit.
 // =====================================================================================
+// Two waves per SIMD, not more: a third (the narrow form would fit) only adds to the keys and values
+// in flight, which then push each other out of the L1 (256 tokens over 8,192 keys: 126 against 88 us).
 template <int CT>
-__global__ void __launch_bounds__(256, 2) attn_prefill_kernel(AttnArgs a) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) attn_prefill_kernel(AttnArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   // Workgroups go to the 8 XCDs in turn, each with an L2 of its own: consecutive ids take the kv
@@ -494,10 +494,16 @@ __global__ void __launch_bounds__(256, 2) attn_prefill_kernel(AttnArgs a) {
         settle_value_page(K);
         lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
         bf16x8 pb[CT];
+        if (full) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-          block_softmax(a, st[ct], full, t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
-        if (!full) hide_values(V);
+          for (int ct = 0; ct < CT; ++ct)
+            block_softmax<true>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+        } else {
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            block_softmax<false>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+          hide_values(V);
+        }
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
@@ -695,7 +701,7 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
                        const int32_t* context_lens, int num_seqs, int Hq, int Hkv, int page, float scale,
                        int window) {
   ME_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
-  ME_CHECK(page >= 8 && page % 8 == 0, "attention (bf16 MFMA path): page size %d must be a multiple of 8", page);
+  ME_CHECK(page >= 8 && (page & (page - 1)) == 0, "attention (bf16 MFMA path): page size %d must be a power of two, 8 or more", page);
   ME_CHECK(q_stride % 8 == 0 && out_stride % 4 == 0, "attention: token strides must keep 16-byte alignment");
   ME_CHECK((reinterpret_cast<uintptr_t>(q) % 16 == 0) && (reinterpret_cast<uintptr_t>(out) % 8 == 0) &&
                (reinterpret_cast<uintptr_t>(k_cache) % 16 == 0) && (reinterpret_cast<uintptr_t>(v_cache) % 16 == 0),
@@ -706,8 +712,8 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
   a.k_cache = (const bf16_t*)k_cache; a.v_cache = (const bf16_t*)v_cache;
   a.block_tables = block_tables; a.bt_stride = bt_stride; a.context_lens = context_lens;
   a.cu_seqlens = nullptr; a.num_seqs = num_seqs; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv;
-  a.page = page; a.page_shift = -1;
-  for (int s = 0; s < 31; ++s) if ((1 << s) == page) a.page_shift = s;
+  a.page = page; a.page_shift = 0;
+  while ((1 << a.page_shift) < page) ++a.page_shift;
   a.scale = scale; a.window = window; a.tok_tile = 1; a.part_size = 0; a.num_parts = 1;
   a.tmp_out = a.tmp_m = a.tmp_l = nullptr;
   a.seg_keys = 0; a.max_segs = 1; a.pf_scratch = nullptr; a.seq_of_token = nullptr; a.seq_base = 0;

@@ -241,7 +241,8 @@ class HipBackend:
         _check(0 <= num_decodes <= B and num_decodes <= T, "attention: bad decode count")
         out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
         win = int(window or 0)
-        mfma = (q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page % 8 == 0 and not force_simple)
+        mfma = (q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page >= 8 and page & (page - 1) == 0
+                and not force_simple)
         if not mfma:
             core().call("me_attn_simple", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _code(q.dtype),
                         k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),

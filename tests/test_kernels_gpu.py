@@ -240,6 +240,8 @@ def test_attention_generic_path_takes_odd_sizes():
     for dtype in (torch.float32, torch.bfloat16):
         args = _attention_case(dtype, 3, 1, 24, 5, [(40, 1), (23, 23), (9, 2)], seed=1)
         close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
+    args = _attention_case(torch.bfloat16, 4, 2, 32, 24, [(100, 1), (50, 50), (30, 3)], seed=3)   # page 24: no power of two
+    close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
     args = _attention_case(torch.bfloat16, 4, 2, 64, 16, [(300, 1), (70, 70)], seed=2)
     close(hip().paged_attention(*args, force_simple=True), hip().paged_attention(*args), 1.5e-2)
 
