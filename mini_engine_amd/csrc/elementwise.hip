@@ -136,44 +136,73 @@ __global__ void rms_norm_kernel(const TX* __restrict__ x, int num_partials, int6
   }
 }
 
-// Many rows (prefill): one wave per row, the row held in registers (n <= 64 * 4 * RW_MAX_QUADS),
-// no LDS and no workgroup barrier; 4 rows per workgroup.
-#define RW_MAX_QUADS 4
-template <typename TX, typename TY>
+// Many rows (prefill): one wave per row, the row held in registers, no LDS and no workgroup
+// barrier; 4 rows per workgroup. A lane takes 8 consecutive values at a time (16 bytes of bfloat16,
+// two 16-byte pieces of float32). Every load of the row is issued before the first value is used:
+// a piece beyond the row's end is read from its start instead and not used.
+#define RW_MAX_OCTS 10  // n <= 64 * 8 * RW_MAX_OCTS = 5120
+template <typename T> struct Oct;
+template <> struct Oct<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+template <> struct Oct<bf16_t> {
+  typedef bf16_t bf16x8v __attribute__((ext_vector_type(8)));
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const bf16x8v t = *reinterpret_cast<const bf16x8v*>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = static_cast<float>(t[i]);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    bf16x8v t;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = static_cast<bf16_t>(v[i]);
+    *reinterpret_cast<bf16x8v*>(p) = t;
+  }
+};
+
+template <typename TX, typename TY, int OCTS>
 __global__ void __launch_bounds__(256)
 rms_norm_rows_kernel(const TX* __restrict__ x, const float* __restrict__ res_in, float* __restrict__ res_out,
                      const float* __restrict__ w, TY* __restrict__ y, int64_t num_rows, int n, float eps) {
   const int lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= num_rows) return;
-  float v[RW_MAX_QUADS][4];
+  float v[OCTS][8], r[OCTS][8];
+#pragma unroll
+  for (int q = 0; q < OCTS; ++q) {
+    const int i = (q * 64 + lane) * 8;
+    const int is = i < n ? i : 0;
+    Oct<TX>::load(x + t * n + is, v[q]);
+    if (res_in) Oct<float>::load(res_in + t * n + is, r[q]);
+  }
   float ss = 0.f;
 #pragma unroll
-  for (int q = 0; q < RW_MAX_QUADS; ++q) {
-    const int i = (q * 64 + lane) * 4;
-    if (i < n) {
-      Vec4<TX>::load(x + t * n + i, v[q]);
-      if (res_in) {
-        float r[4];
-        Vec4<float>::load(res_in + t * n + i, r);
+  for (int q = 0; q < OCTS; ++q) {
+    const bool in = (q * 64 + lane) * 8 < n;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[q][e] += r[e];
-      }
-      if (res_out) Vec4<float>::store(res_out + t * n + i, v[q]);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) ss += v[q][e] * v[q][e];
+    for (int e = 0; e < 8; ++e) {
+      if (res_in) v[q][e] += r[q][e];
+      ss += in ? v[q][e] * v[q][e] : 0.f;
     }
+    if (res_out && in) Oct<float>::store(res_out + t * n + (q * 64 + lane) * 8, v[q]);
   }
   const float inv = rsqrtf(wave_sum(ss) / (float)n + eps);
 #pragma unroll
-  for (int q = 0; q < RW_MAX_QUADS; ++q) {
-    const int i = (q * 64 + lane) * 4;
+  for (int q = 0; q < OCTS; ++q) {
+    const int i = (q * 64 + lane) * 8;
     if (i < n) {
-      float wv[4], o[4];
-      Vec4<float>::load(w + i, wv);
+      float wv[8], o[8];
+      Oct<float>::load(w + i, wv);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = wv[e] * (v[q][e] * inv);
-      Vec4<TY>::store(y + t * n + i, o);
+      for (int e = 0; e < 8; ++e) o[e] = wv[e] * (v[q][e] * inv);
+      Oct<TY>::store(y + t * n + i, o);
     }
   }
 }
@@ -189,15 +218,22 @@ extern "C" int me_rms_norm(const void* x, int x_dtype, int num_partials, int64_t
   auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
   const bool vec = n % 4 == 0 && al(x) && al(res_in) && al(res_out) && al(w) && al(y) &&
                    (num_partials == 1 || partial_stride % 4 == 0);
-  if (vec && num_partials == 1 && num_rows >= 256 && n <= 64 * 4 * RW_MAX_QUADS) {
+  if (vec && num_partials == 1 && num_rows >= 256 && n % 8 == 0 && n <= 64 * 8 * RW_MAX_OCTS) {
     dim3 grid((num_rows + 3) / 4), block(256);
-#define LAUNCH_ROWS(TX, TY) \
-  rms_norm_rows_kernel<TX, TY><<<grid, block, 0, stream>>>((const TX*)x, res_in, res_out, w, (TY*)y, num_rows, n, eps)
-    if (x_dtype == ME_BF16 && y_dtype == ME_BF16) LAUNCH_ROWS(bf16_t, bf16_t);
-    else if (x_dtype == ME_F32 && y_dtype == ME_BF16) LAUNCH_ROWS(float, bf16_t);
-    else if (x_dtype == ME_F32 && y_dtype == ME_F32) LAUNCH_ROWS(float, float);
-    else if (x_dtype == ME_BF16 && y_dtype == ME_F32) LAUNCH_ROWS(bf16_t, float);
+    const int octs = (n + 511) / 512;
+#define LAUNCH_ROWS(TX, TY, O) \
+  rms_norm_rows_kernel<TX, TY, O><<<grid, block, 0, stream>>>((const TX*)x, res_in, res_out, w, (TY*)y, num_rows, n, eps)
+#define PICK_ROWS(TX, TY)                                                                                   \
+  do {                                                                                                      \
+    if (octs <= 2) LAUNCH_ROWS(TX, TY, 2); else if (octs <= 4) LAUNCH_ROWS(TX, TY, 4);                      \
+    else if (octs <= 8) LAUNCH_ROWS(TX, TY, 8); else LAUNCH_ROWS(TX, TY, RW_MAX_OCTS);                     \
+  } while (0)
+    if (x_dtype == ME_BF16 && y_dtype == ME_BF16) PICK_ROWS(bf16_t, bf16_t);
+    else if (x_dtype == ME_F32 && y_dtype == ME_BF16) PICK_ROWS(float, bf16_t);
+    else if (x_dtype == ME_F32 && y_dtype == ME_F32) PICK_ROWS(float, float);
+    else if (x_dtype == ME_BF16 && y_dtype == ME_F32) PICK_ROWS(bf16_t, float);
     else ME_CHECK(false, "rms_norm: bad dtype codes %d %d", x_dtype, y_dtype);
+#undef PICK_ROWS
 #undef LAUNCH_ROWS
     ME_LAUNCH_CHECK();
     return 0;

@@ -221,6 +221,125 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, int64_t row_stride, const flo
   Quad<T>::store(dst + half + 4 * l, o2);
 }
 
+// ------------------------------------------------------------------ many tokens: 8 tokens per workgroup
+// The same arithmetic for steps with many tokens (prefill). Grid (groups of 8 consecutive tokens,
+// q/k workgroups + one value workgroup). q and k heads: LPH = D/16 lanes share a head, a lane reads 8 values of each
+// half (16 bytes), their 8 (cos, sin), and writes both back. Value heads: a thread takes 8 channels
+// of a head, reads them for the 8 tokens, transposes the 8x8 block in registers and writes one
+// 16-byte piece per channel into the transposed page (when the 8 slots are consecutive places of
+// one page, starting at a multiple of 8; otherwise value by value).
+typedef bf16_t bf16x8r __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4r __attribute__((ext_vector_type(4)));
+
+template <int LPH>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_tile_kernel(bf16_t* __restrict__ qkv, int64_t row_stride, const float* __restrict__ q_w,
+                               const float* __restrict__ k_w, float eps, const float* __restrict__ table,
+                               const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+                               bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int Hq, int Hkv, int D,
+                               int page, int store, int64_t num_tokens, int qk_groups) {
+  const int64_t t0 = (int64_t)blockIdx.x * 8;
+  const int cnt = (int)min((int64_t)8, num_tokens - t0);
+  const int half = D >> 1;
+  const int heads = Hq + Hkv;
+  const int l = threadIdx.x % LPH;
+  // ---- q and k heads: workgroups y < qk_groups, one (token, head) per LPH lanes
+  if ((int)blockIdx.y < qk_groups) {
+    const int item = blockIdx.y * (256 / LPH) + threadIdx.x / LPH;
+    if (item >= cnt * heads) return;
+    const int ti = item / heads, head = item - ti * heads;
+    const int64_t t = t0 + ti;
+    const bool is_q = head < Hq;
+    bf16_t* row = qkv + t * row_stride + (int64_t)head * D;
+    const bf16x8r a = *reinterpret_cast<const bf16x8r*>(row + 8 * l);
+    const bf16x8r b = *reinterpret_cast<const bf16x8r*>(row + half + 8 * l);
+    float x1[8], x2[8];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      x1[i] = static_cast<float>(a[i]); x2[i] = static_cast<float>(b[i]);
+      ss += x1[i] * x1[i] + x2[i] * x2[i];
+    }
+    const float* w = is_q ? q_w : k_w;
+    float inv = 1.f;
+    if (w) {
+#pragma unroll
+      for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, ME_WAVE);
+      inv = rsqrtf(ss / (float)D + eps);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { x1[i] *= inv; x2[i] *= inv; }
+    if (w) {
+      const float4 wa = *reinterpret_cast<const float4*>(w + 8 * l), wb = *reinterpret_cast<const float4*>(w + 8 * l + 4);
+      const float4 wc = *reinterpret_cast<const float4*>(w + half + 8 * l), wd = *reinterpret_cast<const float4*>(w + half + 8 * l + 4);
+      const float w1[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w}, w2[8] = {wc.x, wc.y, wc.z, wc.w, wd.x, wd.y, wd.z, wd.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { x1[i] *= w1[i]; x2[i] *= w2[i]; }
+    }
+    if (table) {
+      const float4* cs = reinterpret_cast<const float4*>(table + ((int64_t)positions[t] * half + 8 * l) * 2);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {   // a float4 holds (cos, sin) of two pairs
+        const float4 c = cs[i];
+        const float a0 = x1[2 * i], b0 = x2[2 * i], a1 = x1[2 * i + 1], b1 = x2[2 * i + 1];
+        x1[2 * i] = a0 * c.x - b0 * c.y; x2[2 * i] = b0 * c.x + a0 * c.y;
+        x1[2 * i + 1] = a1 * c.z - b1 * c.w; x2[2 * i + 1] = b1 * c.z + a1 * c.w;
+      }
+    }
+    bf16_t* dst = row;
+    if (!is_q && store) {
+      const int slot = slots[t];
+      if (slot < 0) return;
+      const int64_t pg = slot / page, off = slot - pg * page;
+      dst = k_cache + ((pg * Hkv + (head - Hq)) * (int64_t)page + off) * D;
+    }
+    bf16x8r o1, o2;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { o1[i] = static_cast<bf16_t>(x1[i]); o2[i] = static_cast<bf16_t>(x2[i]); }
+    *reinterpret_cast<bf16x8r*>(dst + 8 * l) = o1;
+    *reinterpret_cast<bf16x8r*>(dst + half + 8 * l) = o2;
+    return;
+  }
+  // ---- value heads: the last workgroup of the 8 tokens
+  const int s0 = slots[t0];
+  bool run = cnt == 8 && s0 >= 0 && (s0 & 7) == 0;
+  if (run) {
+#pragma unroll
+    for (int i = 1; i < 8; ++i) run = run && slots[t0 + i] == s0 + i;
+  }
+  const int dvecs = D >> 3;
+  for (int unit = threadIdx.x; unit < Hkv * dvecs; unit += 256) {
+    const int kvh = unit / dvecs, dv = unit - kvh * dvecs;
+    const bf16_t* src = qkv + t0 * row_stride + (int64_t)(heads + kvh) * D + 8 * dv;
+    if (run) {
+      u32x4r tok[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tok[i] = *reinterpret_cast<const u32x4r*>(src + i * row_stride);
+      const int64_t pg = s0 / page, off = s0 - pg * page;
+      bf16_t* dst = v_cache + ((pg * Hkv + kvh) * (int64_t)D + 8 * dv) * page + off;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {   // channel d of the 8 tokens: word d/2 of each token, low or high half
+        u32x4r o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t lo = tok[2 * j][d >> 1], hi = tok[2 * j + 1][d >> 1];
+          o[j] = (d & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+        }
+        *reinterpret_cast<u32x4r*>(dst + (int64_t)d * page) = o;
+      }
+    } else {
+      for (int i = 0; i < cnt; ++i) {
+        const int slot = slots[t0 + i];
+        if (slot < 0) continue;
+        const int64_t pg = slot / page, off = slot - pg * page;
+        bf16_t* dst = v_cache + ((pg * Hkv + kvh) * (int64_t)D + 8 * dv) * page + off;
+#pragma unroll
+        for (int d = 0; d < 8; ++d) dst[(int64_t)d * page] = src[i * row_stride + d];
+      }
+    }
+  }
+}
+
 extern "C" int me_qk_norm_rope_store(void* qkv, int dtype, int64_t num_tokens, int64_t row_stride,
                                      const float* q_w, const float* k_w, float eps,
                                      const float* table, int64_t table_positions,
@@ -243,6 +362,27 @@ extern "C" int me_qk_norm_rope_store(void* qkv, int dtype, int64_t num_tokens, i
                    reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(q_w) % 16 == 0 && reinterpret_cast<uintptr_t>(k_w) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(table) % 16 == 0;
+  // many tokens of bfloat16: 8 tokens per workgroup (16 lanes-worth of bytes per lane)
+  const int lph16 = D / 16;
+  const bool tile = vec && dtype == ME_BF16 && num_tokens >= 64 && D % 16 == 0 && lph16 >= 1 && lph16 <= 64 &&
+                    (lph16 & (lph16 - 1)) == 0 && (!store || (page % 8 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0));
+  if (tile) {
+    const int per_group = 256 / lph16;
+    const int qk_groups = (8 * (Hq + Hkv) + per_group - 1) / per_group;
+    dim3 grid((unsigned)((num_tokens + 7) / 8), qk_groups + (store ? 1 : 0)), block(256);
+#define LAUNCH_TILE(L)                                                                                     \
+  qk_norm_rope_store_tile_kernel<L><<<grid, block, 0, stream>>>((bf16_t*)qkv, row_stride, q_w, k_w, eps, table, \
+                                                                positions, slots, (bf16_t*)k_cache,       \
+                                                                (bf16_t*)v_cache, Hq, Hkv, D, page, store, num_tokens, qk_groups)
+    switch (lph16) {
+      case 1: LAUNCH_TILE(1); break; case 2: LAUNCH_TILE(2); break; case 4: LAUNCH_TILE(4); break;
+      case 8: LAUNCH_TILE(8); break; case 16: LAUNCH_TILE(16); break; case 32: LAUNCH_TILE(32); break;
+      default: LAUNCH_TILE(64); break;
+    }
+#undef LAUNCH_TILE
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   if (vec) {
     const int hpw = 64 / lph;
     const int qk_blocks = (Hq + Hkv + 4 * hpw - 1) / (4 * hpw);

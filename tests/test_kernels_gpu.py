@@ -32,7 +32,8 @@ def test_gather_rows(dtype, rows, width):
     assert torch.equal(hip().gather_rows(src, idx), twin.gather_rows(src, idx))
 
 
-@pytest.mark.parametrize("T,n", [(1, 80), (13, 1000), (64, 4096), (3, 5120), (300, 1024), (257, 72), (1000, 1028)])
+@pytest.mark.parametrize("T,n", [(1, 80), (13, 1000), (64, 4096), (3, 5120), (300, 1024), (257, 72), (1000, 1028),
+                                 (300, 520), (257, 4104), (256, 5120), (260, 5128)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rms_norm(dtype, T, n):
     torch.manual_seed(T * n)
@@ -100,6 +101,42 @@ def test_qk_norm_rope_store(dtype, Hq, Hkv, D, page):
     a, b = qkv[:, :Hq * D].clone(), qkv[:, :Hq * D].clone()
     hip().qk_norm_rope_store(a, qw, qw, 1e-5, table, pos, None, None, None, Hq, 0, D, page, False)
     twin.qk_norm_rope_store(b, qw, qw, 1e-5, table, pos, None, None, None, Hq, 0, D, page, False)
+    close(a, b, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 16, 16), (6, 2, 32, 8), (5, 5, 48, 8), (16, 8, 128, 16), (2, 1, 256, 32),
+                                           (3, 3, 64, 24)])
+def test_qk_norm_rope_store_many_tokens(dtype, Hq, Hkv, D, page):
+    """The form for many tokens (8 per workgroup): prompts written to consecutive slots from page
+    starts and from the middle of a page, a token count that is no multiple of 8, scattered slots,
+    skipped tokens."""
+    torch.manual_seed(D + page)
+    T, P, pages = 203, 512, 40
+    qkv = torch.randn(T, (Hq + 2 * Hkv) * D, device=DEV).to(dtype)
+    qw, kw = torch.rand(D, device=DEV) + 0.5, torch.rand(D, device=DEV) + 0.5
+    ang = torch.outer(torch.arange(P, dtype=torch.float32), 1.0 / (1e4 ** (torch.arange(0, D, 2).float() / D)))
+    table = torch.stack((ang.cos(), ang.sin()), -1).contiguous().to(DEV)
+    pos = torch.randint(0, P, (T,), device=DEV, dtype=torch.int32)
+    slots = torch.empty(T, dtype=torch.int64)
+    slots[:96] = torch.arange(96) + 5 * page                    # a prompt from a page start
+    slots[96:150] = torch.arange(54) + 20 * page + 3            # a chunk that starts inside a page
+    slots[150:] = (torch.randperm(8 * page)[:T - 150] + 30 * page)   # scattered
+    slots[[7, 100, 160]] = -1
+    slots = slots.to(torch.int32).to(DEV)
+    tol = 2e-6 if dtype == torch.float32 else 4e-3
+    a, b = qkv.clone(), qkv.clone()
+    ka, va = _caches(pages, Hkv, page, D, dtype); kb, vb = _caches(pages, Hkv, page, D, dtype)
+    hip().qk_norm_rope_store(a, qw, kw, 1e-5, table, pos, slots, ka, va, Hq, Hkv, D, page, True)
+    twin.qk_norm_rope_store(b, qw, kw, 1e-5, table, pos, slots, kb, vb, Hq, Hkv, D, page, True)
+    close(a[:, :Hq * D], b[:, :Hq * D], tol)
+    assert torch.equal(torch.isnan(ka), torch.isnan(kb)) and torch.equal(torch.isnan(va), torch.isnan(vb))
+    close(torch.nan_to_num(ka), torch.nan_to_num(kb), tol)
+    assert torch.equal(torch.nan_to_num(va), torch.nan_to_num(vb))
+    assert torch.equal(a[:, Hq * D:], qkv[:, Hq * D:])
+    a, b = qkv[:, :(Hq + Hkv) * D].clone(), qkv[:, :(Hq + Hkv) * D].clone()
+    hip().qk_norm_rope_store(a, None, None, 1e-5, table, pos, None, None, None, Hq, Hkv, D, page, False)
+    twin.qk_norm_rope_store(b, None, None, 1e-5, table, pos, None, None, None, Hq, Hkv, D, page, False)
     close(a, b, tol)
 
 
