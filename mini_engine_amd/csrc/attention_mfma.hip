@@ -484,12 +484,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       settle_value_page(K);
       lookup_pages(a, bt, t0 + 32, L, tile_lo, n, g, pn);
       load_v(a, K, kvh, t0, L, n, g, V);
-      while (true) {
-        const bool full = t0 <= full_hi && t0 >= full_lo;
-        if (!full) hide_keys(K);
-        f32x4 st[CT][2];
+      // The scores of a block are issued at the end of the iteration before, behind the value
+      // products of the block before: the matrix cores then work on both while the vector ALU
+      // does the loop's bookkeeping and the first softmax, instead of each waiting for the other.
+      bool full = t0 <= full_hi && t0 >= full_lo;
+      if (!full) hide_keys(K);
+      f32x4 st[CT][2];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) block_scores(K, qb[ct], g, st[ct]);
+      for (int ct = 0; ct < CT; ++ct) block_scores(K, qb[ct], g, st[ct]);
+      while (true) {
+        // here: st = scores of block t0, V = its values (in flight), K free for the next keys
         load_kv(a, pn, kvh, t0 + 32, L, n, g, K);
         settle_value_page(K);
         lookup_pages(a, bt, t0 + 64, L, tile_lo, n, g, pn);
@@ -512,12 +516,245 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         load_v(a, K, kvh, t0 + 32, L, n, g, V);
         t0 += 32;
         if (t0 > last) break;
+        full = t0 <= full_hi && t0 >= full_lo;
+        if (!full) hide_keys(K);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) block_scores(K, qb[ct], g, st[ct]);
       }
     }
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
       const float ls = column_sum(l[ct]);
       if (valid[ct] && tr.nseg > 1) {      // a segment's share: unnormalised, for the merge kernel
+        float* p = a.pf_scratch + (((int64_t)tq[ct] * a.Hq + head[ct]) * a.max_segs + seg) * (HD + 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          *reinterpret_cast<f32x4*>(p + 16 * dt + 4 * g) = acc[ct][dt];
+        if (g == 0) { p[HD] = m[ct]; p[HD + 1] = ls; }
+      } else if (valid[ct]) {
+        const float inv = ls > 0.f ? 1.f / ls : 0.f;
+        bf16_t* o = a.out + tq[ct] * a.out_stride + (int64_t)head[ct] * HD + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          bf16x4 r;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) r[i] = static_cast<bf16_t>(acc[ct][dt][i] * inv);
+          *reinterpret_cast<bf16x4*>(o + 16 * dt) = r;
+        }
+      }
+    }
+  }
+}
+
+// =====================================================================================
+// Prefill / chunk kernel, keys and values shared through LDS (head sizes up to 128).
+// The four waves of a workgroup need the same 32-key blocks. Fetched by each wave for itself
+// they make four times the L2 traffic that the tile needs (the 32 KB L1 cannot hold what four
+// waves have in flight), and that traffic, not arithmetic, is what bounds the kernel above. Here
+// the 256 threads fetch a block once, each its 16-byte pieces, one block ahead into registers,
+// and put it into LDS, from which every wave reads its matrix operands:
+//   keys    [32 rows][HD + 8]: row tt*16 + n holds key 8*(n>>2) + 4*tt + (n&3) of the block, the
+//           order in which the lanes of an A operand want them (see the top of the file); with
+//           the 16 bytes of padding the 16 lanes of a read hit different banks;
+//   values  [HD rows][32 + 8]: channel-major as in the cache.
+// What must not be used (keys at or past the context, in pages that are not held) is zeroed when
+// it is put into LDS. All waves walk the tile's whole key range in step, one barrier per block
+// (two LDS buffers); a block outside a wave's own range is masked like any other.
+// Same grid and tile geometry as attn_prefill_kernel.
+// =====================================================================================
+#define PF_KROW (2 * HD + 16)            // bytes per key row in LDS
+#define PF_VROW 80                        // bytes per value row in LDS
+#define PF_BUF (32 * PF_KROW + HD * PF_VROW)
+#define PF_PIECES ((4 * HD + 255) / 256)  // 16-byte pieces of a block's keys (and of its values) per thread
+
+struct StagedBlock {
+  bf16x8 k[PF_PIECES], v[PF_PIECES];
+  bool kok[PF_PIECES];
+  int vkeys[PF_PIECES];
+};
+struct StagedPages {   // table entries as loaded, for the block after the staged one
+  int k[PF_PIECES], v[PF_PIECES];
+};
+
+__device__ __forceinline__ void pf_lookup(const AttnArgs& a, const int32_t* __restrict__ bt, int t0, int L,
+                                          int lo_min, int tid, StagedPages& pg) {
+#pragma unroll
+  for (int j = 0; j < PF_PIECES; ++j) {
+    const int p = tid + 256 * j;
+    const int key = t0 + p / (HD / 8);                 // a key row
+    const bool kok = p < 4 * HD && key < L && key >= (lo_min & ~7);
+    pg.k[j] = bt[kok ? key >> a.page_shift : 0];
+    const int key0 = t0 + 8 * (p & 3);                 // a group of 8 keys of one channel
+    const bool vok = p < 4 * HD && key0 < L && key0 + 7 >= lo_min;
+    pg.v[j] = bt[vok ? key0 >> a.page_shift : 0];
+  }
+}
+
+__device__ __forceinline__ void pf_fetch(const AttnArgs& a, const StagedPages& pg, int kvh, int t0, int L,
+                                         int lo_min, int tid, StagedBlock& st) {
+#pragma unroll
+  for (int j = 0; j < PF_PIECES; ++j) {
+    const int p = tid + 256 * j;
+    const int row = p / (HD / 8), ch = p - row * (HD / 8);
+    const int key = t0 + row;
+    const bool kok = p < 4 * HD && key < L && key >= (lo_min & ~7) && pg.k[j] >= 0;
+    st.kok[j] = kok;
+    const bf16_t* kp = a.k_cache + (((int64_t)(kok ? pg.k[j] : 0) * a.Hkv + kvh) * a.page + (kok ? key & (a.page - 1) : 0)) * HD + 8 * ch;
+    st.k[j] = ld8(kp);
+    const int d = p >> 2, key0 = t0 + 8 * (p & 3);
+    const bool vok = p < 4 * HD && key0 < L && key0 + 7 >= lo_min && pg.v[j] >= 0;
+    st.vkeys[j] = vok ? L - key0 : 0;
+    const bf16_t* vp = a.v_cache + (((int64_t)(vok ? pg.v[j] : 0) * a.Hkv + kvh) * HD + (p < 4 * HD ? d : 0)) * a.page + (vok ? key0 & (a.page - 1) : 0);
+    st.v[j] = ld8(vp);
+  }
+}
+
+__device__ __forceinline__ void pf_commit(const StagedBlock& st, int tid, unsigned char* buf) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const bf16x8 z = zero8();
+#pragma unroll
+  for (int j = 0; j < PF_PIECES; ++j) {
+    const int p = tid + 256 * j;
+    if (p < 4 * HD) {
+      const int row = p / (HD / 8), ch = p - row * (HD / 8);
+      const int lrow = ((row >> 2) & 1) * 16 + ((row & 3) | ((row >> 3) << 2));
+      *reinterpret_cast<bf16x8*>(buf + lrow * PF_KROW + 16 * ch) = st.kok[j] ? st.k[j] : z;
+      u32x4 w = __builtin_bit_cast(u32x4, st.v[j]);
+      const int nv = st.vkeys[j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] &= (2 * i < nv ? 0x0000ffffu : 0u) | (2 * i + 1 < nv ? 0xffff0000u : 0u);
+      *reinterpret_cast<u32x4*>(buf + 32 * PF_KROW + (p >> 2) * PF_VROW + 16 * (p & 3)) = w;
+    }
+  }
+}
+
+// the LDS writes of this wave done, every wave at the same point, nothing moved across by the compiler
+__device__ __forceinline__ void pf_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int CT>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) attn_prefill_shared_kernel(AttnArgs a) {
+  extern __shared__ __align__(16) unsigned char pf_lds[];   // [2][PF_BUF]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  const int kvh = blockIdx.x % a.Hkv;
+  const int x = gridDim.x / a.Hkv - 1 - blockIdx.x / a.Hkv;
+  int lo_b = 0, hi_b = a.num_seqs - 1;
+  while (lo_b < hi_b) {
+    const int mid = (lo_b + hi_b + 1) >> 1;
+    if (a.cu_seqlens[mid] / a.tok_tile + mid <= x) lo_b = mid; else hi_b = mid - 1;
+  }
+  const int b = lo_b;
+  const int q0 = a.cu_seqlens[b], q_len = a.cu_seqlens[b + 1] - q0;
+  const int tok0 = (x - (q0 / a.tok_tile + b)) * a.tok_tile;
+  if (tok0 >= q_len) return;
+  const int L = a.context_lens[b];
+  const int start = L - q_len;
+  const int32_t* bt = a.block_tables + (int64_t)b * a.bt_stride;
+  const TileRange tr = tile_range(a, tok0, q_len, L);
+  const int ncols = tr.tile_tokens * a.G;
+  const int tile_lo = tr.tile_lo;
+  const int seg = blockIdx.z;
+  if (seg >= tr.nseg) return;
+  const int seg_lo = a.seg_keys > 0 ? tr.tile_base + seg * a.seg_keys : tr.tile_base;
+  const int seg_hi = (a.seg_keys > 0 && seg + 1 < tr.nseg) ? seg_lo + a.seg_keys : (1 << 30);
+  const int last = min(tr.pos_last, seg_hi - 1);   // the same key range for every wave of the workgroup
+  const float c = a.scale * 1.4426950408889634f;
+  (void)c;
+
+  // every wave runs every round (a wave without columns in a round masks everything and writes nothing)
+  for (int c_base = 0; c_base < ncols; c_base += 4 * 16 * CT) {
+    const bool active = c_base + wave * 16 * CT < ncols;
+    const int c0 = active ? c_base + wave * 16 * CT : 0;
+    bf16x8 qb[CT][KS];
+    int col_lo[CT], col_hi[CT];
+    int64_t tq[CT];
+    int head[CT];
+    bool valid[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int cc = c0 + 16 * ct + n;
+      valid[ct] = active && cc < ncols;
+      const int tl = valid[ct] ? cc / a.G : 0;
+      const int hh = valid[ct] ? cc - tl * a.G : 0;
+      tq[ct] = q0 + tok0 + tl;
+      head[ct] = kvh * a.G + hh;
+      const int pos = start + tok0 + tl;
+      col_hi[ct] = valid[ct] ? pos : -1;
+      col_lo[ct] = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+      load_q(a.q + tq[ct] * a.q_stride + (int64_t)head[ct] * HD, valid[ct], g, qb[ct]);
+    }
+    const int c_last = min(ncols, c0 + 16 * CT) - 1;
+    const int pos_first = start + tok0 + c0 / a.G, pos_last = start + tok0 + c_last / a.G;
+    const int full_hi = active ? pos_first - 31 : -(1 << 30);
+    const int full_lo = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;
+    float m[CT], l[CT];
+    f32x4 acc[CT][DT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      m[ct] = NEG; l[ct] = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    int t0 = seg_lo;
+    StagedBlock stg;
+    StagedPages pg;
+    pf_barrier();                                    // the round before has finished with both buffers
+    pf_lookup(a, bt, t0, L, tile_lo, tid, pg);
+    pf_fetch(a, pg, kvh, t0, L, tile_lo, tid, stg);
+    pf_lookup(a, bt, t0 + 32, L, tile_lo, tid, pg);
+    pf_commit(stg, tid, pf_lds);
+    int cur = 0;
+    while (true) {
+      pf_barrier();                                  // block t0 is in buffer cur
+      pf_fetch(a, pg, kvh, t0 + 32, L, tile_lo, tid, stg);      // the next block, into registers
+      pf_lookup(a, bt, t0 + 64, L, tile_lo, tid, pg);
+      const unsigned char* kb = pf_lds + cur * PF_BUF;
+      const unsigned char* vb = kb + 32 * PF_KROW;
+      const bool full = t0 <= full_hi && t0 >= full_lo;
+      f32x4 st[CT][2];
+      const bf16x8 z = zero8();
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bool dok = HD % 32 == 0 || (32 * ks + 8 * g) < HD;
+          bf16x8 ka = *reinterpret_cast<const bf16x8*>(kb + (tt * 16 + n) * PF_KROW + (dok ? 64 * ks + 16 * g : 0));
+          ka = dok ? ka : z;
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[ct][ks], st[ct][tt], 0, 0, 0);
+        }
+      }
+      bf16x8 pb[CT];
+      if (full) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          block_softmax<true>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+      } else {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          block_softmax<false>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16x8 va = *reinterpret_cast<const bf16x8*>(vb + (16 * dt + n) * PF_VROW + 16 * g);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct], acc[ct][dt], 0, 0, 0);
+      }
+      pf_commit(stg, tid, pf_lds + (cur ^ 1) * PF_BUF);
+      cur ^= 1;
+      t0 += 32;
+      if (t0 > last) break;
+    }
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const float ls = column_sum(l[ct]);
+      if (valid[ct] && tr.nseg > 1) {
         float* p = a.pf_scratch + (((int64_t)tq[ct] * a.Hq + head[ct]) * a.max_segs + seg) * (HD + 2);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -726,7 +963,7 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                                const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                int bt_stride, const int32_t* context_lens, const int32_t* cu_seqlens,
                                int num_seqs, int64_t num_tokens, int Hq, int Hkv, int page, float scale,
-                               int window, int col_tiles_per_wave, int seg_keys, int max_segs, float* pf_scratch,
+                               int window, int col_tiles_per_wave, int shared, int seg_keys, int max_segs, float* pf_scratch,
                                const int32_t* seq_of_token, int seq_base, hipStream_t stream) {
   if (num_seqs == 0 || num_tokens == 0) return 0;
   AttnArgs a;
@@ -747,8 +984,20 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
     a.seq_of_token = seq_of_token; a.seq_base = seq_base;
   }
   const dim3 grid((unsigned)(tiles * Hkv), 1, a.max_segs);
-  if (ct == 2) attn_prefill_kernel<2><<<grid, dim3(256), 0, stream>>>(a);
-  else attn_prefill_kernel<1><<<grid, dim3(256), 0, stream>>>(a);
+  // Keys and values through LDS where the two buffers fit (head sizes up to 128), except for the
+  // wide form at about one workgroup per CU or fewer: there the waves of a workgroup have no
+  // others to fill their waits at the barriers, and fetching per wave is faster (2,048 tokens of
+  // one prompt: 77 against 93 us; with more workgroups, 8,192 tokens: 648 against 521 us).
+  // shared: 0 never, 1 by this rule, 2 wherever it fits.
+  const bool through_lds = 2 * PF_BUF <= 65536 &&
+                           (shared == 2 || (shared == 1 && (ct == 1 || tiles * Hkv * a.max_segs > 320)));
+  if (through_lds) {
+    if (ct == 2) attn_prefill_shared_kernel<2><<<grid, dim3(256), 2 * PF_BUF, stream>>>(a);
+    else attn_prefill_shared_kernel<1><<<grid, dim3(256), 2 * PF_BUF, stream>>>(a);
+  } else {
+    if (ct == 2) attn_prefill_kernel<2><<<grid, dim3(256), 0, stream>>>(a);
+    else attn_prefill_kernel<1><<<grid, dim3(256), 0, stream>>>(a);
+  }
   ME_LAUNCH_CHECK();
   if (a.max_segs > 1) {
     const int64_t rows = num_tokens * Hq;

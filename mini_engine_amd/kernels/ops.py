@@ -65,7 +65,7 @@ _CORE_PROTOS = {
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
-    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, P, P, I, P],
+    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, P, P, I, P],
     "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, P],
 }
 
@@ -266,7 +266,7 @@ class HipBackend:
                      out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
                      block_tables.stride(0), context_lens.data_ptr() + num_decodes * 4, prefill_cu.data_ptr(),
-                     B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, PREFILL_COL_TILES, seg_keys, max_segs,
+                     B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, PREFILL_COL_TILES, PREFILL_THROUGH_LDS, seg_keys, max_segs,
                      _ptr(pf), seq_of_token.data_ptr() + num_decodes * 4, num_decodes, _stream())
         return out
 
@@ -387,6 +387,7 @@ LIBRARY_MIN_ROWS = 4
 LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
 LIBRARY_MAX_K = 16384
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
+PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS: 0 never, 1 chosen by the launcher, 2 wherever it fits
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 # The fused form evaluates the gate in every workgroup (N/16 of them), which is free while the
 # product waits for its weights but not over a long K: at 4096x12288, one row, fused 63 us against

@@ -207,12 +207,20 @@ def _attention_case(dtype, Hq, Hkv, D, page, seqs, window=None, seed=0, peak=Non
     return args
 
 
-SHAPES = [(4, 2, 16, 16), (6, 2, 32, 8), (4, 1, 48, 16), (16, 8, 128, 16), (8, 8, 64, 32), (32, 1, 64, 16), (2, 2, 128, 64)]
+@pytest.fixture(params=[0, 2], ids=["per_wave", "through_lds"])
+def prefill_form(request, monkeypatch):
+    """Both forms of the prefill kernel (the launcher would choose by the size of the launch)."""
+    monkeypatch.setattr(ops, "PREFILL_THROUGH_LDS", request.param)
+    return request.param
+
+
+SHAPES = [(4, 2, 16, 16), (6, 2, 32, 8), (4, 1, 48, 16), (16, 8, 128, 16), (8, 8, 64, 32), (32, 1, 64, 16), (2, 2, 128, 64),
+          (80, 1, 32, 16)]      # the last: more heads in a group than one round of a workgroup's columns
 
 
 @pytest.mark.parametrize("Hq,Hkv,D,page", SHAPES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_attention_prefill_ragged(dtype, Hq, Hkv, D, page):
+def test_attention_prefill_ragged(prefill_form, dtype, Hq, Hkv, D, page):
     """Ragged prompts, chunks that attend to earlier chunks, lengths at tile and page edges."""
     seqs = [(5, 5), (33, 33), (64, 2), (65, 33), (129, 17), (page, page), (page + 1, 2), (200, 64), (31, 31)]
     args = _attention_case(dtype, Hq, Hkv, D, page, seqs, seed=D + page)
@@ -230,7 +238,7 @@ def test_attention_decode_batches(dtype, Hq, Hkv, D, page):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_attention_far_key_stands_out(dtype):
+def test_attention_far_key_stands_out(prefill_form, dtype):
     """One key among hundreds gets all the weight: a kernel that drops or misplaces a block,
     a partition or a page shows an O(1) error here that random scores would average away."""
     for peak in (0, 15, 16, 255, 256, 700, 1023):
@@ -240,7 +248,7 @@ def test_attention_far_key_stands_out(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [1, 7, 16, 24, 100])
-def test_attention_window_edges(dtype, window):
+def test_attention_window_edges(prefill_form, dtype, window):
     """Keys just inside and just outside the window; pages behind it are not held (-1 in the
     table, NaN in memory)."""
     seqs = [(150, 1), (33, 1), (window, 1), (window + 1, 1), (150, 40), (70, 70), (window + 5, 3)]
@@ -251,7 +259,7 @@ def test_attention_window_edges(dtype, window):
 
 @pytest.mark.parametrize("seg_keys", [32, 96, 256])
 @pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 64, 16), (16, 8, 128, 16), (6, 2, 32, 8), (3, 1, 48, 32)])
-def test_attention_prefill_cut_into_segments(monkeypatch, seg_keys, Hq, Hkv, D, page):
+def test_attention_prefill_cut_into_segments(prefill_form, monkeypatch, seg_keys, Hq, Hkv, D, page):
     """Long tiles cut into key segments run by different workgroups and merged: every segment
     count from 1 up, a segment that holds none of a wave's keys, the peak in each segment, a
     window, and a context bound that is too small (the last segment then takes the rest)."""
