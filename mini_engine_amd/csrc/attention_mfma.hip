@@ -984,13 +984,11 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
     a.seq_of_token = seq_of_token; a.seq_base = seq_base;
   }
   const dim3 grid((unsigned)(tiles * Hkv), 1, a.max_segs);
-  // Keys and values through LDS where the two buffers fit (head sizes up to 128), except for the
-  // wide form at about one workgroup per CU or fewer: there the waves of a workgroup have no
-  // others to fill their waits at the barriers, and fetching per wave is faster (2,048 tokens of
-  // one prompt: 77 against 93 us; with more workgroups, 8,192 tokens: 648 against 521 us).
-  // shared: 0 never, 1 by this rule, 2 wherever it fits.
-  const bool through_lds = 2 * PF_BUF <= 65536 &&
-                           (shared == 2 || (shared == 1 && (ct == 1 || tiles * Hkv * a.max_segs > 320)));
+  // Keys and values through LDS where the two buffers fit (head sizes up to 128); the caller cuts
+  // long key ranges so that there are workgroups enough for that form to pay (with one workgroup
+  // per CU its waves have no others to fill their waits at the barriers).
+  // shared: 0 never, otherwise wherever it fits.
+  const bool through_lds = 2 * PF_BUF <= 65536 && shared != 0;
   if (through_lds) {
     if (ct == 2) attn_prefill_shared_kernel<2><<<grid, dim3(256), 2 * PF_BUF, stream>>>(a);
     else attn_prefill_shared_kernel<1><<<grid, dim3(256), 2 * PF_BUF, stream>>>(a);

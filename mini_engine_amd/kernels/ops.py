@@ -260,7 +260,7 @@ class HipBackend:
         if T > num_decodes:
             _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
             Tp = T - num_decodes
-            seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq)
+            seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq, D)
             pf = torch.empty((Tp * Hq * max_segs * (D + 2),), dtype=torch.float32, device=q.device) if max_segs > 1 else None
             lib.call("me_attn_prefill", q.data_ptr() + num_decodes * q.stride(0) * es, q.stride(0),
                      out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
@@ -387,7 +387,7 @@ LIBRARY_MIN_ROWS = 4
 LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
 LIBRARY_MAX_K = 16384
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
-PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS: 0 never, 1 chosen by the launcher, 2 wherever it fits
+PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS wherever it fits (0: never)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 # The fused form evaluates the gate in every workgroup (N/16 of them), which is free while the
 # product waits for its weights but not over a long K: at 4096x12288, one row, fused 63 us against
@@ -410,23 +410,28 @@ def _scratch(num_floats: int, device) -> torch.Tensor:
     return buf
 
 
-def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int) -> tuple:
+def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D: int = 128) -> tuple:
     """(keys per segment, most segments per tile) for the prefill kernel; (0, 1): no cutting.
 
-    A step with few new tokens over a long context (a late chunk of a long prompt) gives the
-    kernel few workgroups, each walking the whole context. Cutting the key range into segments
-    run by different workgroups fills the GPU; a second kernel merges the segments' results.
-    Measured at 16x128 heads: 256 tokens over 8,192 keys 355 -> 147 us. With enough workgroups
-    already, cutting only adds the merge: 2,048 tokens over 2,048 keys 89 -> 100 us, so it is
-    left whole. PREFILL_SEGMENT_KEYS forces a segment size."""
+    A tile's key range grows with its position, and a step with few new tokens over a long context
+    gives the kernel few workgroups, each walking the whole context. Cutting the ranges into
+    segments of at least 1,024 keys, run by different workgroups and merged by a second kernel,
+    evens the work out and fills the GPU: two segments for launches of 129 to 640 workgroups, as
+    many as give 768 workgroups below that. Measured at 16x128 heads (us, whole / cut): 64 tokens
+    over 32,768 keys 1406 / 99, 1,024 over 4,096 136 / 97, 2,048 over 8,192 333 / 237, 4,096
+    tokens of one prompt 179 / 153; 2,048 tokens of one prompt gain nothing (the merge costs what
+    the balance wins). PREFILL_SEGMENT_KEYS forces a size."""
     span = min(max_context, window + 256) if window else max_context
     if PREFILL_SEGMENT_KEYS is not None:
         seg = PREFILL_SEGMENT_KEYS
         return (seg, -(-span // seg) + 1) if seg > 0 and span > seg else (0, 1)
     workgroups = max(1, num_tokens * Hq // (128 if num_tokens * Hq >= 32768 else 64))
-    if workgroups >= 192 or span < 1024:
+    segs = (2 if workgroups <= 640 else 1) if workgroups > 128 else -(-768 // workgroups)
+    segs = min(segs, span // 1024)
+    # the partial results are float32 [tokens, heads, segments + 1, D + 2]: keep them under 256 MB
+    segs = min(segs, (1 << 28) // (num_tokens * Hq * (D + 2) * 4) - 1)
+    if segs <= 1:
         return 0, 1
-    segs = min(-(-512 // workgroups), span // 256)
     seg = -(-(-(-span // segs)) // 32) * 32
     return seg, -(-span // seg) + 1
 
