@@ -576,39 +576,49 @@ struct StagedPages {   // table entries as loaded, for the block after the stage
   int k[PF_PIECES], v[PF_PIECES];
 };
 
+// INSIDE: every key of the block lies before the context length and no page of the sequence has
+// been given back (no window), so nothing has to be tested, clamped or zeroed.
+template <bool INSIDE>
 __device__ __forceinline__ void pf_lookup(const AttnArgs& a, const int32_t* __restrict__ bt, int t0, int L,
                                           int lo_min, int tid, StagedPages& pg) {
 #pragma unroll
   for (int j = 0; j < PF_PIECES; ++j) {
     const int p = tid + 256 * j;
+    const bool in = p < 4 * HD;
     const int key = t0 + p / (HD / 8);                 // a key row
-    const bool kok = p < 4 * HD && key < L && key >= (lo_min & ~7);
+    const bool kok = in && (INSIDE || (key < L && key >= (lo_min & ~7)));
     pg.k[j] = bt[kok ? key >> a.page_shift : 0];
     const int key0 = t0 + 8 * (p & 3);                 // a group of 8 keys of one channel
-    const bool vok = p < 4 * HD && key0 < L && key0 + 7 >= lo_min;
+    const bool vok = in && (INSIDE || (key0 < L && key0 + 7 >= lo_min));
     pg.v[j] = bt[vok ? key0 >> a.page_shift : 0];
   }
 }
 
+template <bool INSIDE>
 __device__ __forceinline__ void pf_fetch(const AttnArgs& a, const StagedPages& pg, int kvh, int t0, int L,
                                          int lo_min, int tid, StagedBlock& st) {
+  const int64_t page_stride = (int64_t)a.Hkv * a.page * HD;      // elements per page, keys and values alike
 #pragma unroll
   for (int j = 0; j < PF_PIECES; ++j) {
     const int p = tid + 256 * j;
+    const bool in = p < 4 * HD;
     const int row = p / (HD / 8), ch = p - row * (HD / 8);
     const int key = t0 + row;
-    const bool kok = p < 4 * HD && key < L && key >= (lo_min & ~7) && pg.k[j] >= 0;
+    const bool kok = in && (INSIDE || (key < L && key >= (lo_min & ~7) && pg.k[j] >= 0));
     st.kok[j] = kok;
-    const bf16_t* kp = a.k_cache + (((int64_t)(kok ? pg.k[j] : 0) * a.Hkv + kvh) * a.page + (kok ? key & (a.page - 1) : 0)) * HD + 8 * ch;
+    const bf16_t* kp = a.k_cache + (int64_t)(kok ? pg.k[j] : 0) * page_stride +
+                       ((kvh * a.page + (kok ? key & (a.page - 1) : 0)) * HD + 8 * ch);
     st.k[j] = ld8(kp);
-    const int d = p >> 2, key0 = t0 + 8 * (p & 3);
-    const bool vok = p < 4 * HD && key0 < L && key0 + 7 >= lo_min && pg.v[j] >= 0;
-    st.vkeys[j] = vok ? L - key0 : 0;
-    const bf16_t* vp = a.v_cache + (((int64_t)(vok ? pg.v[j] : 0) * a.Hkv + kvh) * HD + (p < 4 * HD ? d : 0)) * a.page + (vok ? key0 & (a.page - 1) : 0);
+    const int d = in ? p >> 2 : 0, key0 = t0 + 8 * (p & 3);
+    const bool vok = in && (INSIDE || (key0 < L && key0 + 7 >= lo_min && pg.v[j] >= 0));
+    st.vkeys[j] = INSIDE ? 8 : (vok ? L - key0 : 0);
+    const bf16_t* vp = a.v_cache + (int64_t)(vok ? pg.v[j] : 0) * page_stride +
+                       ((kvh * HD + d) * a.page + (vok ? key0 & (a.page - 1) : 0));
     st.v[j] = ld8(vp);
   }
 }
 
+template <bool INSIDE>
 __device__ __forceinline__ void pf_commit(const StagedBlock& st, int tid, unsigned char* buf) {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   const bf16x8 z = zero8();
@@ -618,11 +628,13 @@ __device__ __forceinline__ void pf_commit(const StagedBlock& st, int tid, unsign
     if (p < 4 * HD) {
       const int row = p / (HD / 8), ch = p - row * (HD / 8);
       const int lrow = ((row >> 2) & 1) * 16 + ((row & 3) | ((row >> 3) << 2));
-      *reinterpret_cast<bf16x8*>(buf + lrow * PF_KROW + 16 * ch) = st.kok[j] ? st.k[j] : z;
+      *reinterpret_cast<bf16x8*>(buf + lrow * PF_KROW + 16 * ch) = (INSIDE || st.kok[j]) ? st.k[j] : z;
       u32x4 w = __builtin_bit_cast(u32x4, st.v[j]);
-      const int nv = st.vkeys[j];
+      if (!INSIDE) {
+        const int nv = st.vkeys[j];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) w[i] &= (2 * i < nv ? 0x0000ffffu : 0u) | (2 * i + 1 < nv ? 0xffff0000u : 0u);
+        for (int i = 0; i < 4; ++i) w[i] &= (2 * i < nv ? 0x0000ffffu : 0u) | (2 * i + 1 < nv ? 0xffff0000u : 0u);
+      }
       *reinterpret_cast<u32x4*>(buf + 32 * PF_KROW + (p >> 2) * PF_VROW + 16 * (p & 3)) = w;
     }
   }
@@ -700,15 +712,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     StagedBlock stg;
     StagedPages pg;
     pf_barrier();                                    // the round before has finished with both buffers
-    pf_lookup(a, bt, t0, L, tile_lo, tid, pg);
-    pf_fetch(a, pg, kvh, t0, L, tile_lo, tid, stg);
-    pf_lookup(a, bt, t0 + 32, L, tile_lo, tid, pg);
-    pf_commit(stg, tid, pf_lds);
+    pf_lookup<false>(a, bt, t0, L, tile_lo, tid, pg);
+    pf_fetch<false>(a, pg, kvh, t0, L, tile_lo, tid, stg);
+    pf_lookup<false>(a, bt, t0 + 32, L, tile_lo, tid, pg);
+    pf_commit<false>(stg, tid, pf_lds);
     int cur = 0;
     while (true) {
       pf_barrier();                                  // block t0 is in buffer cur
-      pf_fetch(a, pg, kvh, t0 + 32, L, tile_lo, tid, stg);      // the next block, into registers
-      pf_lookup(a, bt, t0 + 64, L, tile_lo, tid, pg);
+      // the next block, into registers; the page ids of the one after it
+      const bool inside1 = a.window == 0 && t0 + 64 <= L, inside2 = a.window == 0 && t0 + 96 <= L;
+      if (inside1) pf_fetch<true>(a, pg, kvh, t0 + 32, L, tile_lo, tid, stg);
+      else pf_fetch<false>(a, pg, kvh, t0 + 32, L, tile_lo, tid, stg);
+      if (inside2) pf_lookup<true>(a, bt, t0 + 64, L, tile_lo, tid, pg);
+      else pf_lookup<false>(a, bt, t0 + 64, L, tile_lo, tid, pg);
       const unsigned char* kb = pf_lds + cur * PF_BUF;
       const unsigned char* vb = kb + 32 * PF_KROW;
       const bool full = t0 <= full_hi && t0 >= full_lo;
@@ -745,7 +761,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int ct = 0; ct < CT; ++ct)
           acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct], acc[ct][dt], 0, 0, 0);
       }
-      pf_commit(stg, tid, pf_lds + (cur ^ 1) * PF_BUF);
+      if (inside1) pf_commit<true>(stg, tid, pf_lds + (cur ^ 1) * PF_BUF);
+      else pf_commit<false>(stg, tid, pf_lds + (cur ^ 1) * PF_BUF);
       cur ^= 1;
       t0 += 32;
       if (t0 > last) break;
