@@ -25,6 +25,11 @@ def test_prefill_segments_cover_the_span_and_hold_1024_keys_or_more():
 
 def test_ksplit_keeps_256_of_k_per_split_and_fills_the_gpu():
     assert ops.choose_ksplit(8, 4096, 1024) == 1                       # 256 feature tiles already
+    assert ops.choose_ksplit(8, 4096, 12288) == 1                      # 256 tiles over a long K: even, left whole
+    assert ops.choose_ksplit(1, 5120, 8192) == 4                       # 320 tiles load the compute units unevenly
+    assert ops.choose_ksplit(8, 5120, 25600) == 4
+    assert ops.choose_ksplit(64, 5120, 25600) == 1                     # many rows: left to the library
+    assert ops.choose_ksplit(8, 6144, 1024) == 1                       # uneven but short: left whole
     for M, N, K in ((8, 1024, 2048), (1, 1024, 3072), (16, 80, 224), (8, 1024, 256)):
         ks = ops.choose_ksplit(M, N, K)
         assert 1 <= ks <= 8 and (ks == 1 or K // ks >= 256)
