@@ -336,6 +336,14 @@ def test_linear_partials_are_used_where_tiles_are_few():
     w = torch.randn(1024, 3072, device=DEV).bfloat16()
     assert hip().linear(x, w, None, allow_partials=True).dim() == 3
     assert hip().linear(x, torch.randn(9000, 3072, device=DEV).bfloat16(), None, allow_partials=True).dim() == 2
+    # 320 feature tiles over a long K: four splits, so that the compute units are evenly loaded; the ring
+    # path with its fetches past the end (12.5 steps of 128 per split, K not a multiple of 128)
+    for M, N, K in ((3, 5120, 6408), (16, 5104, 4096)):
+        x = torch.randn(M, K, device=DEV).bfloat16()
+        w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+        parts = hip().linear(x, w, None, allow_partials=True)
+        assert parts.shape == (4, M, N) and parts.dtype == torch.float32
+        close(parts.sum(0), x.double() @ w.double().t(), 2e-5)
 
 
 @pytest.mark.parametrize("M,N,K", [(200, 384, 80), (2048, 1024, 1024), (65, 100, 200), (70, 96, 44)])
