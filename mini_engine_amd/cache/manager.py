@@ -101,6 +101,8 @@ class CacheManager:
         self.held: dict = {}
         self.prefix_caching = bool(enable_prefix_caching and num_state_slots == 0
                                    and all(w is None for w in windows) and len(windows) >= 1)
+        self._any_window = any(w is not None for w in windows)
+        self.epoch = 0          # counts free() calls: while it stands still no request's pages have changed hands
 
     # -- queries ---------------------------------------------------------------------------
     @property
@@ -204,6 +206,14 @@ class CacheManager:
         (reference engine/block_manager.py:80-100)."""
         ps = self.page_size
         held = self.held.get(req)
+        if held is not None and hit is None and not self._any_window:
+            # the common call of a decode step: the new token's page is held already
+            total = -(-(num_computed + num_new) // ps)
+            for table in held.tables:
+                if len(table) < total:
+                    break
+            else:
+                return True
         new_req = held is None
         nhit = hit.num_pages if hit else 0
         if nhit:
@@ -246,6 +256,7 @@ class CacheManager:
         pages are recycled before its first (which are the likeliest prefix hits), and its
         state slot (reference engine/block_manager.py:115-123)."""
         held = self.held.pop(req)
+        self.epoch += 1
         for gi, g in enumerate(self.groups):
             for page in reversed(held.tables[gi]):
                 if page != -1:

@@ -12,6 +12,9 @@ mechanism differs. Nothing is cleared with memset nodes inside the graph.
 """
 from __future__ import annotations
 
+import gc
+import weakref
+
 import numpy as np
 import torch
 
@@ -50,6 +53,9 @@ class _Captured:
             self.put(f"bt{g}", -1)
         self.row_req = [None] * B                            # which request's table a row holds
         self.row_len = [[0] * B for _ in range(self.G)]      # how many of its entries are written
+        self.row_tab = [[None] * B for _ in range(self.G)]   # the manager's table they were copied from
+        self.last_starts = None                              # positions of the step before, or None
+        self.last_epoch = -1                                 # the cache manager's epoch at that step
         self.on_gpu = runner.device.type == "cuda"
         self.pinned = [torch.empty(n, dtype=torch.int32, pin_memory=self.on_gpu) for _ in range(2)]
         self.events = [None, None]
@@ -93,11 +99,12 @@ class DecodeGraphs:
     def __init__(self, runner, max_bucket: int = 256, capture: bool = True):
         """capture=False runs the padded, fixed-layout step eagerly every time (no graph): the same
         metadata path without the capture, for machines without a GPU."""
-        self.runner = runner
-        self.max_bucket = max_bucket
+        self.runner = weakref.proxy(runner)      # the runner owns this object: no cycle, so that an engine that
+        self.max_bucket = max_bucket             # goes out of use is freed at once, not by a later collection
         self.capture = capture
         self.captured: dict = {}
         self.replays = 0
+        self.advances = 0        # of those, steps whose tables and slots were carried on from the step before
 
     def eligible(self, entries) -> bool:
         r = self.runner
@@ -126,6 +133,71 @@ class DecodeGraphs:
             raise ValueError(f"token id outside 0..{r.vocab_size - 1}")
         cap.put("tokens", tok); cap.put("positions", pos); cap.put("context_lens", ctx)
         cap.put("first_chunk", (pos == 0) & (ctx > 0))
+        reqs = [e.req for e in entries]
+        continues = self._continues(cap, reqs, pos, B)
+        cap.last_starts = None                       # stays so if what follows raises
+        if continues:
+            self._advance(cap, entries, pos, B)
+            self.advances += 1
+        else:
+            self._rewrite(cap, entries, B)
+            cap.row_req[:B] = reqs
+            for j in range(B, bucket):
+                cap.row_req[j] = None
+        cap.last_starts = pos
+        cap.last_epoch = r.manager.epoch
+        cap.upload()
+        self.replays += 1
+        if not self.capture:
+            return self._forward(cap)[:B]
+        if cap.graph is None:
+            self._capture(cap)
+        cap.graph.replay()
+        return cap.logits[:B]
+
+    def _continues(self, cap: _Captured, reqs: list, pos, B: int) -> bool:
+        """Whether this step is the one before with every request one position on: the same
+        requests in the same rows, no pages given back by anyone since (a request that was
+        preempted and fed again holds other pages at the same positions), no windowed group
+        (its tables lose entries as the window moves)."""
+        m = self.runner.manager
+        if cap.last_starts is None or cap.last_epoch != m.epoch or m._any_window:
+            return False
+        bucket = cap.bucket
+        if cap.row_req[:B] != reqs or (B < bucket and cap.row_req[B] is not None):
+            return False
+        return bool(np.array_equal(pos[:B], cap.last_starts[:B] + 1))
+
+    def _advance(self, cap: _Captured, entries: list, pos, B: int) -> None:
+        """The tables and slots of a step that continues the one before: a row whose new position
+        lies in the page of its last one takes the next slot; only rows that enter a page are looked up."""
+        r = self.runner
+        ps = r.manager.page_size
+        entering = np.flatnonzero(pos[:B] % ps == 0)
+        for g in range(cap.G):
+            o, _ = cap.seg[f"slots{g}"]
+            cap.master[o:o + B] += 1
+            if entering.size:
+                ob, _ = cap.seg[f"bt{g}"]
+                bt = cap.master[ob:ob + cap.bucket * cap.MB].reshape(cap.bucket, cap.MB)
+                for j in entering.tolist():
+                    e = entries[j]
+                    t = r.manager.block_table(e.req, g)
+                    k = cap.row_len[g][j]
+                    if len(t) > k:
+                        bt[j, k:len(t)] = t[k:]
+                        cap.row_len[g][j] = len(t)
+                    page = t[e.start // ps] if e.start // ps < len(t) else -1
+                    if page < 0:
+                        raise RuntimeError(f"request {e.req!r} has no page for position {e.start} (group {g}); "
+                                           f"allocate before stepping")
+                    cap.master[o + j] = page * ps
+
+    def _rewrite(self, cap: _Captured, entries: list, B: int) -> None:
+        """The tables and slots of every row, from the cache manager's tables."""
+        r = self.runner
+        ps = r.manager.page_size
+        bucket = cap.bucket
         for g in range(cap.G):
             o, _ = cap.seg[f"bt{g}"]
             bt = cap.master[o:o + bucket * cap.MB].reshape(bucket, cap.MB)
@@ -133,9 +205,12 @@ class DecodeGraphs:
             windowed = r.manager.groups[g].window is not None
             for j, e in enumerate(entries):
                 t = r.manager.block_table(e.req, g)
-                if cap.row_req[j] != e.req or cap.row_len[g][j] > len(t) or windowed:
+                # another table than the row was copied from: another request, or the same one after it
+                # gave its pages back and was fed again (same id, same length, other pages)
+                if cap.row_tab[g][j] is not t or cap.row_len[g][j] > len(t) or windowed:
                     bt[j, :] = -1
                     cap.row_len[g][j] = 0
+                    cap.row_tab[g][j] = t
                 k = cap.row_len[g][j]
                 if len(t) > k:
                     bt[j, k:len(t)] = t[k:]
@@ -149,17 +224,8 @@ class DecodeGraphs:
                 if cap.row_req[j] is not None:
                     bt[j, :] = -1
                     cap.row_len[g][j] = 0
+                    cap.row_tab[g][j] = None
             cap.put(f"slots{g}", slots)
-        for j in range(bucket):
-            cap.row_req[j] = entries[j].req if j < B else None
-        cap.upload()
-        self.replays += 1
-        if not self.capture:
-            return self._forward(cap)[:B]
-        if cap.graph is None:
-            self._capture(cap)
-        cap.graph.replay()
-        return cap.logits[:B]
 
     def _forward(self, cap: _Captured):
         r = self.runner
@@ -172,6 +238,15 @@ class DecodeGraphs:
         self._forward(cap)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            cap.logits = self._forward(cap)
+        # No garbage collection while the stream is capturing: a collector run that finds an old
+        # engine's graphs, events or pinned buffers frees them with calls that a capturing stream
+        # refuses, and the process aborts inside a destructor. (torch collects once on entering.)
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                cap.logits = self._forward(cap)
+        finally:
+            if collecting:
+                gc.enable()
         cap.graph = graph

@@ -101,19 +101,22 @@ class LLMEngine:
         """One scheduler step. Returns (finished [(seq_id, completion ids)], prefill tokens run,
         decode requests run, ids of the requests that got a token)."""
         seqs = self.scheduler.schedule()
-        num_decode = sum(1 for s in seqs if s.num_scheduled_tokens == 1)
-        num_prefill = sum(s.num_scheduled_tokens for s in seqs if s.num_scheduled_tokens > 1)
-        entries = []
+        num_decode = num_prefill = 0
+        entries, samplers = [], []
         for s in seqs:
             a, n = s.num_computed_tokens, s.num_scheduled_tokens
-            entries.append(StepEntry(s.seq_id, s.token_ids[a:a + n], a, [n - 1] if s.samples_this_step else []))
+            if n == 1:
+                num_decode += 1
+            else:
+                num_prefill += n
+            samples = a + n == len(s.token_ids)
+            if samples:
+                samplers.append(s)
+            entries.append(StepEntry(s.seq_id, s.token_ids[a:a + n], a, [n - 1] if samples else []))
         logits = self.runner.step(entries)
-        samplers = [s for s in seqs if s.samples_this_step]
-        sampled = {}
-        if samplers:
-            tokens = self.sampler(logits, samplers)
-            sampled = {s.seq_id: t for s, t in zip(samplers, tokens)}
-        emitted = self.scheduler.postprocess(seqs, [sampled.get(s.seq_id) for s in seqs])
+        tokens = iter(self.sampler(logits, samplers) if samplers else ())
+        sampled = [next(tokens) if e.want else None for e in entries]
+        emitted = self.scheduler.postprocess(seqs, sampled)
         outputs = [(s.seq_id, s.completion_token_ids) for s in emitted if s.is_finished]
         return outputs, num_prefill, num_decode, [s.seq_id for s in emitted]
 

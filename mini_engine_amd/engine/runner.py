@@ -98,19 +98,23 @@ class ModelRunner:
         if not entries:
             return None
         ps = self.manager.page_size
-        seen = set()
+        if len({e.req for e in entries}) != len(entries):
+            seen = set()
+            for e in entries:
+                if e.req in seen:
+                    raise ValueError(f"request {e.req!r} appears twice in one step")
+                seen.add(e.req)
+        most = self.max_positions
         for e in entries:
-            if e.req in seen:
-                raise ValueError(f"request {e.req!r} appears twice in one step")
-            seen.add(e.req)
-            if not e.tokens:
+            n = len(e.tokens)
+            if n == 0:
                 raise ValueError(f"request {e.req!r} brings no tokens")
-            if e.start < 0 or e.start + len(e.tokens) > self.max_positions:
-                raise ValueError(f"request {e.req!r}: positions {e.start}..{e.start + len(e.tokens) - 1} "
-                                 f"exceed the engine's limit of {self.max_positions} tokens")
+            if e.start < 0 or e.start + n > most:
+                raise ValueError(f"request {e.req!r}: positions {e.start}..{e.start + n - 1} "
+                                 f"exceed the engine's limit of {most} tokens")
             for w in e.want:
-                if not 0 <= w < len(e.tokens):
-                    raise ValueError(f"request {e.req!r}: wanted place {w} outside its {len(e.tokens)} tokens")
+                if not 0 <= w < n:
+                    raise ValueError(f"request {e.req!r}: wanted place {w} outside its {n} tokens")
         if self.graphs is not None and self.graphs.eligible(entries):
             logits = self.graphs.step(entries)
             wanted = [i for i, e in enumerate(entries) if e.want]

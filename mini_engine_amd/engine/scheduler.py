@@ -131,19 +131,23 @@ class Scheduler:
         budget = self.max_num_batched_tokens
         scheduled, ids = [], set()
         preempted = False
-        decodes = [s for s in self.running if s.num_uncomputed_tokens == 1]
-        partials = [s for s in self.running if s.num_uncomputed_tokens > 1]
+        decodes, partials = [], []
+        for s in self.running:
+            (decodes if len(s.token_ids) - s.num_computed_tokens == 1 else partials).append(s)
+        allocate = self.manager.allocate
         for seq in decodes + partials:
             if budget == 0:
                 break
             if seq.status != SequenceStatus.RUNNING:     # preempted earlier in this loop
                 continue
-            n = self._cap(seq.num_uncomputed_tokens, budget)
-            before = self.num_preemptions
-            ok = self._allocate_or_preempt(seq, n, ids)
-            preempted |= self.num_preemptions > before
-            if not ok:
-                break
+            owed = len(seq.token_ids) - seq.num_computed_tokens
+            n = 1 if owed == 1 else self._cap(owed, budget)
+            if not allocate(seq.seq_id, seq.num_computed_tokens, n):     # pages ran out: the slow way
+                before = self.num_preemptions
+                ok = self._allocate_or_preempt(seq, n, ids)
+                preempted |= self.num_preemptions > before
+                if not ok:
+                    break
             seq.num_scheduled_tokens = n
             budget -= n
             scheduled.append(seq)
@@ -185,17 +189,20 @@ class Scheduler:
     def postprocess(self, seqs: list, token_ids: list) -> list:
         """token_ids[i] is the token sampled for seqs[i], or None if it did not sample."""
         emitted = []
+        publish = self.manager.publish_full_pages if self.manager.prefix_caching else None
         for seq, token_id in zip(seqs, token_ids):
-            sampled = seq.samples_this_step
             seq.num_computed_tokens += seq.num_scheduled_tokens
             seq.num_scheduled_tokens = 0
-            self.manager.publish_full_pages(seq.seq_id, seq.token_ids, seq.num_computed_tokens)
+            sampled = seq.num_computed_tokens == len(seq.token_ids)      # the step reached the end of what is known
+            if publish is not None:
+                publish(seq.seq_id, seq.token_ids, seq.num_computed_tokens)
             if not sampled:
                 continue
             seq.append_token(token_id)
             emitted.append(seq)
-            done = (token_id == self.eos and not seq.sampling_params.ignore_eos) or \
-                seq.num_completion_tokens == seq.sampling_params.max_tokens
+            sp = seq.sampling_params
+            done = (token_id == self.eos and not sp.ignore_eos) or \
+                len(seq.token_ids) - seq.num_prompt_tokens == sp.max_tokens
             if done:
                 seq.status = SequenceStatus.FINISHED
                 self._release(seq)

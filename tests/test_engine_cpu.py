@@ -181,6 +181,41 @@ def test_padded_decode_layout_without_capture(folders, plain_backend, name):
         assert helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]])) <= helpers.TOL_F32, r
 
 
+def test_decode_rows_follow_a_request_that_was_fed_again(folders, plain_backend):
+    """Decode steps that continue the one before carry their tables and slots on; a request that gave
+    its pages back and was fed again sits at the same positions on other pages, and must be looked up."""
+    V, page, folder = helpers.CONFIGS["A"]["vocab_size"], helpers.PAGE["A"], folders("A")
+    model = load_model(folder, "cpu", torch.float32, 512)
+    manager = CacheManager(80, page, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, torch.float32, "cpu", 512, poison_cache=True, use_graphs=True)
+    ids = {r: helpers.random_ids(40 + 4 * page + 8, V, 40 + i) for i, r in enumerate(("a", "c", "x"))}
+    d = helpers.Driver(runner, manager)
+    d.step({"a": ids["a"][:40], "c": ids["c"][:33]})
+    pos = {"a": 40, "c": 33}
+
+    def decode(n):
+        for _ in range(n):
+            d.step({r: ids[r][pos[r]:pos[r] + 1] for r in ("a", "c")})
+            for r in pos:
+                pos[r] += 1
+
+    decode(2 * page + 3)                                   # across page edges
+    carried = runner.graphs.advances
+    assert carried >= 2 * page
+    before = list(manager.block_table("c"))
+    manager.free("c"); d.fed.pop("c")
+    d.step({"x": ids["x"][:pos["c"]]}, want_all=False)     # takes the pages c gave back
+    d.step({"c": ids["c"][:pos["c"]]}, want_all=False)     # c again, whole, on other pages
+    assert manager.block_table("c") != before
+    decode(1)
+    assert runner.graphs.advances == carried               # not carried on: the tables were read again
+    decode(page + 2)
+    assert runner.graphs.advances == carried + page + 2
+    for r in ("a", "c"):
+        got = d.result(r)
+        assert helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]])) <= helpers.TOL_F32, r
+
+
 def test_toy_architecture_on_cpu(plain_backend):
     """A stateful mixer, a layer run twice, a call that reads another call's cache and an unfused
     position encoding, registered from tests/toy_arch.py, stepped through the real runner."""
