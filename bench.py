@@ -6,7 +6,9 @@ The default run has the layer sizes of Qwen3-0.6B (28 layers, hidden 1024, 16 qu
 of 128, intermediate 3072, vocabulary 151936, tied head) with seeded random weights, bfloat16, a
 batch of 8 requests each holding a 2,048-token context. A "step" is one decode step of the whole
 batch: the engine's own step function, cache manager and sampler (greedy), from token ids to the
-next token ids on the host. One JSON line is printed:
+next token ids on the host. As in LLMEngine.step, a step is launched with its input tokens still on
+the device while the host fetches the tokens of the step before (--no-run-ahead: one after the
+other); all of them reach the host inside the timed span. One JSON line is printed:
   value        decoded tokens per second at the default batch
   prefill      one 2,048-token prompt in one step: tokens/s, ms, fraction of the bf16 MFMA peak
   roofline     bytes the decode step must read (every weight once + the live requests' cache) / time
@@ -64,7 +66,7 @@ def prefill_flops(cfg, T: int) -> float:
 
 class Bench:
     def __init__(self, cfg, dtype: str, page: int, max_batch: int, context: int, gen: int, seed: int = 0,
-                 graphs: bool = True, min_pages: int = 0, max_len: int = 0):
+                 graphs: bool = True, min_pages: int = 0, max_len: int = 0, run_ahead: bool = True):
         import torch
         from mini_engine_amd.cache.manager import CacheManager
         from mini_engine_amd.engine.runner import ModelRunner
@@ -73,6 +75,7 @@ class Bench:
 
         self.torch = torch
         self.cfg, self.page, self.context, self.gen = cfg, page, context, gen
+        self.run_ahead = run_ahead
         self.dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
         self.max_len = max(context + gen + 64, max_len)
         t0 = time.time()
@@ -106,8 +109,12 @@ class Bench:
         return best
 
     def time_decode(self, batch: int, steps: int, warmup: int):
-        """`batch` requests with `context` tokens each in the cache, then warmup + steps decode steps."""
-        from mini_engine_amd.engine.runner import StepEntry
+        """`batch` requests with `context` tokens each in the cache, then warmup + steps decode steps.
+
+        With run_ahead (the engine's default way of decoding, LLMEngine.step) a step is launched with its
+        tokens still on the device and the tokens of the step before are fetched behind it; every step's
+        tokens reach the host inside the timed span, the last ones before the clock stops."""
+        from mini_engine_amd.engine.runner import PENDING, StepEntry
         torch = self.torch
         reqs = [("d", batch, i) for i in range(batch)]
         last = []
@@ -116,23 +123,39 @@ class Bench:
             last.append(int(self.runner.sample(logits, [0.0], [(0, 0)])[0]))
         pos = self.context
         temps, keys = [0.0] * batch, [(0, 0)] * batch
+        ahead = self.run_ahead and self.runner.graphs is not None and self.runner.graphs.takes(batch)
+        in_flight = None
 
         def one():
-            nonlocal last, pos
+            nonlocal last, pos, in_flight
             entries = []
             for r, tok in zip(reqs, last):
                 assert self.manager.allocate(r, pos, 1)
-                entries.append(StepEntry(r, [tok], pos, [0]))
+                entries.append(StepEntry(r, [PENDING if in_flight is not None else tok], pos, [0]))
             logits = self.runner.step(entries)
-            last = self.runner.sample(logits, temps, keys)  # token ids on the host: the step is complete
+            if not ahead:
+                last = self.runner.sample(logits, temps, keys)  # token ids on the host: the step is complete
+            else:
+                launched = self.runner.sample_async(logits, temps, keys, reqs)
+                if in_flight is not None:
+                    last = in_flight.tokens()              # the tokens of the step before, on the host
+                in_flight = launched
             pos += 1
+
+        def drain():
+            nonlocal last, in_flight
+            if in_flight is not None:
+                last = in_flight.tokens()
+                in_flight = None
 
         for _ in range(warmup):
             one()
+        drain()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
             one()
+        drain()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         ctx_mid = pos - steps / 2.0                        # mean context length over the timed steps
@@ -154,7 +177,7 @@ class Bench:
         max_tokens = [randint(100, 1024) for _ in range(num_seqs)]
         conf = SimpleNamespace(max_num_seqs=256, max_num_batched_tokens=budget, long_prefill_token_threshold=0,
                                enable_chunked_prefill=True, scheduling_policy="fcfs", eos=-1, max_model_len=max_model_len,
-                               seed=0)
+                               seed=0, run_ahead=self.run_ahead)
         llm = LLMEngine.from_parts(conf, self.model, self.manager, self.runner)
         sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
         llm.generate([[1, 2, 3]], SamplingParams(max_tokens=4), use_tqdm=False)
@@ -186,6 +209,8 @@ def main(argv=None) -> int:
     ap.add_argument("--offline", type=int, default=256,
                     help="also run the reference's offline workload with this many requests (0: skip)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
+    ap.add_argument("--no-run-ahead", action="store_true",
+                    help="fetch every decode step's tokens before the next step is launched")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -198,7 +223,8 @@ def main(argv=None) -> int:
     points = [int(p) for p in args.points.split(",") if p]
     off_pages = args.offline * -(-2048 // args.page) if args.offline else 0
     bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed,
-                  graphs=not args.no_graphs, min_pages=off_pages, max_len=2048 if args.offline else 0)
+                  graphs=not args.no_graphs, min_pages=off_pages, max_len=2048 if args.offline else 0,
+                  run_ahead=not args.no_run_ahead)
     item = 2 if args.dtype == "bfloat16" else 4
 
     T = args.prefill_tokens
@@ -234,7 +260,7 @@ def main(argv=None) -> int:
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "tied": bool(cfg.tie_word_embeddings), "page": args.page, "global_batch": args.batch,
                    "seq_len": args.context, "gen": args.gen, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs},
+                   "hip_graphs": not args.no_graphs, "run_ahead": not args.no_run_ahead and not args.no_graphs},
         "prefill": prefill, "roofline": roofline, "points": pts,
     }
     if offline is not None:

@@ -2,7 +2,7 @@
 
 Added beside the reference's fields: ``dtype`` (bfloat16 or a true float32 path),
 ``seed`` (sampling noise is a function of seed, request and output index),
-``enable_prefix_caching`` and ``use_graphs``; ``num_kvcache_blocks`` may be given
+``enable_prefix_caching``, ``use_graphs`` and ``run_ahead``; ``num_kvcache_blocks`` may be given
 (the reference always sizes the pool itself, ``engine/model_runner.py:46-48``).
 """
 from __future__ import annotations
@@ -32,6 +32,7 @@ class EngineConfig:
     seed: int = 0
     enable_prefix_caching: bool = True
     use_graphs: bool = True
+    run_ahead: bool = True                # launch the next plain decode step before this one's tokens are fetched
     model_config: object = field(default=None, repr=False)
 
     def __post_init__(self):

@@ -20,6 +20,8 @@ import torch
 
 from .context import GroupStep, StepContext
 
+PENDING = -1      # the runner's marker for a token that is still on the device (runner.PENDING)
+
 BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 CONTEXT_STEP = 1024      # the context cap of a captured graph is a multiple of this
 
@@ -106,10 +108,14 @@ class DecodeGraphs:
         self.replays = 0
         self.advances = 0        # of those, steps whose tables and slots were carried on from the step before
 
-    def eligible(self, entries) -> bool:
+    def takes(self, num_entries: int) -> bool:
+        """Whether a step of this many single-token entries goes through here."""
         r = self.runner
         return ((r.device.type == "cuda" or not self.capture) and not r.pool.has_state and bool(r.plan.group_needs)
-                and len(entries) <= self.max_bucket and all(len(e.tokens) == 1 for e in entries))
+                and num_entries <= self.max_bucket)
+
+    def eligible(self, entries) -> bool:
+        return self.takes(len(entries)) and all(len(e.tokens) == 1 for e in entries)
 
     def step(self, entries: list):
         """Logits [len(entries), vocab] for a step in which every request brings one token."""
@@ -129,6 +135,9 @@ class DecodeGraphs:
         tok[:B] = [e.tokens[0] for e in entries]
         pos[:B] = [e.start for e in entries]
         ctx[:B] = pos[:B] + 1
+        pending = np.flatnonzero(tok[:B] == PENDING)          # tokens still on the device (checked by the runner)
+        if pending.size:
+            tok[pending] = 0
         if r.vocab_size is not None and (tok.min() < 0 or tok.max() >= r.vocab_size):
             raise ValueError(f"token id outside 0..{r.vocab_size - 1}")
         cap.put("tokens", tok); cap.put("positions", pos); cap.put("context_lens", ctx)
@@ -147,6 +156,8 @@ class DecodeGraphs:
         cap.last_starts = pos
         cap.last_epoch = r.manager.epoch
         cap.upload()
+        if pending.size:
+            self._take_pending(cap, entries, pending, B)
         self.replays += 1
         if not self.capture:
             return self._forward(cap)[:B]
@@ -154,6 +165,20 @@ class DecodeGraphs:
             self._capture(cap)
         cap.graph.replay()
         return cap.logits[:B]
+
+    def _take_pending(self, cap: _Captured, entries: list, pending, B: int) -> None:
+        """Copy the tokens that the last sampling call left on the device into the step's token rows
+        (after the upload, before the replay, on the same stream)."""
+        last = self.runner.last_sampled
+        src = [last.row_of[entries[j].req] for j in pending.tolist()]
+        tokens = cap.view("tokens")
+        if pending.size == B and src == list(range(B)):
+            tokens[:B].copy_(last.out[:B])
+            return
+        dev = tokens.device
+        dst_i = torch.from_numpy(pending.astype(np.int64)).to(dev)
+        src_i = torch.tensor(src, dtype=torch.long).to(dev)
+        tokens.index_copy_(0, dst_i, last.out.index_select(0, src_i))
 
     def _continues(self, cap: _Captured, reqs: list, pos, B: int) -> bool:
         """Whether this step is the one before with every request one position on: the same

@@ -32,6 +32,14 @@ def _load_tokenizer(model_dir: str):
         return None
 
 
+class _Launched:
+    """A step that has been launched: who samples, where their tokens go, and the handle that fetches them."""
+
+    def __init__(self, samplers, index_of, handle, num_prefill, num_decode):
+        self.samplers, self.index_of, self.handle = samplers, index_of, handle
+        self.num_prefill, self.num_decode = num_prefill, num_decode
+
+
 class LLMEngine:
     def __init__(self, model: str, **kwargs):
         names = {f.name for f in fields(EngineConfig)}
@@ -54,6 +62,10 @@ class LLMEngine:
         self.tokenizer = _load_tokenizer(config.model)
         self.scheduler = Scheduler(config, self.manager)
         self.sampler = Sampler(self.runner, config.seed)
+        self.run_ahead = bool(config.run_ahead)
+        self._in_flight = None
+        self._finishing = []
+        self.steps_run_ahead = 0
 
     @classmethod
     def from_parts(cls, config, model, manager, runner, tokenizer=None):
@@ -64,6 +76,10 @@ class LLMEngine:
         self.device, self.dtype, self.tokenizer = runner.device, runner.dtype, tokenizer
         self.scheduler = Scheduler(config, manager)
         self.sampler = Sampler(runner, config.seed)
+        self.run_ahead = bool(getattr(config, "run_ahead", True))
+        self._in_flight = None
+        self._finishing = []
+        self.steps_run_ahead = 0
         return self
 
     def _size_pool(self, plan) -> int:
@@ -99,10 +115,26 @@ class LLMEngine:
 
     def step(self):
         """One scheduler step. Returns (finished [(seq_id, completion ids)], prefill tokens run,
-        decode requests run, ids of the requests that got a token)."""
+        decode requests run, ids of the requests that got a token).
+
+        With `run_ahead`, while the requests only decode, the next step is launched before this one's
+        tokens are fetched (it takes them from the device), so the GPU does not wait for the host's
+        bookkeeping. A request that samples its end token then runs one step too far; that token is dropped."""
+        if self._in_flight is None:
+            self._in_flight = self._launch()
+        current = self._in_flight
+        self._in_flight = None
+        if (self.run_ahead and current.num_prefill == 0 and self.runner.graphs is not None
+                and self.scheduler.next_step_is_plain_decoding()
+                and self.runner.graphs.takes(len(self.scheduler.running))):
+            self._in_flight = self._launch()
+            self.steps_run_ahead += 1
+        return self._settle(current)
+
+    def _launch(self):
         seqs = self.scheduler.schedule()
         num_decode = num_prefill = 0
-        entries, samplers = [], []
+        entries, index_of = [], []
         for s in seqs:
             a, n = s.num_computed_tokens, s.num_scheduled_tokens
             if n == 1:
@@ -111,17 +143,28 @@ class LLMEngine:
                 num_prefill += n
             samples = a + n == len(s.token_ids)
             if samples:
-                samplers.append(s)
+                index_of.append(a + n)
             entries.append(StepEntry(s.seq_id, s.token_ids[a:a + n], a, [n - 1] if samples else []))
         logits = self.runner.step(entries)
-        tokens = iter(self.sampler(logits, samplers) if samplers else ())
-        sampled = [next(tokens) if e.want else None for e in entries]
-        emitted = self.scheduler.postprocess(seqs, sampled)
+        samplers = [s for s, e in zip(seqs, entries) if e.want]
+        handle = self.sampler.launch(logits, samplers) if samplers else None
+        self.scheduler.advance(seqs)
+        return _Launched(samplers, index_of, handle, num_prefill, num_decode)
+
+    def _settle(self, step):
+        tokens = step.handle.tokens() if step.handle is not None else []
+        emitted = self.scheduler.settle(step.samplers, tokens, step.index_of)
+        # what finished requests hold goes back once no launched step writes to their pages any more:
+        # those of the step before this one now, this one's at once unless a step is already in flight
+        self.scheduler.release_finished(self._finishing)
+        self._finishing = step.samplers if self._in_flight is not None else []
+        if self._in_flight is None:
+            self.scheduler.release_finished(step.samplers)
         outputs = [(s.seq_id, s.completion_token_ids) for s in emitted if s.is_finished]
-        return outputs, num_prefill, num_decode, [s.seq_id for s in emitted]
+        return outputs, step.num_prefill, step.num_decode, [s.seq_id for s in emitted]
 
     def is_finished(self) -> bool:
-        return self.scheduler.is_finished()
+        return self._in_flight is None and self.scheduler.is_finished()
 
     def generate(self, prompts: list, sampling_params, use_tqdm: bool = True, priorities: list | None = None) -> list:
         """Run all prompts (strings or lists of token ids) to completion; results in submission

@@ -31,6 +31,30 @@ class StepEntry:
     want: list = field(default_factory=list)
 
 
+# A decode entry's token may be PENDING: the token that the request sampled in the runner's last
+# sample_async() call, which is still on its way to the host. The step takes it from the device,
+# so that it can be launched before the host has seen the token (decode steps that run one ahead).
+PENDING = -1
+
+
+class SampledTokens:
+    """The token ids of one sampling call, on the device until tokens() fetches them."""
+
+    def __init__(self, out: torch.Tensor, reqs: list | None, host: torch.Tensor | None = None, arrived=None):
+        self.out = out
+        self.reqs = reqs
+        self.row_of = None if reqs is None else {r: i for i, r in enumerate(reqs)}
+        self.host = host            # pinned copy, queued right behind the sampling kernel
+        self.arrived = arrived      # event behind that copy
+
+    def tokens(self) -> list:
+        """Waits for this call's tokens only, not for what was launched after it."""
+        if self.host is None:
+            return self.out.tolist()
+        self.arrived.synchronize()
+        return self.host.tolist()
+
+
 def _pad4(n: int) -> int:
     return (n + 3) & ~3
 
@@ -60,6 +84,12 @@ class ModelRunner:
         self._events = [None, None]
         self._dev = None
         self._flip = 0
+        self.last_sampled: SampledTokens | None = None
+        self._sample_host = [None, None]
+        self._sample_events = [None, None]
+        self._sample_flip = 0
+        self._token_host = [None] * 4     # pinned landing places of sampled tokens; a handle is read before 3 more calls
+        self._token_flip = 0
 
     # -- sizing ----------------------------------------------------------------------------
     @staticmethod
@@ -105,17 +135,23 @@ class ModelRunner:
                     raise ValueError(f"request {e.req!r} appears twice in one step")
                 seen.add(e.req)
         most = self.max_positions
+        graphs = self.graphs is not None and self.graphs.eligible(entries)
         for e in entries:
             n = len(e.tokens)
             if n == 0:
                 raise ValueError(f"request {e.req!r} brings no tokens")
+            if e.tokens[0] == PENDING and not (n == 1 and graphs and self.last_sampled is not None
+                                               and self.last_sampled.row_of is not None
+                                               and e.req in self.last_sampled.row_of):
+                raise ValueError(f"request {e.req!r}: a pending token needs a decode step of single tokens and "
+                                 f"the request among those of the last sample_async() call")
             if e.start < 0 or e.start + n > most:
                 raise ValueError(f"request {e.req!r}: positions {e.start}..{e.start + n - 1} "
                                  f"exceed the engine's limit of {most} tokens")
             for w in e.want:
                 if not 0 <= w < n:
                     raise ValueError(f"request {e.req!r}: wanted place {w} outside its {n} tokens")
-        if self.graphs is not None and self.graphs.eligible(entries):
+        if graphs:
             logits = self.graphs.step(entries)
             wanted = [i for i, e in enumerate(entries) if e.want]
             if not wanted:
@@ -226,9 +262,47 @@ class ModelRunner:
     @torch.inference_mode()
     def sample(self, logits: torch.Tensor, temperatures: list, keys: list) -> list:
         """Token ids for float32 logits [S, V]; keys: (k0, k1) 32-bit pairs per row."""
+        return self.sample_async(logits, temperatures, keys).tokens()
+
+    @torch.inference_mode()
+    def sample_async(self, logits: torch.Tensor, temperatures: list, keys: list, reqs: list | None = None) -> SampledTokens:
+        """The same without waiting for the result. `reqs` names the request of every row: the next
+        step may then give PENDING as the token of any of them."""
         S = logits.shape[0]
-        t = torch.tensor(temperatures, dtype=torch.float32).to(self.device, non_blocking=True)
-        k = torch.tensor(np.asarray(keys, dtype=np.uint32).astype(np.int64).reshape(S, 2) % (1 << 32),
-                         dtype=torch.int64)
-        k = torch.where(k >= (1 << 31), k - (1 << 32), k).to(torch.int32).to(self.device, non_blocking=True)
-        return ops.sample(logits, t, k).tolist()
+        if reqs is not None and len(reqs) != S:
+            raise ValueError(f"{len(reqs)} requests named for {S} rows of logits")
+        # temperatures and keys travel as one array through pinned memory: a copy from pageable memory
+        # would hold the host until the stream has run everything launched before it
+        i = self._sample_flip
+        self._sample_flip ^= 1
+        on_gpu = self.device.type == "cuda"
+        if self._sample_host[i] is None or self._sample_host[i].numel() < 3 * S:
+            self._sample_host[i] = torch.empty(max(3 * S, 768), dtype=torch.int32, pin_memory=on_gpu)
+            self._sample_events[i] = None
+        elif self._sample_events[i] is not None:
+            self._sample_events[i].synchronize()
+        a = self._sample_host[i].numpy()
+        a[:S] = np.asarray(temperatures, dtype=np.float32).view(np.int32)
+        a[S:3 * S] = np.asarray(keys, dtype=np.uint32).reshape(2 * S).view(np.int32)
+        dev = self._sample_host[i][:3 * S].to(self.device, non_blocking=True)
+        if on_gpu:
+            ev = torch.cuda.Event()
+            ev.record()
+            self._sample_events[i] = ev
+        t = dev[:S].view(torch.float32)
+        k = dev[S:].view(S, 2)
+        out = ops.sample(logits, t, k)
+        host = arrived = None
+        if on_gpu:
+            # the copy to the host is queued now, before any later step: it arrives when this call's
+            # kernels are done, whatever has been launched behind them by then
+            j = self._token_flip
+            self._token_flip = (j + 1) % len(self._token_host)
+            if self._token_host[j] is None or self._token_host[j].numel() < S:
+                self._token_host[j] = torch.empty(max(S, 256), dtype=torch.int32, pin_memory=True)
+            host = self._token_host[j][:S]
+            host.copy_(out, non_blocking=True)
+            arrived = torch.cuda.Event()
+            arrived.record()
+        self.last_sampled = SampledTokens(out, list(reqs) if reqs is not None else None, host, arrived)
+        return self.last_sampled

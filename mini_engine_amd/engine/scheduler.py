@@ -36,6 +36,18 @@ class Scheduler:
     def is_finished(self) -> bool:
         return not self.waiting and not self.running
 
+    def next_step_is_plain_decoding(self) -> bool:
+        """Whether the next schedule() can only be: every running request decodes one token, nobody
+        waits, and pages cannot run out (one new page per request at most). Such a step needs no
+        token value and no request's pages back, so it may be launched before the step in flight
+        has delivered its tokens."""
+        if self.waiting or not self.running or len(self.running) > self.max_num_batched_tokens:
+            return False
+        need = len(self.running)
+        if any(self.manager.num_free_pages(g) < need for g in range(self.manager.num_groups)):
+            return False
+        return all(len(s.token_ids) - s.num_computed_tokens == 1 for s in self.running)
+
     # -- admission ---------------------------------------------------------------------------
     def add(self, seq: Sequence) -> None:
         total = seq.num_prompt_tokens + seq.sampling_params.max_tokens
@@ -186,25 +198,63 @@ class Scheduler:
         return scheduled
 
     # -- after the step ----------------------------------------------------------------------
-    def postprocess(self, seqs: list, token_ids: list) -> list:
-        """token_ids[i] is the token sampled for seqs[i], or None if it did not sample."""
-        emitted = []
+    PLACEHOLDER = -1       # stands in a request's tokens for a sampled token that has not reached the host yet
+
+    def advance(self, seqs: list) -> list:
+        """Bookkeeping of a step that has been launched, before its tokens are known: the scheduled
+        tokens count as computed; a request whose step reached the end of what is known gets a
+        placeholder for the token being sampled, and leaves `running` if that token is its last by
+        max_tokens. Returns the requests that sample, in order."""
+        samplers = []
         publish = self.manager.publish_full_pages if self.manager.prefix_caching else None
-        for seq, token_id in zip(seqs, token_ids):
+        for seq in seqs:
             seq.num_computed_tokens += seq.num_scheduled_tokens
             seq.num_scheduled_tokens = 0
-            sampled = seq.num_computed_tokens == len(seq.token_ids)      # the step reached the end of what is known
-            if publish is not None:
-                publish(seq.seq_id, seq.token_ids, seq.num_computed_tokens)
-            if not sampled:
+            if publish is not None:                      # pages whose tokens are all computed and all known
+                known = len(seq.token_ids) - (seq.token_ids[-1] == self.PLACEHOLDER)
+                publish(seq.seq_id, seq.token_ids, min(seq.num_computed_tokens, known))
+            if seq.num_computed_tokens != len(seq.token_ids):
                 continue
-            seq.append_token(token_id)
-            emitted.append(seq)
-            sp = seq.sampling_params
-            done = (token_id == self.eos and not sp.ignore_eos) or \
-                len(seq.token_ids) - seq.num_prompt_tokens == sp.max_tokens
-            if done:
+            seq.token_ids.append(self.PLACEHOLDER)
+            samplers.append(seq)
+            if len(seq.token_ids) - seq.num_prompt_tokens == seq.sampling_params.max_tokens:
                 seq.status = SequenceStatus.FINISHED
+                self.running.remove(seq)            # its pages are given back when its token is settled
+        return samplers
+
+    def settle(self, samplers: list, token_ids: list, index_of: list) -> list:
+        """The sampled tokens have arrived: index_of[i] is where samplers[i]'s placeholder stands.
+        Puts them in, publishes full pages, finishes on the end token and frees what finished
+        requests hold. A request that an earlier token already finished (it ran one step ahead of
+        its end token) is skipped. Returns the requests that got a token."""
+        emitted = []
+        publish = self.manager.publish_full_pages if self.manager.prefix_caching else None
+        for seq, token_id, at in zip(samplers, token_ids, index_of):
+            if at >= len(seq.token_ids):                 # cut off behind its end token: this token is not wanted
+                continue
+            seq.token_ids[at] = int(token_id)
+            emitted.append(seq)
+            if publish is not None and self.manager.holds(seq.seq_id):
+                publish(seq.seq_id, seq.token_ids, min(seq.num_computed_tokens, at + 1))
+            if token_id == self.eos and not seq.sampling_params.ignore_eos:
+                del seq.token_ids[at + 1:]               # a placeholder of a step that ran ahead
+                if seq.status != SequenceStatus.FINISHED:
+                    seq.status = SequenceStatus.FINISHED
+                    self.running.remove(seq)
+        return emitted
+
+    def release_finished(self, seqs: list) -> None:
+        """Give back what finished requests among `seqs` hold (once no step that writes to their pages is in flight)."""
+        for seq in seqs:
+            if seq.status == SequenceStatus.FINISHED and self.manager.holds(seq.seq_id):
                 self._release(seq)
-                self.running.remove(seq)
+
+    def postprocess(self, seqs: list, token_ids: list) -> list:
+        """token_ids[i] is the token sampled for seqs[i], or None if it did not sample."""
+        at = {id(s): len(s.token_ids) for s in seqs}
+        samplers = self.advance(seqs)
+        wanted = {id(s) for s in samplers}
+        tokens = [t for s, t in zip(seqs, token_ids) if id(s) in wanted]
+        emitted = self.settle(samplers, tokens, [at[id(s)] for s in samplers])
+        self.release_finished(samplers)
         return emitted

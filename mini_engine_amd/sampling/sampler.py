@@ -33,7 +33,12 @@ class Sampler:
     def __call__(self, logits, seqs: list) -> list:
         """One token per row of float32 logits [S, V]; seqs[s] gives temperature, seed, identity
         and how many tokens the request has generated so far."""
+        return self.launch(logits, seqs).tokens()
+
+    def launch(self, logits, seqs: list):
+        """The same, not waiting for the tokens: returns the runner's handle, whose tokens() fetches
+        them. The next decode step of these requests may be started before that."""
         temps = [s.sampling_params.temperature for s in seqs]
         keys = [row_key(self.seed if s.sampling_params.seed is None else s.sampling_params.seed,
                         s.sample_stream, s.num_completion_tokens) for s in seqs]
-        return self.runner.sample(logits, temps, keys)
+        return self.runner.sample_async(logits, temps, keys, [s.seq_id for s in seqs])

@@ -104,6 +104,32 @@ def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(fold
     assert [o["token_ids"] for o in other_seed.generate(prompts, sp, use_tqdm=False)] != out_together
 
 
+def test_running_one_step_ahead_changes_no_token(folders, plain_backend):
+    """Decode steps launched before the step in flight has delivered its tokens: the same tokens as
+    step by step, for greedy and sampled requests, with requests that end by max_tokens and by the
+    end token at different times (a request that samples its end token has already run one step too
+    far; that token is dropped), with and without prefix caching."""
+    from mini_engine_amd import SamplingParams
+    folder = folders("A")
+    prompts = [helpers.random_ids(n, 256, 700 + n) for n in (3, 18, 33, 47)]
+    sps = [SamplingParams(temperature=t, max_tokens=m) for t, m in ((0, 9), (0.7, 30), (0, 22), (0.9, 14))]
+    kw = dict(kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=8, max_num_batched_tokens=64, max_model_len=128, seed=5)
+    free_run = [o["token_ids"] for o in _llm(folder, run_ahead=False, eos=-2, **kw).generate(prompts, sps, use_tqdm=False)]
+    assert [len(o) for o in free_run] == [9, 30, 22, 14]
+    eos = free_run[1][11]                                     # request 1 meets its end token in mid-flight
+    want = [o[:o.index(eos) + 1] if eos in o else o for o in free_run]
+    assert len(want[1]) < 30
+    for caching in (False, True):
+        plain = _llm(folder, run_ahead=False, eos=eos, enable_prefix_caching=caching, **kw)
+        assert [o["token_ids"] for o in plain.generate(prompts, sps, use_tqdm=False)] == want
+        assert plain.steps_run_ahead == 0
+        ahead = _llm(folder, run_ahead=True, eos=eos, enable_prefix_caching=caching, **kw)
+        assert [o["token_ids"] for o in ahead.generate(prompts, sps, use_tqdm=False)] == want
+        assert ahead.steps_run_ahead >= 15
+        ahead.manager.check_invariants()
+        assert ahead.manager.num_free_pages() == 40 and not ahead.manager.held
+
+
 def test_prefix_hits_give_the_same_tokens(folders, plain_backend):
     from mini_engine_amd import SamplingParams
     folder = folders("A")
