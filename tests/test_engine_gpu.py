@@ -107,6 +107,28 @@ def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(fold
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_one_step_ahead_changes_no_token(folders, dtype):
+    """Decode steps launched with their tokens still on the device (taken from the sampling kernel's
+    output between the metadata upload and the graph's replay) give the tokens of steps taken one
+    after the other: greedy and sampled requests, ends by max_tokens and by the end token."""
+    from mini_engine_amd import SamplingParams
+    folder = folders("A")
+    prompts = [helpers.random_ids(n, 256, 700 + n) for n in (3, 18, 33, 47)]
+    sps = [SamplingParams(temperature=t, max_tokens=m) for t, m in ((0, 9), (0.7, 30), (0, 22), (0.9, 14))]
+    kw = dict(kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=8, max_num_batched_tokens=64, max_model_len=128, seed=5)
+    free_run = [o["token_ids"] for o in _llm(folder, dtype, run_ahead=False, eos=-2, **kw).generate(prompts, sps, use_tqdm=False)]
+    eos = free_run[1][11]
+    one_by_one = _llm(folder, dtype, run_ahead=False, eos=eos, **kw)
+    want = [o["token_ids"] for o in one_by_one.generate(prompts, sps, use_tqdm=False)]
+    assert want == [o[:o.index(eos) + 1] if eos in o else o for o in free_run] and len(want[1]) < 30
+    ahead = _llm(folder, dtype, run_ahead=True, eos=eos, **kw)
+    assert [o["token_ids"] for o in ahead.generate(prompts, sps, use_tqdm=False)] == want
+    assert one_by_one.steps_run_ahead == 0 and ahead.steps_run_ahead >= 15
+    ahead.manager.check_invariants()
+    assert ahead.manager.num_free_pages() == 40 and not ahead.manager.held
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_prefix_hits_give_the_same_tokens(folders, dtype):
     """A request whose first pages were written by another request (prefix cache hit) starts its
     prompt behind them: its tokens equal those of a run without the cache."""
