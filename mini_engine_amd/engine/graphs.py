@@ -39,7 +39,7 @@ class _Captured:
         B = bucket
         self.seg, n = {}, 0
         for name, size in (("tokens", B), ("positions", B), ("seq_of_token", B), ("context_lens", B), ("cu", B + 1),
-                           ("state_slots", B), ("first_chunk", B), ("rows", B)):
+                           ("state_slots", B), ("first_chunk", B), ("rows", B), ("take", B)):
             self.seg[name] = (n, size)
             n += _pad4(size)
         for g in range(self.G):
@@ -138,6 +138,10 @@ class DecodeGraphs:
         pending = np.flatnonzero(tok[:B] == PENDING)          # tokens still on the device (checked by the runner)
         if pending.size:
             tok[pending] = 0
+            row_of = r.last_sampled.row_of
+            take = np.full(bucket, -1, dtype=np.int64)       # per row: the row of the last sampling call that holds its token
+            take[pending] = [row_of[entries[j].req] for j in pending.tolist()]
+            cap.put("take", take)
         if r.vocab_size is not None and (tok.min() < 0 or tok.max() >= r.vocab_size):
             raise ValueError(f"token id outside 0..{r.vocab_size - 1}")
         cap.put("tokens", tok); cap.put("positions", pos); cap.put("context_lens", ctx)
@@ -157,7 +161,7 @@ class DecodeGraphs:
         cap.last_epoch = r.manager.epoch
         cap.upload()
         if pending.size:
-            self._take_pending(cap, entries, pending, B)
+            self._take_pending(cap, take, B)
         self.replays += 1
         if not self.capture:
             return self._forward(cap)[:B]
@@ -166,19 +170,17 @@ class DecodeGraphs:
         cap.graph.replay()
         return cap.logits[:B]
 
-    def _take_pending(self, cap: _Captured, entries: list, pending, B: int) -> None:
+    def _take_pending(self, cap: _Captured, take, B: int) -> None:
         """Copy the tokens that the last sampling call left on the device into the step's token rows
-        (after the upload, before the replay, on the same stream)."""
-        last = self.runner.last_sampled
-        src = [last.row_of[entries[j].req] for j in pending.tolist()]
+        (after the upload, before the replay, on the same stream). `take` went up with the metadata."""
+        out = self.runner.last_sampled.out
         tokens = cap.view("tokens")
-        if pending.size == B and src == list(range(B)):
-            tokens[:B].copy_(last.out[:B])
+        if out.numel() == B and np.array_equal(take[:B], np.arange(B)):
+            tokens[:B].copy_(out)
             return
-        dev = tokens.device
-        dst_i = torch.from_numpy(pending.astype(np.int64)).to(dev)
-        src_i = torch.tensor(src, dtype=torch.long).to(dev)
-        tokens.index_copy_(0, dst_i, last.out.index_select(0, src_i))
+        t = cap.view("take")[:B].long()
+        picked = out.index_select(0, t.clamp(min=0)).to(tokens.dtype)
+        tokens[:B].copy_(torch.where(t >= 0, picked, tokens[:B]))
 
     def _continues(self, cap: _Captured, reqs: list, pos, B: int) -> bool:
         """Whether this step is the one before with every request one position on: the same
