@@ -40,15 +40,16 @@ class _Lib:
         self.path = path
         self.cdll = ctypes.CDLL(path)
         self.cdll.me_last_error.restype = c_char_p
+        self.fns = {}
         for name, argtypes in protos.items():
             fn = getattr(self.cdll, name)
             fn.argtypes = argtypes
             fn.restype = c_int
+            self.fns[name] = fn
         self.protos = protos
 
     def call(self, name: str, *args):
-        rc = getattr(self.cdll, name)(*args)
-        if rc != 0:
+        if self.fns[name](*args) != 0:
             raise KernelError(f"{name}: {self.cdll.me_last_error().decode()}")
 
 
@@ -103,8 +104,19 @@ def loaded_libraries() -> list:
     return ([_core.path] if _core else []) + [l.path for l in _attn.values()]
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_device_index: int | None = None
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The handle of torch's current stream (also inside a graph capture, which runs on a stream of its
+    own). Asked for at every launch, so through the short way where torch offers it."""
+    global _device_index
+    if _raw_stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if _device_index is None:
+        _device_index = torch.cuda.current_device()
+    return _raw_stream(_device_index)
 
 
 def _ptr(t: torch.Tensor | None) -> int | None:
