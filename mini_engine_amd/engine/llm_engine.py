@@ -160,7 +160,10 @@ class LLMEngine:
         self._finishing = step.samplers if self._in_flight is not None else []
         if self._in_flight is None:
             self.scheduler.release_finished(step.samplers)
-        outputs = [(s.seq_id, s.completion_token_ids) for s in emitted if s.is_finished]
+        # a request that ends by max_tokens is marked finished when its last step is launched; it is
+        # reported when that step's token has arrived, not with the token before it
+        outputs = [(s.seq_id, s.completion_token_ids) for s in emitted
+                   if s.is_finished and s.token_ids[-1] != Scheduler.PLACEHOLDER]
         return outputs, step.num_prefill, step.num_decode, [s.seq_id for s in emitted]
 
     def is_finished(self) -> bool:

@@ -130,6 +130,47 @@ def test_running_one_step_ahead_changes_no_token(folders, plain_backend):
         assert ahead.manager.num_free_pages() == 40 and not ahead.manager.held
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_running_ahead_under_random_traffic(folders, plain_backend, seed):
+    """Requests arriving while others decode, a pool so small that requests are preempted, ends by
+    max_tokens and by the end token, greedy and sampled: with and without running one step ahead,
+    every request gets the same tokens, and nothing is left held."""
+    import random
+    from mini_engine_amd import SamplingParams
+    folder = folders("B")
+    rng = random.Random(seed)
+    n = 14
+    prompts = [helpers.random_ids(rng.randint(1, 50), 384, 100 * seed + i) for i in range(n)]
+    sps = [SamplingParams(temperature=rng.choice([0.0, 0.8]), max_tokens=rng.randint(1, 40)) for _ in range(n)]
+    arrive = sorted(rng.randint(0, 60) for _ in range(n))      # the step at which a request is added
+    kw = dict(kvcache_block_size=8, num_kvcache_blocks=rng.choice([26, 40, 80]), max_num_seqs=6,
+              max_num_batched_tokens=rng.choice([16, 48]), max_model_len=128, seed=seed,
+              enable_prefix_caching=bool(seed % 2))
+
+    def run(run_ahead, eos):
+        llm = _llm(folder, run_ahead=run_ahead, eos=eos, **kw)
+        out, ids, step, added = {}, [], 0, 0
+        while added < n or not llm.is_finished():
+            while added < n and arrive[added] <= step:
+                ids.append(llm.add_request(prompts[added], sps[added], sample_stream=added)); added += 1
+            if not llm.is_finished():
+                for sid, toks in llm.step()[0]:
+                    assert sid not in out
+                    out[sid] = toks
+            step += 1
+        llm.manager.check_invariants()
+        assert not llm.manager.held and llm.manager.num_free_pages() == kw["num_kvcache_blocks"]
+        return [out[i] for i in ids], llm
+
+    free_run, _ = run(False, -2)
+    eos = max(set(t for o in free_run for t in o[1:]), key=lambda t: sum(o.count(t) for o in free_run))
+    want, plain = run(False, eos)
+    got, ahead = run(True, eos)
+    assert got == want
+    assert any(o[-1] == eos and len(o) < sp.max_tokens for o, sp in zip(want, sps)), "no request met its end token"
+    assert plain.steps_run_ahead == 0 and ahead.steps_run_ahead > 0
+
+
 def test_prefix_hits_give_the_same_tokens(folders, plain_backend):
     from mini_engine_amd import SamplingParams
     folder = folders("A")
