@@ -63,7 +63,7 @@ def _llm(folder, **kw):
 
 
 def test_generate_greedy_matches_plain(folders, plain_backend):
-    """Tiny A as BASELINE names it: prompts 5/17/33, 8 greedy tokens each."""
+    """Tiny A: prompts of 5, 17 and 33 tokens, 8 greedy tokens each."""
     from mini_engine_amd import SamplingParams
     folder = folders("A")
     cfg, w = plain_qwen3.read_model_folder(folder, torch.float64)
@@ -77,7 +77,7 @@ def test_generate_greedy_matches_plain(folders, plain_backend):
 
 
 def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(folders, plain_backend):
-    """Tiny B as BASELINE names it: prompts 1/9/24/40/63, budget 16, temperature 0.8, 12 tokens.
+    """Tiny B: prompts of 1, 9, 24, 40 and 63 tokens, budget 16, temperature 0.8, 12 tokens.
     The same seed must give the same tokens whether requests run together under a tight budget,
     alone, or through a pool so small that requests are preempted and recomputed."""
     from mini_engine_amd import SamplingParams

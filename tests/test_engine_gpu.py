@@ -59,7 +59,7 @@ def _llm(folder, dtype, **kw):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_generate_greedy_matches_plain(folders, dtype):
-    """Tiny A as BASELINE names it (prompts 5/17/33, 8 greedy tokens) and untied tiny B. In bfloat16
+    """Tiny A (prompts of 5, 17 and 33 tokens, 8 greedy tokens each) and untied tiny B. In bfloat16
     a token may differ only where the plain model's two best logits are closer than the tolerance."""
     from mini_engine_amd import SamplingParams
     for name, page in (("A", 16), ("B", 8)):
@@ -85,7 +85,7 @@ def test_generate_greedy_matches_plain(folders, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(folders, dtype):
-    """Tiny B as BASELINE names it: prompts 1/9/24/40/63, budget 16, temperature 0.8, 12 tokens each.
+    """Tiny B: prompts of 1, 9, 24, 40 and 63 tokens, budget 16, temperature 0.8, 12 tokens each.
     In float32 the same seed gives the same tokens together, alone, and under preemption."""
     from mini_engine_amd import SamplingParams
     folder = folders("B")
