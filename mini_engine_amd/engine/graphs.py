@@ -105,6 +105,11 @@ class DecodeGraphs:
         self.max_bucket = max_bucket             # goes out of use is freed at once, not by a later collection
         self.capture = capture
         self.captured: dict = {}
+        # One memory pool for all captured graphs: they replay one after the other on one stream and a
+        # step's logits are sampled before the next graph is launched, so a graph may reuse what the
+        # others' activations and logits occupy (else every (bucket, context cap) keeps its own, and a
+        # batch of 256 holds 150 MB of logits alone per context cap).
+        self.pool = torch.cuda.graph_pool_handle() if (capture and runner.device.type == "cuda") else None
         self.replays = 0
         self.advances = 0        # of those, steps whose tables and slots were carried on from the step before
 
@@ -271,7 +276,7 @@ class DecodeGraphs:
         collecting = gc.isenabled()
         gc.disable()
         try:
-            with torch.cuda.graph(graph):
+            with torch.cuda.graph(graph, pool=self.pool):
                 cap.logits = self._forward(cap)
         finally:
             if collecting:
