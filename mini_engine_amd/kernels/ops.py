@@ -387,14 +387,15 @@ LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go t
 # kernel reads all of x, which at 8 to 16 rows is as much traffic as the weights themselves.
 # Measured with weights streamed from HBM (us, skinny / library), Qwen3-8B sizes:
 #   rows   qkv 6144x4096   o 4096x4096   gate_up 24576x4096   down 4096x12288
-#     1    15.7 / 14.3      9.5 / 15.4      45.0 / 45.5          22.0 / 22.4
-#     4    17.6 / 15.6     10.1 / 15.4      48.5 / 45.5          22.7 / 22.4
-#     8    18.9 / 14.3     10.8 / 15.6      54.3 / 45.4          25.0 / 22.4
-#    16    22.3 / 14.3     12.4 / 15.5      65.9 / 45.6          31.2 / 22.8
-# (o is below the size threshold.) At Qwen3-32B sizes, 8 rows: qkv 10240x5120 36.7 / 24.8,
-# o 5120x8192 33.4 / 20.5, gate_up 51200x5120 96.8 / 96.7, but down 5120x25600 85.3 / 136.4: the
-# library's choice for a very long K is poor, hence LIBRARY_MAX_K. All Qwen3-0.6B products favour
-# the skinny kernel (3.3-5.5 us against 7.4-12 us).
+#     1    13.1 / 14.5      8.3 / 15.4      39.3 / 45.8          21.2 / 22.6
+#     4    14.9 / 14.4      9.2 / 15.6      42.4 / 45.7          21.8 / 22.6
+#     8    15.6 / 14.4      9.1 / 15.5      47.1 / 46.3          24.7 / 22.9
+#    16    18.3 / 14.5     10.5 / 15.6      55.1 / 46.3          31.7 / 23.2
+#    32    27.2 / 15.2     15.3 / 13.1         -                 43.9 / 28.8
+# (o is below the size threshold.) At Qwen3-32B sizes, 8 rows: qkv 10240x5120 31.5 / 24.8,
+# o 5120x8192 29.2 / 20.8 (22.1 with K split in four), gate_up 51200x5120 130 / 95.3, but down
+# 5120x25600 66.8 (K split in four) / 137: the library's choice for a very long K is poor, hence
+# LIBRARY_MAX_K. All Qwen3-0.6B products favour the skinny kernel (3.3-5.5 us against 7.4-12 us).
 LIBRARY_MIN_ROWS = 4
 LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
 LIBRARY_MAX_K = 16384
