@@ -106,6 +106,45 @@ def test_generate_chunked_sampled_is_independent_of_batching_and_preemption(fold
         assert [o["token_ids"] for o in wide.generate(prompts, sp, use_tqdm=False)] == out_together
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16])
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at random (head size, heads and groups, widths and a vocabulary that are no
+    powers of two, layers, page size, window, tied or not): a whole prompt, and the same in portions of
+    changing size with the last 20 tokens one by one, in float32 and bfloat16, against the plain model."""
+    import random
+    from mini_engine_amd.config.model_config import Qwen3Config
+    from mini_engine_amd.weights.random_init import write_random_model
+    rng = random.Random(seed)
+    Hkv, L = rng.choice([1, 2, 3, 5]), rng.choice([1, 2, 3])
+    vocab, page, window = rng.choice([300, 515, 1000, 2049]), rng.choice([8, 16, 32, 64]), rng.choice([None, 24, 40])
+    cfgd = dict(architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=rng.choice([72, 88, 136, 200, 264]),
+                intermediate_size=rng.choice([120, 200, 328, 520]), num_hidden_layers=L,
+                num_attention_heads=Hkv * rng.choice([1, 2, 3, 4, 7]), num_key_value_heads=Hkv,
+                head_dim=rng.choice([16, 32, 48, 64, 128]), rms_norm_eps=rng.choice([1e-6, 1e-5]),
+                rope_theta=rng.choice([1e4, 1e6]), tie_word_embeddings=rng.random() < 0.5, max_position_embeddings=4096)
+    if window:
+        cfgd.update(use_sliding_window=True, sliding_window=window,
+                    layer_types=[rng.choice(["full_attention", "sliding_attention"]) for _ in range(L)])
+    folder = write_random_model(Qwen3Config.from_dict(cfgd), seed, str(tmp_path / "model"), torch.bfloat16)
+    n = rng.choice([70, 150, 300])
+    ids = helpers.random_ids(n, vocab, seed)
+    ref = helpers.plain_logits(folder, ids)
+    cuts, pos = [], 0
+    while pos < n - 20:
+        cuts.append(min(rng.choice([2, 5, 17, 33, 64]), n - 20 - pos)); pos += cuts[-1]
+    for dtype, tol in ((torch.float32, helpers.TOL_F32), (torch.bfloat16, helpers.TOL_BF16)):
+        model = load_model(folder, "cuda", dtype, 512)
+        manager = CacheManager(2 * (-(-n // page) + 2), page, ModelRunner.windows_of(model), enable_prefix_caching=False)
+        runner = ModelRunner(model, manager, dtype, "cuda", 512, poison_cache=True, use_graphs=True)
+        d = helpers.Driver(runner, manager)
+        d.step({"whole": ids}, end=["whole"])
+        pos = 0
+        for c in cuts + [1] * 20:
+            d.step({"cut": ids[pos:pos + c]}); pos += c
+        for r in ("whole", "cut"):
+            assert helpers.rel_err(d.result(r), ref) <= tol, (cfgd, page, n, dtype, r)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_running_one_step_ahead_changes_no_token(folders, dtype):
     """Decode steps launched with their tokens still on the device (taken from the sampling kernel's
