@@ -231,6 +231,147 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
   }
 }
 
+// ------------------------------------------------------------------ the same product for 17 to 64 tokens
+// With that many tokens the skinny kernel's token fetches (all tokens again in every workgroup of 16
+// features) outweigh its weight fetches several times. Here a workgroup owns 64 features, one tile of
+// 16 per wave, and every wave walks the whole k-range of the split; the tokens of 512 k at a time are
+// staged once per workgroup in LDS and serve all four waves, so they cost a quarter as much. Weights go
+// from memory straight into the matrix operand registers, one step ahead, as in the skinny kernel.
+// LDS layout: row m holds the chunk's 64 granules of 16 bytes; granule q lies at q ^ (m & 15) within
+// its group of 16, which spreads the 16 rows a wave reads at once over all banks without padding.
+#define ROWS_CHUNK 512                      // k per staged chunk: 4 steps of 128
+#define ROWS_GRANULES (ROWS_CHUNK / 8)
+
+template <int MT, typename TO, bool EXACT_K>
+__global__ void __launch_bounds__(256)
+gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
+                 TO* __restrict__ y, int64_t ldy, float* __restrict__ partials, int M, int N, int K,
+                 int chunks_per_split) {
+  extern __shared__ __align__(16) unsigned char rows_lds[];
+  bf16_t* xs = reinterpret_cast<bf16_t*>(rows_lds);     // [16 * MT][ROWS_CHUNK]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 64 + wave * 16;
+  const int split = blockIdx.z;
+  const int total_chunks = (K + ROWS_CHUNK - 1) / ROWS_CHUNK;
+  const int c_begin = split * chunks_per_split;
+  const int c_end = min(total_chunks, c_begin + chunks_per_split);
+  const bf16_t* wrow = w + (int64_t)(n0 + r < N ? n0 + r : 0) * ldw;
+  const bf16x8 z = gz8();
+  const int rows = min(M, 16 * MT);
+
+  auto fetch = [&](int s, bool live, bf16x8 (&a)[4]) {
+    const int kb = 128 * s + 8 * g;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = kb + 32 * j;
+      a[j] = *reinterpret_cast<const bf16x8*>(live && (EXACT_K || k < K) ? wrow + k : w);
+    }
+  };
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int s_last = min((K + 127) / 128, 4 * c_end) - 1;       // the split's last step
+  bf16x8 ring[2][4];
+  fetch(4 * c_begin, true, ring[0]);
+  pin_loads();
+
+  for (int c = c_begin; c < c_end; ++c) {
+    // the tokens of this chunk into LDS: 8 granules of a thread go out together
+    const int total = rows * ROWS_GRANULES;
+    for (int e0 = threadIdx.x; e0 < total; e0 += 256 * 8) {
+      bf16x8 v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int e = e0 + 256 * i < total ? e0 + 256 * i : e0;   // beyond the end: the first again, no branch
+        const int m = e / ROWS_GRANULES, q = e % ROWS_GRANULES;
+        const int k = ROWS_CHUNK * c + 8 * q;
+        v[i] = *reinterpret_cast<const bf16x8*>(x + (int64_t)m * ldx + ((EXACT_K || k < K) ? k : 0));
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int e = e0 + 256 * i;
+        if (e < total) {
+          const int m = e / ROWS_GRANULES, q = e % ROWS_GRANULES;
+          bf16x8 t = v[i];
+          if (!EXACT_K && ROWS_CHUNK * c + 8 * q >= K) t = z;
+          *reinterpret_cast<bf16x8*>(xs + m * ROWS_CHUNK + 8 * ((q & ~15) | ((q ^ m) & 15))) = t;
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int s = 4 * c + u;
+      fetch(s + 1, s + 1 <= s_last, ring[(u + 1) & 1]);
+      pin_loads();
+      if (s <= s_last) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bool kok = EXACT_K || 128 * s + 32 * j + 8 * g < K;
+          const bf16x8 a = kok ? ring[u & 1][j] : z;
+          const int q = 16 * u + 4 * j + g;           // granule of k = 128 s + 32 j + 8 g inside the chunk
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const int m = 16 * mt + r < rows ? 16 * mt + r : 0;
+            const bf16x8 b = *reinterpret_cast<const bf16x8*>(xs + m * ROWS_CHUNK + 8 * ((q & ~15) | ((q ^ m) & 15)));
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+          }
+        }
+      }
+    }
+    __syncthreads();      // the next chunk overwrites what the slowest wave may still read
+  }
+  // accumulator: lane (token r, g) holds features n0 + 4g + i
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + r, n = n0 + 4 * g;
+    if (m < M) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < N) {
+          if (partials) partials[((int64_t)split * M + m) * N + n + i] = acc[mt][i];
+          else y[(int64_t)m * ldy + n + i] = from_f32<TO>(acc[mt][i]);
+        }
+    }
+  }
+}
+
+extern "C" int me_gemm_rows_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
+                                 int out_dtype, float* partials, int ksplit, int M, int N, int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  ME_CHECK(M <= 64, "rows gemm: at most 64 rows (%d)", M);
+  ME_CHECK(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
+           "rows gemm: K=%d and the row strides must be multiples of 8", K);
+  ME_CHECK((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0),
+           "rows gemm: operands must be 16-byte aligned");
+  ME_CHECK(ksplit >= 1 && (ksplit == 1) == (partials == nullptr), "rows gemm: partials iff ksplit > 1");
+  const int total_chunks = (K + ROWS_CHUNK - 1) / ROWS_CHUNK;
+  const int chunks_per_split = (total_chunks + ksplit - 1) / ksplit;
+  ME_CHECK((int64_t)(ksplit - 1) * chunks_per_split < total_chunks, "rows gemm: ksplit %d leaves a split without work", ksplit);
+  const int mt = (M + 15) / 16;
+  const size_t lds = (size_t)16 * mt * ROWS_CHUNK * sizeof(bf16_t);
+  dim3 grid((N + 63) / 64, 1, ksplit), block(256);
+  const bool exact = K % 128 == 0;
+#define LAUNCH1(MTV, TO, E)                                                                                     \
+  gemm_rows_kernel<MTV, TO, E><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, \
+                                                             ldy, partials, M, N, K, chunks_per_split)
+#define LAUNCH2(MTV, TO) do { if (exact) LAUNCH1(MTV, TO, true); else LAUNCH1(MTV, TO, false); } while (0)
+#define LAUNCH(TO)                                                                             \
+  do {                                                                                         \
+    if (mt == 1) LAUNCH2(1, TO); else if (mt == 2) LAUNCH2(2, TO); else if (mt == 3) LAUNCH2(3, TO); \
+    else LAUNCH2(4, TO);                                                                       \
+  } while (0)
+  if (out_dtype == ME_F32 || partials) LAUNCH(float);
+  else if (out_dtype == ME_BF16) LAUNCH(bf16_t);
+  else ME_CHECK(false, "rows gemm: bad output dtype code %d", out_dtype);
+#undef LAUNCH
+#undef LAUNCH2
+#undef LAUNCH1
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
 // y: bf16 or float32 [M, N]; or, when ksplit > 1, `partials` float32 [ksplit, M, N] (y unused).
 extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y,
                                    int64_t ldy, int out_dtype, float* partials, int ksplit, int M, int N,

@@ -63,6 +63,7 @@ _CORE_PROTOS = {
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
+    "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
@@ -312,6 +313,12 @@ class HipBackend:
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
             return y
+        if allow_partials and out_dtype == x.dtype and rows_takes(M, N, K):
+            ksplit = rows_ksplit(K)
+            parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
+            core().call("me_gemm_rows_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
+                        ME_F32, parts.data_ptr(), ksplit, M, N, K, _stream())
+            return parts
         ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype
                                             and not library_streams_better(M, N, K)) else 1
         if ksplit > 1:
@@ -399,6 +406,7 @@ LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go t
 LIBRARY_MIN_ROWS = 4
 LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
 LIBRARY_MAX_K = 16384
+ROWS_MIN_WEIGHT = 16 * 1024 * 1024
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS wherever it fits (0: never)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
@@ -454,6 +462,33 @@ def skinny_takes(M: int, N: int, K: int) -> bool:
     """Whether the skinny kernel (without a split over K) takes an aligned bfloat16 product."""
     rows_ok = M <= SKINNY_MAX_M or (M <= SKINNY_WIDE_MAX_M and N * K <= SKINNY_WIDE_MAX_WEIGHT)
     return rows_ok and N < LIBRARY_MIN_N and not library_streams_better(M, N, K)
+
+
+def rows_takes(M: int, N: int, K: int) -> bool:
+    """Whether a product whose consumer adds float32 partial sums goes to the rows kernel (64 features per
+    workgroup, the tokens staged once per workgroup in LDS, K split over up to 8 workgroups): large
+    weights with 17 to 64 rows, where the skinny kernel reads the tokens again for every 16 features and
+    the library streams at 1.7-3.5 TB/s, and from 8 rows on over a K too long for the library.
+    Measured, us (rows kernel / best of library and skinny), weights from HBM:
+      4096 x 4096:   24 rows 10.6 / 13.2,  48 rows 13.5 / 13.6,  64 rows 14.6 / 15.0
+      4096 x 12288:  24 rows 25.0 / 26.9,  48 rows 30.2 / 33.6,  64 rows 31.7 / 37.3
+      5120 x 8192:   24 rows 23.3 / 26.0,  48 rows 28.0 / 43.1,  64 rows 33.3 / 29.2 (left to the library)
+      5120 x 25600:   8 rows 63.2 / 66.8,  32 rows 70.7 / 109,   64 rows 86.6 / 157
+      2560 x 9728:   24 rows 19.2 / 19.1,  48 rows 26.4 / 20.5 (left to the library)"""
+    if N * K < ROWS_MIN_WEIGHT or K < 4096 or K % 8 or M > 64:
+        return False
+    if M > 16:
+        return M <= 32 or K >= 12288
+    return M >= 8 and K > LIBRARY_MAX_K
+
+
+def rows_ksplit(K: int) -> int:
+    """The most splits up to 8 that leave no split without one of the K/512 chunks."""
+    chunks = -(-K // 512)
+    for ks in range(min(8, chunks), 0, -1):
+        if (ks - 1) * -(-chunks // ks) < chunks:
+            return ks
+    return 1
 
 
 def library_streams_better(M: int, N: int, K: int) -> bool:

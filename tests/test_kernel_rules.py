@@ -49,3 +49,14 @@ def test_skinny_kernel_takes_few_rows():
     assert ops.skinny_takes(64, 4096, 1024) and not ops.skinny_takes(65, 4096, 1024)
     assert not ops.skinny_takes(1, 151936, 1024)                       # the head goes to the library
     assert not ops.skinny_takes(8, 24576, 4096)
+
+
+def test_rows_kernel_takes_many_rows_over_large_weights():
+    assert ops.rows_takes(24, 4096, 4096) and not ops.rows_takes(64, 4096, 4096)     # above 32 rows only over a long K
+    assert ops.rows_takes(64, 4096, 12288) and ops.rows_takes(32, 5120, 8192) and not ops.rows_takes(64, 5120, 8192)
+    assert ops.rows_takes(8, 5120, 25600) and not ops.rows_takes(4, 5120, 25600)     # few rows: only where the library is out
+    assert not ops.rows_takes(8, 4096, 12288) and not ops.rows_takes(64, 1024, 3072) and not ops.rows_takes(65, 5120, 25600)
+    for K in (4096, 4104, 9728, 12288, 25600):
+        ks, chunks = ops.rows_ksplit(K), -(-K // 512)
+        assert 1 <= ks <= 8 and (ks - 1) * -(-chunks // ks) < chunks
+

@@ -346,6 +346,21 @@ def test_linear_partials_are_used_where_tiles_are_few():
         close(parts.sum(0), x.double() @ w.double().t(), 2e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(24, 4096, 4096), (17, 4100, 4104), (64, 1400, 12296), (33, 1368, 12288), (9, 1000, 16896)])
+def test_linear_rows_kernel(M, N, K):
+    """17 to 64 rows over large weights (and fewer over a very long K), partial sums allowed: 64 features per
+    workgroup, the tokens staged in LDS chunk by chunk; feature counts and K that are no multiples of 64, 128 or 512."""
+    from mini_engine_amd.kernels import ops
+    assert ops.rows_takes(M, N, K)
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    parts = hip().linear(x, w, None, allow_partials=True)
+    assert parts.shape == (ops.rows_ksplit(K), M, N) and parts.dtype == torch.float32
+    close(parts.sum(0), x.double() @ w.double().t(), 2e-5)
+    xs = torch.randn(M, K + 8, device=DEV).bfloat16()[:, :K]   # a row stride that is not K
+    close(hip().linear(xs, w, None, allow_partials=True).sum(0), xs.double() @ w.double().t(), 2e-5)
+
+
 @pytest.mark.parametrize("M,N,K", [(200, 384, 80), (2048, 1024, 1024), (65, 100, 200), (70, 96, 44)])
 def test_linear_large_and_odd_bf16(M, N, K):
     """Above the skinny range the library product runs; K not a multiple of 8 takes the FMA kernel."""
