@@ -242,6 +242,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
 #define ROWS_CHUNK 512                      // k per staged chunk: 4 steps of 128
 #define ROWS_GRANULES (ROWS_CHUNK / 8)
 
+// EXACT_K: K is a multiple of the chunk, so neither a step nor a staged granule lies beyond K.
 template <int MT, typename TO, bool EXACT_K>
 __global__ void __launch_bounds__(256)
 gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
@@ -352,7 +353,7 @@ extern "C" int me_gemm_rows_bf16(const void* x, int64_t ldx, const void* w, int6
   const int mt = (M + 15) / 16;
   const size_t lds = (size_t)16 * mt * ROWS_CHUNK * sizeof(bf16_t);
   dim3 grid((N + 63) / 64, 1, ksplit), block(256);
-  const bool exact = K % 128 == 0;
+  const bool exact = K % ROWS_CHUNK == 0;   // whole chunks: the staging reads no k beyond K either
 #define LAUNCH1(MTV, TO, E)                                                                                     \
   gemm_rows_kernel<MTV, TO, E><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, \
                                                              ldy, partials, M, N, K, chunks_per_split)
