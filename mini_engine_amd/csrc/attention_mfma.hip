@@ -793,12 +793,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 
 // Merge of the segments of cut tiles: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s.
-// One wave per (token, head), four to a workgroup; rows of tiles that were not cut already hold
-// their result and return.
+// Sixteen lanes per (token, head), each with HD/16 consecutive values; 16 rows to a workgroup. Rows of
+// tiles that were not cut already hold their result and return.
+#define MERGE_EPL (HD / 16)
 __global__ void __launch_bounds__(256) attn_prefill_merge_kernel(AttnArgs a, int64_t rows) {
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   if (row >= rows) return;
-  const int lane = threadIdx.x & 63;
+  const int part = threadIdx.x & 15;
   const int64_t t = row / a.Hq;
   const int hq = (int)(row - t * a.Hq);
   const int b = a.seq_of_token[t] - a.seq_base;
@@ -810,24 +811,31 @@ __global__ void __launch_bounds__(256) attn_prefill_merge_kernel(AttnArgs a, int
   float M = NEG;
   for (int s = 0; s < tr.nseg; ++s) M = fmaxf(M, p[s * (HD + 2) + HD]);
   float ls = 0.f;
-  float o[(HD + 63) / 64];
+  float o[MERGE_EPL];
 #pragma unroll
-  for (int i = 0; i < (HD + 63) / 64; ++i) o[i] = 0.f;
+  for (int i = 0; i < MERGE_EPL; ++i) o[i] = 0.f;
   for (int s = 0; s < tr.nseg; ++s) {
-    const float w = exp2f(p[s * (HD + 2) + HD] - M);
-    ls += w * p[s * (HD + 2) + HD + 1];
+    const float* ps = p + s * (HD + 2);
+    const float w = exp2f(ps[HD] - M);
+    ls += w * ps[HD + 1];
+    float v[MERGE_EPL];
+    if (MERGE_EPL % 2 == 0) {        // rows of HD + 2 floats keep 8-byte alignment only
 #pragma unroll
-    for (int i = 0; i < (HD + 63) / 64; ++i) {
-      const int d = lane + 64 * i;
-      if (d < HD) o[i] += w * p[s * (HD + 2) + d];
+      for (int i = 0; i < MERGE_EPL; i += 2) {
+        const float2 u = *reinterpret_cast<const float2*>(ps + part * MERGE_EPL + i);
+        v[i] = u.x; v[i + 1] = u.y;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < MERGE_EPL; ++i) v[i] = ps[part * MERGE_EPL + i];
     }
+#pragma unroll
+    for (int i = 0; i < MERGE_EPL; ++i) o[i] += w * v[i];
   }
   const float inv = ls > 0.f ? 1.f / ls : 0.f;
+  bf16_t* dst = a.out + t * a.out_stride + (int64_t)hq * HD + part * MERGE_EPL;
 #pragma unroll
-  for (int i = 0; i < (HD + 63) / 64; ++i) {
-    const int d = lane + 64 * i;
-    if (d < HD) a.out[t * a.out_stride + (int64_t)hq * HD + d] = static_cast<bf16_t>(o[i] * inv);
-  }
+  for (int i = 0; i < MERGE_EPL; ++i) dst[i] = static_cast<bf16_t>(o[i] * inv);
 }
 
 // =====================================================================================
@@ -1016,7 +1024,7 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   ME_LAUNCH_CHECK();
   if (a.max_segs > 1) {
     const int64_t rows = num_tokens * Hq;
-    attn_prefill_merge_kernel<<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream>>>(a, rows);
+    attn_prefill_merge_kernel<<<dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream>>>(a, rows);
     ME_LAUNCH_CHECK();
   }
   return 0;
