@@ -931,6 +931,13 @@ __global__ void __launch_bounds__(128) attn_reduce_kernel(AttnArgs a) {
   const int b = blockIdx.x, hq = blockIdx.y;
   const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_parts;
   const int P = a.num_parts;
+  // the first 16 partitions' values of this thread's channel are asked for before the weights are
+  // formed: they do not depend on them, and the two rounds of loads then overlap
+  const int d0 = threadIdx.x;
+  float first[16];
+#pragma unroll
+  for (int p = 0; p < 16; ++p)
+    first[p] = a.tmp_out[(row0 + (p < P ? p : 0)) * HD + (d0 < HD ? d0 : 0)];
   if (threadIdx.x < 64) {
     const int p = threadIdx.x;
     const float mp = p < P ? a.tmp_m[row0 + p] : NEG;
@@ -943,10 +950,16 @@ __global__ void __launch_bounds__(128) attn_reduce_kernel(AttnArgs a) {
   }
   __syncthreads();
   const float inv = inv_s;
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+  for (int d = d0; d < HD; d += blockDim.x) {
     float o = 0.f;
+    int p0 = 0;
+    if (d == d0) {                      // weights beyond P are zero
+#pragma unroll
+      for (int p = 0; p < 16; ++p) o += wgt[p] * first[p];
+      p0 = 16;
+    }
 #pragma unroll 8
-    for (int p = 0; p < P; ++p) o += wgt[p] * a.tmp_out[(row0 + p) * HD + d];
+    for (int p = p0; p < P; ++p) o += wgt[p] * a.tmp_out[(row0 + p) * HD + d];
     a.out[(int64_t)b * a.out_stride + (int64_t)hq * HD + d] = static_cast<bf16_t>(o * inv);
   }
 }
