@@ -86,6 +86,42 @@ __global__ void rms_norm_kernel(const TX* __restrict__ x, int num_partials, int6
   const int64_t t = blockIdx.x;
   const TX* xr = x + t * n;
   float ss = 0.f;
+  if (VEC && n <= (int)blockDim.x * 4) {
+    // every thread has at most one group of 4: it stays in registers, and the norm's weight is asked
+    // for together with the row, so that nothing is fetched behind the workgroup's sum
+    const int i = threadIdx.x * 4;
+    const bool on = i < n;
+    float part[RN_MAX_PARTIALS][4], r[4] = {0.f, 0.f, 0.f, 0.f}, wv[4] = {0.f, 0.f, 0.f, 0.f}, v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (on) {
+#pragma unroll
+      for (int p = 0; p < RN_MAX_PARTIALS; ++p)
+        if (p < num_partials) Vec4<TX>::load(xr + p * partial_stride + i, part[p]);
+      if (res_in) Vec4<float>::load(res_in + t * n + i, r);
+      Vec4<float>::load(w + i, wv);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = part[0][e];
+#pragma unroll
+      for (int p = 1; p < RN_MAX_PARTIALS; ++p)
+        if (p < num_partials) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += part[p][e];
+        }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] += r[e];
+        ss += v[e] * v[e];
+      }
+      if (res_out) Vec4<float>::store(res_out + t * n + i, v);
+    }
+    const float inv1 = rsqrtf(block_sum(ss, scratch) / (float)n + eps);
+    if (on) {
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = wv[e] * (v[e] * inv1);
+      Vec4<TY>::store(y + t * n + i, o);
+    }
+    return;
+  }
   if (VEC) {
     for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
       float part[RN_MAX_PARTIALS][4];
