@@ -173,13 +173,29 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, int64_t row_stride, const flo
   const bool active = head < Hq + Hkv;
   const bool is_q = head < Hq;
   T* row = qkv + t * row_stride + (int64_t)(active ? head : 0) * D;
+  // Everything this thread reads is asked for at once: the position and the slot first (the table's
+  // address hangs on the position), then the row and the norm's weight; the step is a chain of memory
+  // latencies, and each load that waits for arithmetic it does not need adds one.
+  const int pos = table ? positions[t] : 0;
+  const int slot = store ? slots[t] : 0;
+  const float* w = is_q ? q_w : k_w;
   float x1[4], x2[4];
   Quad<T>::load(row + 4 * l, x1);
   Quad<T>::load(row + half + 4 * l, x2);
+  float w1[4] = {1.f, 1.f, 1.f, 1.f}, w2[4] = {1.f, 1.f, 1.f, 1.f};
+  if (w) {
+    Quad<float>::load(w + 4 * l, w1);
+    Quad<float>::load(w + half + 4 * l, w2);
+  }
+  float c0[4] = {1.f, 0.f, 1.f, 0.f}, c1[4] = {1.f, 0.f, 1.f, 0.f};
+  if (table) {
+    const float* cs = table + ((int64_t)pos * half + 4 * l) * 2;   // (cos, sin) of 4 pairs: 8 floats
+    Quad<float>::load(cs, c0);
+    Quad<float>::load(cs + 4, c1);
+  }
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) ss += x1[i] * x1[i] + x2[i] * x2[i];
-  const float* w = is_q ? q_w : k_w;
   float inv = 1.f;
   if (w) {
 #pragma unroll
@@ -190,17 +206,10 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, int64_t row_stride, const flo
 #pragma unroll
   for (int i = 0; i < 4; ++i) { o1[i] = x1[i] * inv; o2[i] = x2[i] * inv; }
   if (w) {
-    float w1[4], w2[4];
-    Quad<float>::load(w + 4 * l, w1);
-    Quad<float>::load(w + half + 4 * l, w2);
 #pragma unroll
     for (int i = 0; i < 4; ++i) { o1[i] *= w1[i]; o2[i] *= w2[i]; }
   }
   if (table) {
-    const float* cs = table + ((int64_t)positions[t] * half + 4 * l) * 2;   // (cos, sin) of 4 pairs: 8 floats
-    float c0[4], c1[4];
-    Quad<float>::load(cs, c0);
-    Quad<float>::load(cs + 4, c1);
     const float c[4] = {c0[0], c0[2], c1[0], c1[2]}, sn[4] = {c0[1], c0[3], c1[1], c1[3]};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -212,7 +221,6 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, int64_t row_stride, const flo
   if (!active) return;
   T* dst = row;
   if (!is_q && store) {
-    const int slot = slots[t];
     if (slot < 0) return;
     const int64_t pg = slot / page, off = slot - pg * page;
     dst = k_cache + ((pg * Hkv + (head - Hq)) * (int64_t)page + off) * D;

@@ -23,7 +23,7 @@ def test_prefill_segments_cover_the_span_and_hold_1024_keys_or_more():
     assert ops.prefill_segments(1 << 20, 0, 8192, 64)[1] <= 3         # the partial results stay under 256 MB
 
 
-def test_ksplit_keeps_256_of_k_per_split_and_fills_the_gpu():
+def test_ksplit_keeps_512_of_k_per_split_and_fills_the_gpu():
     assert ops.choose_ksplit(8, 4096, 1024) == 1                       # 256 feature tiles already
     assert ops.choose_ksplit(8, 4096, 12288) == 1                      # 256 tiles over a long K: even, left whole
     assert ops.choose_ksplit(1, 5120, 8192) == 4                       # 320 tiles load the compute units unevenly
@@ -32,7 +32,7 @@ def test_ksplit_keeps_256_of_k_per_split_and_fills_the_gpu():
     assert ops.choose_ksplit(8, 6144, 1024) == 1                       # uneven but short: left whole
     for M, N, K in ((8, 1024, 2048), (1, 1024, 3072), (16, 80, 224), (8, 1024, 256)):
         ks = ops.choose_ksplit(M, N, K)
-        assert 1 <= ks <= 8 and (ks == 1 or K // ks >= 256)
+        assert 1 <= ks <= 8 and (ks == 1 or K // ks >= 512)
 
 
 def test_large_weights_with_several_rows_go_to_the_library():
