@@ -437,19 +437,28 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D:
 
     A tile's key range grows with its position, and a step with few new tokens over a long context
     gives the kernel few workgroups, each walking the whole context. Cutting the ranges into
-    segments of at least 1,024 keys, run by different workgroups and merged by a second kernel,
-    evens the work out and fills the GPU: two segments for launches of 129 to 640 workgroups, as
-    many as give 768 workgroups below that. Measured at 16x128 heads (us, whole / cut): 64 tokens
-    over 32,768 keys 1406 / 99, 1,024 over 4,096 136 / 97, 2,048 over 8,192 333 / 237, 4,096
-    tokens of one prompt 179 / 153; 2,048 tokens of one prompt gain nothing (the merge costs what
-    the balance wins). PREFILL_SEGMENT_KEYS forces a size."""
+    segments of at least 512 keys (1,024 over ranges beyond 4,096), run by different workgroups and merged by a second kernel,
+    evens the work out and fills the GPU: two segments for launches of 257 to 640 workgroups; three
+    for 129 to 256 when the ranges start short (a prompt from its beginning: tiles of 64 to all keys,
+    which thirds balance better than halves) and two when they are all long (a later portion of a
+    prompt: twice the workgroups fill the slots evenly); as many as give 768 workgroups below that.
+    Measured at 16x128 heads (us, whole / cut): 64 tokens over 32,768 keys 1406 / 99, 1,024 over 4,096
+    116 / 86, 2,048 over 8,192 333 / 237, one prompt of 4,096 tokens 166 / 135, of 2,048 86 / 56, of
+    1,536 52 / 43, of 1,024 36 / 33, 512 over 2,048 62 / 37. PREFILL_SEGMENT_KEYS forces a size."""
     span = min(max_context, window + 256) if window else max_context
     if PREFILL_SEGMENT_KEYS is not None:
         seg = PREFILL_SEGMENT_KEYS
         return (seg, -(-span // seg) + 1) if seg > 0 and span > seg else (0, 1)
     workgroups = max(1, num_tokens * Hq // (128 if num_tokens * Hq >= 32768 else 64))
-    segs = (2 if workgroups <= 640 else 1) if workgroups > 128 else -(-768 // workgroups)
-    segs = min(segs, span // 1024)
+    if workgroups > 640:
+        segs = 1
+    elif workgroups > 256:
+        segs = 2
+    elif workgroups > 128:
+        segs = 3 if 2 * (max_context - num_tokens) < span else 2
+    else:
+        segs = -(-768 // workgroups)
+    segs = min(segs, span // (512 if span <= 4096 else 1024))      # segments of 512 keys or more, 1,024 over long ranges
     # the partial results are float32 [tokens, heads, segments + 1, D + 2]: keep them under 256 MB
     segs = min(segs, (1 << 28) // (num_tokens * Hq * (D + 2) * 4) - 1)
     if segs <= 1:

@@ -10,15 +10,18 @@ def test_decode_partitions_cover_the_context():
         assert part * parts >= ctx and part * (parts - 1) < ctx
 
 
-def test_prefill_segments_cover_the_span_and_hold_1024_keys_or_more():
+def test_prefill_segments_cover_the_span_and_hold_512_keys_or_more():
     assert ops.prefill_segments(8192, 0, 8192, 16) == (0, 1)          # workgroups enough: left whole
-    assert ops.prefill_segments(1900, 0, 4, 16) == (0, 1)             # short span: left whole
+    assert ops.prefill_segments(900, 0, 4, 16) == (0, 1)              # short span: left whole
     for ctx, window, tokens, heads in ((8192, 0, 256, 16), (32768, 0, 64, 16), (40000, 0, 2, 32), (5000, 3000, 8, 4),
-                                       (2048, 0, 2048, 16), (4096, 0, 4096, 16)):
+                                       (2048, 0, 2048, 16), (4096, 0, 4096, 16), (1900, 0, 4, 16), (1536, 0, 1536, 16),
+                                       (4096, 0, 1024, 16), (2048, 0, 512, 16)):
         seg, most = ops.prefill_segments(ctx, window, tokens, heads)
         span = min(ctx, window + 256) if window else ctx
-        assert seg >= 1024 and seg % 32 == 0 and (most - 1) * seg >= span
+        assert seg >= (512 if span <= 4096 else 1024) and seg % 32 == 0 and (most - 1) * seg >= span
         assert tokens * heads * most * 130 * 4 <= 1 << 28
+    assert ops.prefill_segments(2048, 0, 2048, 16)[0] == 704          # a prompt from its beginning: thirds
+    assert ops.prefill_segments(4096, 0, 1024, 16)[0] == 2048         # a later portion, all ranges long: halves
     assert ops.prefill_segments(8192, 512, 64, 16) == (0, 1)          # a window bounds the span
     assert ops.prefill_segments(1 << 20, 0, 8192, 64)[1] <= 3         # the partial results stay under 256 MB
 

@@ -274,7 +274,7 @@ def test_attention_prefill_cut_into_segments(prefill_form, monkeypatch, seg_keys
 def test_attention_prefill_segments_chosen_automatically():
     """A short chunk at the end of a long context is cut by the engine's own rule."""
     seqs = [(2500, 33), (1100, 2)]
-    assert ops.prefill_segments(2500, 0, 35, 4)[1] > 1 and ops.prefill_segments(1500, 0, 1500, 16) == (0, 1)
+    assert ops.prefill_segments(2500, 0, 35, 4)[1] > 1 and ops.prefill_segments(900, 0, 900, 16) == (0, 1)
     for peak in (None, 3, 1200, 2467):
         args = _attention_case(torch.bfloat16, 4, 2, 64, 16, seqs, seed=5, peak=peak)
         close(hip().paged_attention(*args, max_prefill_context=2500), twin.paged_attention(*args), 1.5e-2)
