@@ -89,18 +89,19 @@ class Bench:
     def _ids(self, n):
         return self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen_ids).tolist()
 
-    def prefill(self, rid, n, want_last=True):
+    def prefill(self, rid, n, want_last=True, ids=None):
         from mini_engine_amd.engine.runner import StepEntry
         assert self.manager.allocate(rid, 0, n)
-        return self.runner.step([StepEntry(rid, self._ids(n), 0, [n - 1] if want_last else [])])
+        return self.runner.step([StepEntry(rid, ids if ids is not None else self._ids(n), 0, [n - 1] if want_last else [])])
 
     def time_prefill(self, T: int, reps: int = 3):
         torch = self.torch
         best = None
         for i in range(reps + 1):                          # the first run warms up
+            ids = self._ids(T)                             # drawing the prompt is not the engine's work
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            self.prefill(("p", i), T)
+            self.prefill(("p", i), T, ids=ids)
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
             self.manager.free(("p", i))
