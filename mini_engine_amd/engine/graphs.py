@@ -98,11 +98,12 @@ class _Captured:
 
 
 class DecodeGraphs:
-    def __init__(self, runner, max_bucket: int = 256, capture: bool = True):
+    def __init__(self, runner, max_bucket: int = 256, capture: bool = True, max_graphs: int = 64):
         """capture=False runs the padded, fixed-layout step eagerly every time (no graph): the same
         metadata path without the capture, for machines without a GPU."""
         self.runner = weakref.proxy(runner)      # the runner owns this object: no cycle, so that an engine that
         self.max_bucket = max_bucket             # goes out of use is freed at once, not by a later collection
+        self.max_graphs = max(4, max_graphs)     # (bucket, context cap) pairs kept; the one unused for longest goes first
         self.capture = capture
         self.captured: dict = {}
         # One memory pool for all captured graphs: they replay one after the other on one stream and a
@@ -130,9 +131,12 @@ class DecodeGraphs:
         need_ctx = max(e.start for e in entries) + 1
         ctx_cap = min(-(-need_ctx // CONTEXT_STEP) * CONTEXT_STEP, -(-r.max_positions // 8) * 8)
         key = (bucket, ctx_cap)
-        cap = self.captured.get(key)
+        cap = self.captured.pop(key, None)
         if cap is None:
-            cap = self.captured[key] = _Captured(r, bucket, ctx_cap)
+            cap = _Captured(r, bucket, ctx_cap)
+            while len(self.captured) >= self.max_graphs:      # its last replay lies max_graphs - 1 steps or more back
+                del self.captured[next(iter(self.captured))]
+        self.captured[key] = cap                              # most recently used last
         ps = r.manager.page_size
         tok = np.zeros(bucket, dtype=np.int64)
         pos = np.zeros(bucket, dtype=np.int64)

@@ -283,6 +283,29 @@ def test_decode_rows_follow_a_request_that_was_fed_again(folders, plain_backend)
         assert helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]])) <= helpers.TOL_F32, r
 
 
+def test_decode_layouts_are_dropped_least_recently_used_first(folders, plain_backend):
+    """Only so many (batch bucket, context cap) layouts are kept; one that was dropped is built again."""
+    V, page, folder = helpers.CONFIGS["A"]["vocab_size"], helpers.PAGE["A"], folders("A")
+    model = load_model(folder, "cpu", torch.float32, 512)
+    manager = CacheManager(120, page, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, torch.float32, "cpu", 512, poison_cache=True, use_graphs=True)
+    runner.graphs.max_graphs = 4
+    names = [f"r{i}" for i in range(9)]
+    ids = {r: helpers.random_ids(40, V, 300 + i) for i, r in enumerate(names)}
+    d = helpers.Driver(runner, manager)
+    d.step({r: ids[r][:20] for r in names})
+    pos = 20
+    for count in (1, 2, 3, 5, 9, 1, 9, 2):                 # buckets 1, 2, 4, 8, 16, then some of them again
+        d.step({r: ids[r][pos:pos + 1] for r in names[:count]})
+        for r in names[count:]:                            # the others keep pace through a step of their own
+            d.step({r: ids[r][pos:pos + 1]})
+        pos += 1
+        assert len(runner.graphs.captured) <= 4
+    for r in names:
+        got = d.result(r)
+        assert helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]])) <= helpers.TOL_F32, r
+
+
 def test_toy_architecture_on_cpu(plain_backend):
     """A stateful mixer, a layer run twice, a call that reads another call's cache and an unfused
     position encoding, registered from tests/toy_arch.py, stepped through the real runner."""
