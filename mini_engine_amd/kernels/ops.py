@@ -64,6 +64,7 @@ _CORE_PROTOS = {
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
+    "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
@@ -134,6 +135,44 @@ def _is_i32(t: torch.Tensor, n: int | None = None) -> bool:
 
 
 # --------------------------------------------------------------------------- the HIP backend
+
+LIBRARY_WORKSPACE_BYTES = 64 << 20
+_library_workspace: torch.Tensor | None = None
+_library_direct: bool | None = None      # None: not asked yet
+
+
+def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M, K] . w[N, K]^T through hipBLASLt, bfloat16 operands, float32 accumulation (reference
+    layers/linear.py:25-26: its F.linear is a library product too).
+
+    Called through the core library, which keeps the descriptors and the chosen algorithm of every
+    shape, so a call costs a few microseconds of host time; torch's own route to the same library
+    kernel costs several times that for every call, which is what bounds steps that are not replayed
+    from a graph. torch's route stays as the way out when the process holds no hipBLASLt that the core
+    library can find, or when it offers nothing for a shape. The workspace is allocated once, outside
+    any graph capture (the first product of a process is never a captured one: a step runs eagerly
+    before it is captured)."""
+    global _library_workspace, _library_direct
+    if _library_direct is None:
+        core().cdll.me_gemm_library_available.restype = c_int
+        _library_direct = bool(core().cdll.me_gemm_library_available())
+    if _library_direct and _library_workspace is None and not torch.cuda.is_current_stream_capturing():
+        _library_workspace = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+    if _library_direct and _library_workspace is not None:
+        M, K = x.shape
+        N = w.shape[0]
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        rc = core().fns["me_gemm_library_bf16"](x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
+                                               _code(out_dtype), _library_workspace.data_ptr(),
+                                               LIBRARY_WORKSPACE_BYTES, M, N, K, _stream())
+        if rc == 0:
+            return y
+        if rc != -3:
+            raise KernelError(f"me_gemm_library_bf16: {core().cdll.me_last_error().decode()}")
+    if out_dtype == torch.float32:
+        return torch.mm(x, w.t(), out_dtype=torch.float32)
+    return torch.matmul(x, w.t())
+
 
 class HipBackend:
     """Each method is one kernel (or one dispatch among kernels of the same meaning)."""
@@ -333,9 +372,7 @@ class HipBackend:
             return y
         # many rows, or the head over a large vocabulary: the library product (float32 accumulation; the
         # float32 output form keeps the logits unrounded)
-        if out_dtype == torch.float32:
-            return torch.mm(x, w.t(), out_dtype=torch.float32)
-        return torch.matmul(x, w.t())
+        return library_product(x, w, out_dtype)
 
     def silu_mul_linear(self, gu: torch.Tensor, w: torch.Tensor, allow_partials: bool = False):
         """(silu(gu[:, :I]) * gu[:, I:]) . w[N, I]^T: the gating fused into the product for few

@@ -373,6 +373,33 @@ def test_linear_large_and_odd_bf16(M, N, K):
     close(hip().linear(xs, w), xs.double() @ w.double().t(), 6e-3)
 
 
+@pytest.mark.parametrize("M,N,K", [(200, 384, 80), (2048, 1024, 1024), (65, 100, 200), (4, 6000, 4096), (300, 1531, 1024), (1, 152000, 1024)])
+def test_library_product_is_called_directly(M, N, K):
+    """The library product goes through the core library's own call of hipBLASLt (the process's copy is
+    found, so no step falls back to torch's route) and agrees with the exact product: bfloat16 and float32
+    outputs, a row stride that is not K, a feature count that is no multiple of 8, graph capture."""
+    from mini_engine_amd.kernels import ops
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    ref = x.double() @ w.double().t()
+    close(ops.library_product(x, w, torch.bfloat16), ref, 6e-3)
+    assert ops._library_direct is True and ops._library_workspace is not None
+    close(ops.library_product(x, w, torch.float32), ref, 2e-5)
+    xs = torch.randn(M, K + 8, device=DEV).bfloat16()[:, :K]
+    close(ops.library_product(xs, w, torch.bfloat16), xs.double() @ w.double().t(), 6e-3)
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            y = ops.library_product(x, w, torch.float32)
+    for _ in range(3):                        # every replay, with eager work between them
+        x.copy_(torch.randn(M, K, device=DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        close(y, x.double() @ w.double().t(), 2e-5)
+        close(ops.library_product(x, w, torch.float32), x.double() @ w.double().t(), 2e-5)
+
+
 # ------------------------------------------------------------------------------- sampling
 
 def test_sample_greedy_and_noise():
