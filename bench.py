@@ -170,12 +170,32 @@ class Bench:
         random ids below 10000, max_tokens 100-1024, temperature 0.6, ignore_eos, max_num_seqs 256,
         max_model_len 2048, chunked prefill under a 16k budget. Returns (sum of max_tokens / seconds, record)."""
         from random import randint, seed
-        from types import SimpleNamespace
-        from mini_engine_amd.engine.llm_engine import LLMEngine
-        from mini_engine_amd.sampling.sampling_params import SamplingParams
         seed(0)
         prompts = [[randint(0, 10000) % self.cfg.vocab_size for _ in range(randint(100, 1024))] for _ in range(num_seqs)]
         max_tokens = [randint(100, 1024) for _ in range(num_seqs)]
+        rate, record = self.serve(prompts, max_tokens, budget, max_model_len)
+        record["reference_a100_tok_s"] = 4205.0
+        return rate, record
+
+    def mixed_lengths(self, num_seqs: int, budget: int = 2048, max_model_len: int = 8192):
+        """Nine short prompts (128-512 tokens) to one long (4,096-7,680), 128-256 output tokens each, chunked
+        prefill under a 2,048 budget: long prompts go through the cache in portions while the others decode
+        beside them, so most steps are mixed ones. Same sampling and engine settings as `offline`."""
+        from random import randint, random, seed
+        seed(0)
+        lengths = [randint(4096, 7680) if random() < 0.1 else randint(128, 512) for _ in range(num_seqs)]
+        prompts = [[randint(0, 10000) % self.cfg.vocab_size for _ in range(n)] for n in lengths]
+        max_tokens = [randint(128, 256) for _ in range(num_seqs)]
+        rate, record = self.serve(prompts, max_tokens, budget, max_model_len)
+        record["long_prompts"] = sum(n >= 4096 for n in lengths)
+        return rate, record
+
+    def serve(self, prompts, max_tokens, budget: int, max_model_len: int):
+        """All requests handed to the engine at once (scheduler, sampler and step function as `LLM.generate`
+        uses them; temperature 0.6, ignore_eos, at most 256 running). Returns (output tokens / second, record)."""
+        from types import SimpleNamespace
+        from mini_engine_amd.engine.llm_engine import LLMEngine
+        from mini_engine_amd.sampling.sampling_params import SamplingParams
         conf = SimpleNamespace(max_num_seqs=256, max_num_batched_tokens=budget, long_prefill_token_threshold=0,
                                enable_chunked_prefill=True, scheduling_policy="fcfs", eos=-1, max_model_len=max_model_len,
                                seed=0, run_ahead=self.run_ahead)
@@ -188,8 +208,8 @@ class Bench:
         dt = time.perf_counter() - t0
         total = sum(max_tokens)
         return total / dt, {"value": round(total / dt, 1), "unit": "output tokens/s", "seconds": round(dt, 2),
-                            "requests": num_seqs, "input_tokens": sum(len(p) for p in prompts), "output_tokens": total,
-                            "preemptions": llm.scheduler.num_preemptions, "reference_a100_tok_s": 4205.0}
+                            "requests": len(prompts), "input_tokens": sum(len(p) for p in prompts), "output_tokens": total,
+                            "budget": budget, "preemptions": llm.scheduler.num_preemptions}
 
 
 def main(argv=None) -> int:
@@ -209,6 +229,8 @@ def main(argv=None) -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--offline", type=int, default=256,
                     help="also run the reference's offline workload with this many requests (0: skip)")
+    ap.add_argument("--mixed-lengths", type=int, default=0,
+                    help="also run this many requests with nine short prompts to one long under a 2,048 budget (0: skip)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="fetch every decode step's tokens before the next step is launched")
@@ -223,8 +245,10 @@ def main(argv=None) -> int:
     cfg, full_layers = model_config(args.model_size, args.layers)
     points = [int(p) for p in args.points.split(",") if p]
     off_pages = args.offline * -(-2048 // args.page) if args.offline else 0
+    if args.mixed_lengths:      # room for every request at its full length (a tenth of them long): no preemption
+        off_pages = max(off_pages, args.mixed_lengths * -(-(768 + 8192 // 8) // args.page))
     bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed,
-                  graphs=not args.no_graphs, min_pages=off_pages, max_len=2048 if args.offline else 0,
+                  graphs=not args.no_graphs, min_pages=off_pages, max_len=8192 if args.mixed_lengths else 2048 if args.offline else 0,
                   run_ahead=not args.no_run_ahead)
     item = 2 if args.dtype == "bfloat16" else 4
 
@@ -250,6 +274,11 @@ def main(argv=None) -> int:
         _, offline = bench.offline(args.offline)
         print(f"[bench] reference offline workload: {offline['value']} output tokens/s", file=sys.stderr, flush=True)
 
+    mixed = None
+    if args.mixed_lengths:
+        _, mixed = bench.mixed_lengths(args.mixed_lengths)
+        print(f"[bench] short and long prompts mixed: {mixed['value']} output tokens/s", file=sys.stderr, flush=True)
+
     line = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens; % roofline",
         "value": round(args.batch / step_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
@@ -266,6 +295,8 @@ def main(argv=None) -> int:
     }
     if offline is not None:
         line["offline"] = offline
+    if mixed is not None:
+        line["mixed_lengths"] = mixed
     print(json.dumps(line), flush=True)
     return 0
 

@@ -25,6 +25,7 @@ struct Api {
   decltype(&hipblasLtMatmulDescCreate) desc_create = nullptr;
   decltype(&hipblasLtMatmulDescSetAttribute) desc_set = nullptr;
   decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
+  decltype(&hipblasLtMatrixLayoutSetAttribute) layout_set = nullptr;
   decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
   decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
   decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
@@ -42,7 +43,7 @@ struct Plan {
   bool ok = false;
 };
 
-using PlanKey = std::tuple<int, int, int, int, int64_t, int64_t, int64_t, int, size_t>;
+using PlanKey = std::tuple<int, int, int, int, int64_t, int64_t, int64_t, int, size_t, int>;
 
 std::mutex g_mutex;
 Api g_api;
@@ -65,6 +66,7 @@ bool look_up_api() {
              bind(lib, "hipblasLtMatmulDescCreate", g_api.desc_create) &&
              bind(lib, "hipblasLtMatmulDescSetAttribute", g_api.desc_set) &&
              bind(lib, "hipblasLtMatrixLayoutCreate", g_api.layout_create) &&
+             bind(lib, "hipblasLtMatrixLayoutSetAttribute", g_api.layout_set) &&
              bind(lib, "hipblasLtMatmulPreferenceCreate", g_api.pref_create) &&
              bind(lib, "hipblasLtMatmulPreferenceSetAttribute", g_api.pref_set) &&
              bind(lib, "hipblasLtMatmulPreferenceDestroy", g_api.pref_destroy) &&
@@ -75,8 +77,17 @@ bool look_up_api() {
 
 // Row-major y = x . w^T is, in the library's column-major terms, D[N, M] = op_T(A)[N, K] . B[K, M]
 // with A = w seen as [K, N] (leading dimension ldw) and B = x seen as [K, M] (leading dimension ldx).
+// With splits > 1 the product is a strided batch over slices of K: slice s reads k in [s K/splits,
+// (s+1) K/splits) of both operands (the slices of one operand interleave in memory, which read-only
+// operands may) and writes its own [M, N] of partial sums.
+bool set_batch(hipblasLtMatrixLayout_t layout, int32_t count, int64_t stride) {
+  return g_api.layout_set(layout, HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &count, sizeof(count)) == HIPBLAS_STATUS_SUCCESS &&
+         g_api.layout_set(layout, HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET, &stride, sizeof(stride)) ==
+             HIPBLAS_STATUS_SUCCESS;
+}
+
 bool make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
-               int out_dtype, size_t workspace_bytes) {
+               int out_dtype, size_t workspace_bytes, int splits) {
   const hipDataType out_type = out_dtype == ME_F32 ? HIP_R_32F : HIP_R_16BF;
   if (g_api.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
   const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
@@ -85,6 +96,8 @@ bool make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int64_t l
   if (g_api.layout_create(&p.a, HIP_R_16BF, K, N, ldw) != HIPBLAS_STATUS_SUCCESS) return false;
   if (g_api.layout_create(&p.b, HIP_R_16BF, K, M, ldx) != HIPBLAS_STATUS_SUCCESS) return false;
   if (g_api.layout_create(&p.c, out_type, N, M, ldy) != HIPBLAS_STATUS_SUCCESS) return false;
+  if (splits > 1 && !(set_batch(p.a, splits, K) && set_batch(p.b, splits, K) && set_batch(p.c, splits, (int64_t)M * ldy)))
+    return false;
   hipblasLtMatmulPreference_t pref = nullptr;
   if (g_api.pref_create(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
   const uint64_t max_ws = workspace_bytes;
@@ -114,13 +127,19 @@ extern "C" int me_gemm_library_available() {
 // `workspace_bytes` that the caller owns and that every call on one stream may share. Allocates no
 // device memory. Returns 0; -3 if no hipBLASLt is loaded in the process or it offers no algorithm for
 // the shape within the workspace (the caller takes another path); -1/-2 on other failures.
+// splits > 1: K is cut in that many equal slices and y is float32 [splits, M, ldy], the partial sums
+// of the slices, for a consumer that adds them; this is how a product with few output tiles and a long
+// K fills the GPU with the library's kernels.
 extern "C" int me_gemm_library_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
                                     int out_dtype, void* workspace, size_t workspace_bytes, int M, int N, int K,
-                                    hipStream_t stream) {
+                                    int splits, hipStream_t stream) {
   ME_CHECK(M >= 1 && N >= 1 && K >= 1, "gemm_library: empty product %d x %d x %d", M, N, K);
   ME_CHECK(ldx >= K && ldw >= K && ldy >= N, "gemm_library: a row stride is shorter than its row");
   ME_CHECK(out_dtype == ME_BF16 || out_dtype == ME_F32, "gemm_library: unknown output dtype %d", out_dtype);
   ME_CHECK(x != nullptr && w != nullptr && y != nullptr, "gemm_library: null operand");
+  ME_CHECK(splits >= 1 && K % splits == 0 && (splits == 1 || ((K / splits) % 8 == 0 && out_dtype == ME_F32)),
+           "gemm_library: %d splits of K=%d need equal slices of a multiple of 8 and float32 partial sums", splits, K);
+  const int Ks = K / splits;
   int device = 0;
   ME_CHECK(hipGetDevice(&device) == hipSuccess, "gemm_library: no current device");
   const Plan* plan = nullptr;
@@ -141,11 +160,11 @@ extern "C" int me_gemm_library_bf16(const void* x, int64_t ldx, const void* w, i
       h = g_handles.emplace(device, made).first;
     }
     handle = h->second;
-    const PlanKey key{device, M, N, K, ldx, ldw, ldy, out_dtype, workspace_bytes};
+    const PlanKey key{device, M, N, K, ldx, ldw, ldy, out_dtype, workspace_bytes, splits};
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
       Plan made;
-      made.ok = make_plan(handle, made, M, N, K, ldx, ldw, ldy, out_dtype, workspace == nullptr ? 0 : workspace_bytes);
+      made.ok = make_plan(handle, made, M, N, Ks, ldx, ldw, ldy, out_dtype, workspace == nullptr ? 0 : workspace_bytes, splits);
       it = g_plans.emplace(key, made).first;
     }
     if (!it->second.ok) {

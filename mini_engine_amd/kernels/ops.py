@@ -64,7 +64,7 @@ _CORE_PROTOS = {
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
-    "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, P],
+    "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
@@ -141,7 +141,19 @@ _library_workspace: torch.Tensor | None = None
 _library_direct: bool | None = None      # None: not asked yet
 
 
-def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+def library_is_direct() -> bool:
+    """Whether the core library found a hipBLASLt in the process that it can call itself. Without a GPU
+    (the dispatch rules are also asked on their own) the answer is yes, as on every GPU box."""
+    global _library_direct
+    if _library_direct is None:
+        if not torch.cuda.is_available():
+            return True
+        core().cdll.me_gemm_library_available.restype = c_int
+        _library_direct = bool(core().cdll.me_gemm_library_available())
+    return _library_direct
+
+
+def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, splits: int = 1) -> torch.Tensor:
     """x [M, K] . w[N, K]^T through hipBLASLt, bfloat16 operands, float32 accumulation (reference
     layers/linear.py:25-26: its F.linear is a library product too).
 
@@ -151,24 +163,27 @@ def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) ->
     from a graph. torch's route stays as the way out when the process holds no hipBLASLt that the core
     library can find, or when it offers nothing for a shape. The workspace is allocated once, outside
     any graph capture (the first product of a process is never a captured one: a step runs eagerly
-    before it is captured)."""
-    global _library_workspace, _library_direct
-    if _library_direct is None:
-        core().cdll.me_gemm_library_available.restype = c_int
-        _library_direct = bool(core().cdll.me_gemm_library_available())
-    if _library_direct and _library_workspace is None and not torch.cuda.is_current_stream_capturing():
+    before it is captured).
+
+    splits > 1: K is cut in that many equal slices, computed as one strided batch; the result is their
+    float32 partial sums [splits, M, N] for a consumer that adds them, or None where only torch's
+    route is open (the caller then takes its other path)."""
+    global _library_workspace
+    if library_is_direct() and _library_workspace is None and not torch.cuda.is_current_stream_capturing():
         _library_workspace = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
     if _library_direct and _library_workspace is not None:
         M, K = x.shape
         N = w.shape[0]
-        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        y = torch.empty((M, N) if splits == 1 else (splits, M, N), dtype=out_dtype, device=x.device)
         rc = core().fns["me_gemm_library_bf16"](x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                                                _code(out_dtype), _library_workspace.data_ptr(),
-                                               LIBRARY_WORKSPACE_BYTES, M, N, K, _stream())
+                                               LIBRARY_WORKSPACE_BYTES, M, N, K, splits, _stream())
         if rc == 0:
             return y
         if rc != -3:
             raise KernelError(f"me_gemm_library_bf16: {core().cdll.me_last_error().decode()}")
+    if splits > 1:
+        return None                 # partial sums over slices of K only through the direct call
     if out_dtype == torch.float32:
         return torch.mm(x, w.t(), out_dtype=torch.float32)
     return torch.matmul(x, w.t())
@@ -328,7 +343,7 @@ class HipBackend:
         """x [M, K] . w[N, K]^T (reference layers/linear.py:25-26: F.linear, no bias).
 
         float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 32 rows (64 for
-        smaller weights or when K is split), the library product (hipBLASLt through torch) above that, for the head over a
+        smaller weights or when K is split), the library product (hipBLASLt, library_product) above that, for the head over a
         large vocabulary and for large weights with several rows (library_streams_better), the FMA
         kernel for shapes the MFMA kernel refuses. With allow_partials a
         skinny product with few output features may split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
@@ -352,6 +367,10 @@ class HipBackend:
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
             return y
+        if allow_partials and out_dtype == x.dtype and library_splits(M, N, K) > 1:
+            parts = library_product(x, w, torch.float32, library_splits(M, N, K))
+            if parts is not None:
+                return parts
         if allow_partials and out_dtype == x.dtype and rows_takes(M, N, K):
             ksplit = rows_ksplit(K)
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
@@ -510,6 +529,35 @@ def skinny_takes(M: int, N: int, K: int) -> bool:
     return rows_ok and N < LIBRARY_MIN_N and not library_streams_better(M, N, K)
 
 
+LIBRARY_SPLIT_MIN_ROWS = 33
+LIBRARY_SPLIT_MAX_ROWS = 1024
+LIBRARY_SPLIT_MIN_WEIGHT = 16 << 20
+
+
+def library_splits(M: int, N: int, K: int) -> int:
+    """In how many slices of K the library computes a product whose consumer adds float32 partial sums
+    (1: not this way). o and down have few output features and a long K, so the library's plain call
+    covers the output with too few tiles to fill the GPU (it has no split over K of its own for these
+    shapes); as a strided batch over slices of K it runs the same large-tile kernels on 2-8 times the
+    tiles. From 33 rows (below, the skinny and the rows kernel are as fast or faster) to 1,024 (above,
+    the tiles suffice and the partial sums, S x M x N x 4 bytes written and read again, cost more than
+    the split gains), for weights of 16 M elements or more. Measured, us (plain call / slices), weights
+    from HBM:
+      4096 x 4096:    48 rows 13.9 / 12.4 (8),  128 rows 24.4 / 15.3 (8),  256 rows 22.7 / 20.0 (8),  1024 rows 44.4 / 38.6 (2)
+      4096 x 12288:   48 rows 33.6 / 25.7 (8),  128 rows 67.4 / 29.2 (8),  256 rows 55.3 / 34.5 (8),  512 rows 83.1 / 52.9 (4)
+      5120 x 8192:    48 rows 42.8 / 25.2 (8),  128 rows 44.7 / 29.9 (8),  256 rows 74.2 / 34.0 (8),  512 rows 68.0 / 46.5 (4)
+      5120 x 25600:   48 rows 152 / 55.9 (8),   128 rows 182 / 65.9 (8),   256 rows 263 / 80.2 (8),   1024 rows 350 / 222 (2)
+    (the rows kernel at 48 and 64 rows of 5120 x 25600: 82 and 87)."""
+    if not (LIBRARY_SPLIT_MIN_ROWS <= M <= LIBRARY_SPLIT_MAX_ROWS) or N * K < LIBRARY_SPLIT_MIN_WEIGHT:
+        return 1
+    if not library_is_direct():
+        return 1
+    splits = 8 if M <= 256 else 4 if M <= 512 else 2
+    while splits > 1 and (K % (8 * splits) or K // splits < 512):
+        splits //= 2
+    return splits
+
+
 def rows_takes(M: int, N: int, K: int) -> bool:
     """Whether a product whose consumer adds float32 partial sums goes to the rows kernel (64 features per
     workgroup, the tokens staged once per workgroup in LDS, K split over up to 8 workgroups): large
@@ -521,7 +569,7 @@ def rows_takes(M: int, N: int, K: int) -> bool:
       5120 x 8192:   24 rows 23.3 / 26.0,  48 rows 28.0 / 43.1,  64 rows 33.3 / 29.2 (left to the library)
       5120 x 25600:   8 rows 63.2 / 66.8,  32 rows 70.7 / 109,   64 rows 86.6 / 157
       2560 x 9728:   24 rows 19.2 / 19.1,  48 rows 26.4 / 20.5 (left to the library)"""
-    if N * K < ROWS_MIN_WEIGHT or K < 4096 or K % 8 or M > 64:
+    if N * K < ROWS_MIN_WEIGHT or K < 4096 or K % 8 or M > 64 or library_splits(M, N, K) > 1:
         return False
     if M > 16:
         return M <= 32 or K >= 12288

@@ -56,10 +56,25 @@ def test_skinny_kernel_takes_few_rows():
 
 def test_rows_kernel_takes_many_rows_over_large_weights():
     assert ops.rows_takes(24, 4096, 4096) and not ops.rows_takes(64, 4096, 4096)     # above 32 rows only over a long K
-    assert ops.rows_takes(64, 4096, 12288) and ops.rows_takes(32, 5120, 8192) and not ops.rows_takes(64, 5120, 8192)
+    assert ops.rows_takes(32, 4096, 12288) and ops.rows_takes(32, 5120, 8192) and not ops.rows_takes(64, 5120, 8192)
+    assert not ops.rows_takes(64, 4096, 12288)       # from 33 rows the library's slices of K take these weights
+    assert ops.rows_takes(64, 1400, 12296)           # ... unless K has no equal slices of a multiple of 8
     assert ops.rows_takes(8, 5120, 25600) and not ops.rows_takes(4, 5120, 25600)     # few rows: only where the library is out
     assert not ops.rows_takes(8, 4096, 12288) and not ops.rows_takes(64, 1024, 3072) and not ops.rows_takes(65, 5120, 25600)
     for K in (4096, 4104, 9728, 12288, 25600):
         ks, chunks = ops.rows_ksplit(K), -(-K // 512)
         assert 1 <= ks <= 8 and (ks - 1) * -(-chunks // ks) < chunks
 
+
+
+def test_library_slices_of_k_for_o_and_down_at_many_rows():
+    assert ops.library_splits(32, 4096, 12288) == 1 and ops.library_splits(33, 4096, 12288) == 8
+    assert ops.library_splits(256, 5120, 25600) == 8 and ops.library_splits(257, 5120, 25600) == 4
+    assert ops.library_splits(512, 5120, 8192) == 4 and ops.library_splits(1024, 5120, 8192) == 2
+    assert ops.library_splits(1025, 5120, 8192) == 1
+    assert ops.library_splits(128, 1024, 3072) == 1 and ops.library_splits(128, 2048, 8192) == 8   # 16 M elements or more
+    assert ops.library_splits(64, 1400, 12296) == 1      # 12296 = 8 x 1537: no two equal slices of a multiple of 8
+    assert ops.library_splits(64, 4096, 4096 + 32) == 4  # 4128 = 4 x 1032
+    for M, N, K in ((100, 4096, 4096), (300, 5120, 17408), (40, 2560, 9728)):
+        s = ops.library_splits(M, N, K)
+        assert s > 1 and K % (8 * s) == 0 and K // s >= 512

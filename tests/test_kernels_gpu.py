@@ -346,7 +346,7 @@ def test_linear_partials_are_used_where_tiles_are_few():
         close(parts.sum(0), x.double() @ w.double().t(), 2e-5)
 
 
-@pytest.mark.parametrize("M,N,K", [(24, 4096, 4096), (17, 4100, 4104), (20, 4000, 4224), (64, 1400, 12296), (33, 1368, 12288), (9, 1000, 16896)])
+@pytest.mark.parametrize("M,N,K", [(24, 4096, 4096), (17, 4100, 4104), (20, 4000, 4224), (64, 1400, 12296), (32, 1368, 12288), (9, 1000, 16896)])
 def test_linear_rows_kernel(M, N, K):
     """17 to 64 rows over large weights (and fewer over a very long K), partial sums allowed: 64 features per
     workgroup, the tokens staged in LDS chunk by chunk; feature counts and K that are no multiples of 64, 128 or 512."""
@@ -398,6 +398,29 @@ def test_library_product_is_called_directly(M, N, K):
         torch.cuda.synchronize()
         close(y, x.double() @ w.double().t(), 2e-5)
         close(ops.library_product(x, w, torch.float32), x.double() @ w.double().t(), 2e-5)
+
+
+@pytest.mark.parametrize("M,N,K", [(33, 4096, 4096), (128, 4096, 4096), (200, 2560, 9728), (300, 4096, 12288), (700, 5120, 8192), (64, 1368, 12288 + 64)])
+def test_linear_library_slices_of_k(M, N, K):
+    """o and down at 33 to 1,024 rows over large weights: the library runs slices of K as one strided batch
+    and the consumer adds the float32 partial sums."""
+    from mini_engine_amd.kernels import ops
+    splits = ops.library_splits(M, N, K)
+    assert splits == (8 if M <= 256 else 4 if M <= 512 else 2) and K % (8 * splits) == 0
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    parts = hip().linear(x, w, None, allow_partials=True)
+    assert parts.shape == (splits, M, N) and parts.dtype == torch.float32
+    close(parts.sum(0), x.double() @ w.double().t(), 2e-5)
+    xs = torch.randn(M, K + 8, device=DEV).bfloat16()[:, :K]   # a row stride that is not K
+    close(hip().linear(xs, w, None, allow_partials=True).sum(0), xs.double() @ w.double().t(), 2e-5)
+    # the norm that follows takes them as they are
+    res = torch.randn(M, N, device=DEV)
+    nw = torch.rand(N, device=DEV) + 0.5
+    y, new_res = hip().rms_norm(parts, nw, 1e-6, res, torch.bfloat16)
+    want_y, want_res = twin.rms_norm(parts.sum(0), nw, 1e-6, res, torch.bfloat16)
+    close(new_res, want_res, 1e-6)
+    close(y, want_y, 6e-3)
 
 
 # ------------------------------------------------------------------------------- sampling
