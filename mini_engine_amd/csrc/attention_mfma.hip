@@ -843,7 +843,18 @@ __global__ void __launch_bounds__(256) attn_prefill_merge_kernel(AttnArgs a, int
 // the 4 waves of a workgroup take the 32-key blocks of the partition in turn and are merged
 // through LDS. With one partition the result is written directly; otherwise the partition's
 // (max, sum, unnormalised output) go to scratch for the reduce kernel.
+// The number of partitions is that of the longest context in the batch. A sequence's partitions
+// beyond its own context (or wholly before its window) have no keys: their workgroups leave at once
+// and write nothing, and the reduce kernel reads only the range decode_part_range gives. The last
+// partitions are dispatched first (grid z counts down): only long sequences have them, so in a batch
+// of contexts of very different lengths the longest sequences start first instead of last.
 // =====================================================================================
+__device__ __forceinline__ void decode_part_range(const AttnArgs& a, int L, int& first, int& end) {
+  const int lo = a.window > 0 ? max(0, L - a.window) : 0;
+  first = min((lo & ~31) / a.part_size, a.num_parts - 1);
+  end = max(first + 1, min(a.num_parts, (L + a.part_size - 1) / a.part_size));
+}
+
 __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
   extern __shared__ float lds[];  // [4 waves][cols][HD + 2]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -851,8 +862,13 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
   const int b = blockIdx.x;
   const int col_tiles = (a.G + 15) / 16;
   const int kvh = blockIdx.y / col_tiles, ctile = blockIdx.y - kvh * col_tiles;
-  const int part = blockIdx.z;
+  const int part = a.num_parts - 1 - blockIdx.z;
   const int L = a.context_lens[b];
+  if (a.num_parts > 1) {
+    int first, end;
+    decode_part_range(a, L, first, end);
+    if (part < first || part >= end) return;
+  }
   const int pos = L - 1;
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int32_t* bt = a.block_tables + (int64_t)b * a.bt_stride;
@@ -929,8 +945,10 @@ __global__ void __launch_bounds__(128) attn_reduce_kernel(AttnArgs a) {
   __shared__ float wgt[RED_MAX_PARTS];
   __shared__ float inv_s;
   const int b = blockIdx.x, hq = blockIdx.y;
-  const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_parts;
-  const int P = a.num_parts;
+  int part0, part_end;
+  decode_part_range(a, a.context_lens[b], part0, part_end);
+  const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_parts + part0;
+  const int P = part_end - part0;
   // the first 16 partitions' values of this thread's channel are asked for before the weights are
   // formed: they do not depend on them, and the two rounds of loads then overlap
   const int d0 = threadIdx.x;

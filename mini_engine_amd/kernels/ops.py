@@ -474,6 +474,9 @@ GATED_MAX_M = 16
 _TARGET_WORKGROUPS = 512
 _COMPUTE_UNITS = 256
 _DECODE_WORKGROUPS = 4096
+_DECODE_WHOLE_WORKGROUPS = 2048
+_DECODE_WHOLE_MAX_KEYS = 4096
+_DECODE_MAX_PARTITION = 2048
 _scratch_buf: dict = {}
 _scratch_retired: list = []      # outgrown buffers stay alive: a captured graph may still write to them
 
@@ -612,12 +615,21 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int) -> tup
     A workgroup's 4 waves take 32 keys each per round, so a partition of 128 keys is one round
     with every load in flight at once; partitions grow beyond that only when (sequences x kv
     heads x partitions) already gives several workgroups per compute unit, or to keep the
-    number of partitions to merge at 64 or less. (The reference's rule: layers/ops.py:44-51,
-    split when sequences x kv heads cannot fill the SMs, 256-key partitions.)"""
+    number of partitions to merge at 64 or less. A partition holds at most 2,048 keys (as long as 64
+    partitions cover the context): a workgroup goes through its keys round by round, so in a batch with
+    a few long contexts among short ones the long partitions are what is still running at the end
+    (128 sequences, four of 16 k keys among 100-2,048: 4096 x 4 311 us, 2048 x 8 283 us, 1024 x 16 280 us).
+    From 2,048 workgroups on (256 sequences x 8 kv heads) a context up to 4,096 keys is one partition and
+    needs no reduce kernel (256 x 4,096 keys: 719 us against 752 us in two; 256 x 100-600 keys: 74 against
+    83 us). (The reference's rule: layers/ops.py:44-51, split when sequences x kv heads cannot fill the
+    SMs, 256-key partitions.)"""
     col_tiles = (Hq // Hkv + 15) // 16
     base = max(1, num_seqs * Hkv * col_tiles)
     ctx = max(1, max_context)
-    want = max(1, min(64, -(-_DECODE_WORKGROUPS // base)))
+    if base >= _DECODE_WHOLE_WORKGROUPS and ctx <= _DECODE_WHOLE_MAX_KEYS:
+        return -(-ctx // 128) * 128, 1
+    want = max(1, -(-_DECODE_WORKGROUPS // base), -(-ctx // _DECODE_MAX_PARTITION))
+    want = min(64, want)
     part = max(128, -(-(-(-ctx // want)) // 128) * 128)
     parts = max(1, -(-ctx // part))
     return part, parts

@@ -8,6 +8,13 @@ def test_decode_partitions_cover_the_context():
         part, parts = ops.decode_partitions(S, Hq, Hkv, ctx)
         assert part % 128 == 0 and parts <= 64 or part * 64 >= ctx
         assert part * parts >= ctx and part * (parts - 1) < ctx
+    assert ops.decode_partitions(8, 16, 8, 2048) == (128, 16)
+    # a partition holds at most 2,048 keys while 64 partitions cover the context
+    assert ops.decode_partitions(128, 16, 8, 16384) == (2048, 8) and ops.decode_partitions(256, 16, 8, 8192) == (2048, 4)
+    assert ops.decode_partitions(3, 6, 2, 130000) == (2048, 64) and ops.decode_partitions(4, 16, 8, 1 << 20) == (16384, 64)
+    # 2,048 workgroups without a split: contexts up to 4,096 keys stay whole
+    assert ops.decode_partitions(256, 16, 8, 2048) == (2048, 1) and ops.decode_partitions(256, 16, 8, 4096) == (4096, 1)
+    assert ops.decode_partitions(255, 16, 8, 2048)[1] > 1 and ops.decode_partitions(256, 16, 8, 4097)[1] > 1
 
 
 def test_prefill_segments_cover_the_span_and_hold_512_keys_or_more():

@@ -237,6 +237,24 @@ def test_attention_decode_batches(dtype, Hq, Hkv, D, page):
         close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
 
 
+@pytest.mark.parametrize("window", [None, 100, 1000])
+def test_attention_decode_contexts_of_very_different_lengths(window):
+    """One batch with contexts from 1 to 3,000 keys: the partitions are those of the longest, so most
+    sequences have partitions without keys (beyond their context, or wholly before their window), whose
+    workgroups write nothing and which the reduce kernel must not read. The peak key sits in the first,
+    a middle and the last partition of the long sequences."""
+    torch.empty(1 << 24, device=DEV).fill_(float("nan"))      # what freed memory holds is not zero
+    seqs = [(3000, 1), (40, 1), (1, 1), (700, 1), (2049, 1), (128, 1), (129, 1), (2999, 1)]
+    for peak in (None, 0, 1500, 2998):
+        if window is not None and peak is not None and peak < 2999 - window:
+            continue                                           # a peak outside the window is seen by nobody
+        args = _attention_case(torch.bfloat16, 16, 8, 128, 16, seqs, window=window, seed=7, peak=peak)
+        close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
+    many = [(100 + 37 * i % 1900, 1) for i in range(256)]     # 2,048 workgroups: one partition, no reduce
+    args = _attention_case(torch.bfloat16, 16, 8, 128, 16, many, window=window, seed=8)
+    close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_far_key_stands_out(prefill_form, dtype):
     """One key among hundreds gets all the weight: a kernel that drops or misplaces a block,
@@ -292,7 +310,8 @@ def test_attention_generic_path_takes_odd_sizes():
 
 
 def test_decode_partitions_rule():
-    for S, Hq, Hkv, ctx in ((1, 16, 8, 2048), (8, 16, 8, 2048), (64, 16, 8, 2304), (1, 32, 8, 100), (3, 6, 2, 130000)):
+    for S, Hq, Hkv, ctx in ((1, 16, 8, 2048), (8, 16, 8, 2048), (64, 16, 8, 2304), (1, 32, 8, 100), (3, 6, 2, 130000),
+                            (256, 16, 8, 4096), (256, 16, 8, 4097), (128, 16, 8, 16384)):
         part, parts = ops.decode_partitions(S, Hq, Hkv, ctx)
         assert part % 128 == 0 and part * parts >= ctx and part * (parts - 1) < ctx
 
