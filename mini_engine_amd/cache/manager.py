@@ -265,6 +265,18 @@ class CacheManager:
             self.free_slots.append(held.state_slot)
 
     # -- checks (used by tests) ------------------------------------------------------------
+    def forget_prefixes(self) -> None:
+        """Drops every published prefix: pages keep their owners, but no later request can hit what
+        is cached now (a benchmark that replays the same prompts under another setting starts cold;
+        the reference builds a new block manager for this, bench_latency.py:51)."""
+        for grp in self.groups:
+            grp.by_hash.clear()
+            for page in range(grp.num_pages):
+                grp.hash[page] = -1
+                grp.tokens[page] = None
+        for held in self.held.values():
+            held.num_hashed = 0
+
     def check_invariants(self) -> None:
         for gi, g in enumerate(self.groups):
             free = list(g.free)
