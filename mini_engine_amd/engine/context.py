@@ -25,6 +25,7 @@ class StepContext:
     prefill_cu: torch.Tensor | None  # int32 [B - Dn + 1] the same for the non-decode requests, from 0
     max_decode_context: int
     max_prefill_context: int = 0     # largest context among the requests with more than one new token
+    decode_contexts_even: bool = False   # the decode requests' contexts are (nearly) equally long
     groups: list = field(default_factory=list)       # GroupStep per page group
     state_slots: torch.Tensor | None = None          # int32 [B]
     first_chunk: torch.Tensor | None = None          # int32 [B]: 1 if the request's tokens start at position 0

@@ -2,7 +2,8 @@
 
 A decode step of a small model is a few hundred short kernels; launched one by one their
 launch cost exceeds their run time. For steps in which every request brings exactly one
-token, the whole forward pass is captured once per (batch bucket, context cap) and replayed:
+token, the whole forward pass is captured once per (batch bucket, context cap, contexts equally
+long or not) and replayed:
 the step's metadata lives in one device array of fixed layout that is rewritten before each
 replay. Rows beyond the real batch are padding: context length 0, slot -1 (nothing is
 written to the cache), token 0.
@@ -18,6 +19,7 @@ import weakref
 import numpy as np
 import torch
 
+from ..kernels import ops
 from .context import GroupStep, StepContext
 
 PENDING = -1      # the runner's marker for a token that is still on the device (runner.PENDING)
@@ -31,8 +33,8 @@ def _pad4(n: int) -> int:
 
 
 class _Captured:
-    def __init__(self, runner, bucket: int, ctx_cap: int):
-        self.bucket, self.ctx_cap = bucket, ctx_cap
+    def __init__(self, runner, bucket: int, ctx_cap: int, even: bool = False):
+        self.bucket, self.ctx_cap, self.even = bucket, ctx_cap, even
         ps = runner.manager.page_size
         self.G = runner.manager.num_groups
         self.MB = -(-ctx_cap // ps)
@@ -80,6 +82,7 @@ class _Captured:
             num_tokens=B, num_seqs=B, num_decodes=B, positions=self.view("positions"),
             seq_of_token=self.view("seq_of_token"), context_lens=self.view("context_lens"),
             cu_seqlens=self.view("cu"), prefill_cu=None, max_decode_context=self.ctx_cap,
+            decode_contexts_even=self.even,
             groups=[GroupStep(self.view(f"bt{g}").view(B, self.MB), self.view(f"slots{g}")) for g in range(self.G)],
             state_slots=self.view("state_slots"), first_chunk=self.view("first_chunk"),
             q_lens=[1] * B, starts=[0] * B)
@@ -130,10 +133,12 @@ class DecodeGraphs:
         bucket = next(b for b in BUCKETS if b >= B)
         need_ctx = max(e.start for e in entries) + 1
         ctx_cap = min(-(-need_ctx // CONTEXT_STEP) * CONTEXT_STEP, -(-r.max_positions // 8) * 8)
-        key = (bucket, ctx_cap)
+        # whether the contexts are equally long is part of the layout: the decode kernel's grid depends on it
+        even = ops.decode_contexts_even(B, min(e.start for e in entries) + 1, need_ctx)
+        key = (bucket, ctx_cap, even)
         cap = self.captured.pop(key, None)
         if cap is None:
-            cap = _Captured(r, bucket, ctx_cap)
+            cap = _Captured(r, bucket, ctx_cap, even)
             while len(self.captured) >= self.max_graphs:      # its last replay lies max_graphs - 1 steps or more back
                 del self.captured[next(iter(self.captured))]
         self.captured[key] = cap                              # most recently used last

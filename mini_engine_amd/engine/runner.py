@@ -235,11 +235,13 @@ class ModelRunner:
             o, size = seg[name]
             return dev[o:o + size]
 
+        decode_ctx = [s + 1 for s, q in zip(starts, q_lens) if q == 1]
         ctx = StepContext(
             num_tokens=T, num_seqs=B, num_decodes=Dn, positions=view("positions"),
             seq_of_token=view("seq_of_token"), context_lens=view("context_lens"), cu_seqlens=view("cu"),
             prefill_cu=view("prefill_cu") if Dn < B else None,
-            max_decode_context=max((s + 1 for s, q in zip(starts, q_lens) if q == 1), default=0),
+            max_decode_context=max(decode_ctx, default=0),
+            decode_contexts_even=bool(decode_ctx) and ops.decode_contexts_even(len(decode_ctx), min(decode_ctx), max(decode_ctx)),
             max_prefill_context=max((s + q for s, q in zip(starts, q_lens) if q != 1), default=0),
             groups=[GroupStep(view(f"bt{g}").view(B, MB[g]), view(f"slots{g}")) for g in range(G)],
             state_slots=view("state_slots"), first_chunk=view("first_chunk"), q_lens=q_lens, starts=starts)

@@ -87,5 +87,6 @@ class Attention(Mixer):
         o = ops.paged_attention(q, cache.k, cache.v, cache.page_size, grp.block_tables, step.context_lens,
                                 step.seq_of_token, step.positions, step.prefill_cu, step.num_decodes,
                                 step.max_decode_context, self.scale, self.window, Hq, Hkv, D,
-                                max_prefill_context=step.max_prefill_context)
+                                max_prefill_context=step.max_prefill_context,
+                                even_contexts=step.decode_contexts_even)
         return self.o.forward(o, allow_partials=True)

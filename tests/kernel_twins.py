@@ -73,7 +73,7 @@ def store_kv(k, v, slots, k_cache, v_cache, page):
 
 def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_of_token, positions,
                     prefill_cu, num_decodes, max_decode_context, scale, window, Hq, Hkv, D,
-                    force_simple=False, max_prefill_context=0, compute_dtype=torch.float32):
+                    force_simple=False, max_prefill_context=0, even_contexts=False, compute_dtype=torch.float32):
     """Token by token: gather the keys this token may see through its request's block table
     and nothing else (so unowned pages are never read), softmax, weighted sum."""
     T = q.shape[0]

@@ -85,3 +85,10 @@ def test_library_slices_of_k_for_o_and_down_at_many_rows():
     for M, N, K in ((100, 4096, 4096), (300, 5120, 17408), (40, 2560, 9728)):
         s = ops.library_splits(M, N, K)
         assert s > 1 and K % (8 * s) == 0 and K // s >= 512
+
+
+def test_requests_stay_on_one_xcd_only_when_their_contexts_are_equally_long():
+    assert ops.decode_contexts_even(8, 2048, 2048) and ops.decode_contexts_even(64, 2000, 2100)
+    assert not ops.decode_contexts_even(64, 1900, 2100) and not ops.decode_contexts_even(256, 100, 2048)
+    assert not ops.decode_contexts_even(7, 2048, 2048)          # fewer requests than XCDs: spread
+    assert not ops.decode_contexts_even(8, 0, 0)                # unknown

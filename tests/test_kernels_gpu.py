@@ -253,6 +253,10 @@ def test_attention_decode_contexts_of_very_different_lengths(window):
     many = [(100 + 37 * i % 1900, 1) for i in range(256)]     # 2,048 workgroups: one partition, no reduce
     args = _attention_case(torch.bfloat16, 16, 8, 128, 16, many, window=window, seed=8)
     close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
+    # both orders of the grid (each request on one XCD, each request spread over all) give the same bits
+    for seqs in ([(2070 + i % 3, 1) for i in range(16)], [(3000, 1), (40, 1), (700, 1)], many):
+        args = _attention_case(torch.bfloat16, 16, 8, 128, 16, seqs, window=window, seed=9)
+        assert torch.equal(hip().paged_attention(*args, even_contexts=True), hip().paged_attention(*args, even_contexts=False))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
