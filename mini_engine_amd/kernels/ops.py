@@ -346,11 +346,13 @@ class HipBackend:
         """x [M, K] . w[N, K]^T (reference layers/linear.py:25-26: F.linear, no bias).
 
         float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 32 rows (64 for
-        smaller weights or when K is split), the library product (hipBLASLt, library_product) above that, for the head over a
-        large vocabulary and for large weights with several rows (library_streams_better), the FMA
-        kernel for shapes the MFMA kernel refuses. With allow_partials a
-        skinny product with few output features may split K over workgroups and return float32 partial sums [S, M, N] for a consumer that
-        adds them."""
+        smaller weights or when K is split), the library product (hipBLASLt, library_product) above
+        that, for the head over a large vocabulary and for large weights with several rows
+        (library_streams_better), the FMA kernel for shapes the MFMA kernel refuses.
+        With allow_partials the result may be float32 partial sums [S, M, N] over slices of K for a
+        consumer that adds them: from the skinny kernel when the output features are few
+        (choose_ksplit), from the rows kernel for 17-32 rows over large weights (rows_takes), from the
+        library as a strided batch for 33-1,024 rows over large weights (library_splits)."""
         _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: {tuple(x.shape)} x {tuple(w.shape)}^T")
         _check(x.dtype == w.dtype, f"linear: activation {x.dtype} and weight {w.dtype} differ")
         _check(x.stride(1) == 1 and w.stride(1) == 1, "linear: rows must be contiguous")
@@ -370,8 +372,9 @@ class HipBackend:
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
             return y
-        if allow_partials and out_dtype == x.dtype and library_splits(M, N, K) > 1:
-            parts = library_product(x, w, torch.float32, library_splits(M, N, K))
+        splits = library_splits(M, N, K) if (allow_partials and out_dtype == x.dtype) else 1
+        if splits > 1:
+            parts = library_product(x, w, torch.float32, splits)
             if parts is not None:
                 return parts
         if allow_partials and out_dtype == x.dtype and rows_takes(M, N, K):
