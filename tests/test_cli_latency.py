@@ -81,9 +81,10 @@ def test_serving_arrivals_gives_every_request_its_tokens_and_times(folders, plai
         llm.manager.check_invariants()
         assert r["num_long"] == sum(a.long for a in arrivals) and r["steps"] > 0 and r["preemptions"] == 0
         assert r["output_tokens"] == sum(a.max_tokens for a in arrivals) and r["out_tok_s"] > 0
-        assert 0 < r["ttft_p50_ms"] <= r["ttft_p99_ms"] and 0 < r["itl_p50_ms"] <= r["itl_p99_ms"] <= r["itl_max_ms"]
-        assert r["tpot_mean_ms"] > 0
-    assert rows["c16"]["steps"] >= rows["pf"]["steps"]      # portions of 16 tokens need more steps than whole prompts
+        # times are wall-clock: only what holds whatever the machine's speed
+        assert 0 <= r["ttft_p50_ms"] <= r["ttft_p99_ms"] and 0 <= r["itl_p50_ms"] <= r["itl_p99_ms"] <= r["itl_max_ms"]
+        assert r["ttft_long_p50_ms"] is not None and r["ttft_short_p99_ms"] is not None and r["tpot_mean_ms"] >= 0
+    assert rows["c16"]["steps"] >= 90 // 16                  # the longest prompt alone needs that many portions
 
 
 @pytest.mark.gpu
