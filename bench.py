@@ -25,22 +25,7 @@ import time
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-SIZES = {
-    # name: (layers, hidden, q heads, kv heads, head_dim, intermediate, vocab, tied)
-    "tinyA": (2, 64, 4, 2, 16, 128, 256, True),
-    "0.6b": (28, 1024, 16, 8, 128, 3072, 151936, True),
-    "8b": (36, 4096, 32, 8, 128, 12288, 151936, False),
-    "32b": (64, 5120, 64, 8, 128, 25600, 151936, False),
-}
-
-
-def model_config(size: str, layers: int | None):
-    from mini_engine_amd.config.model_config import Qwen3Config
-    L, h, Hq, Hkv, D, I, V, tied = SIZES[size]
-    return Qwen3Config.from_dict(dict(
-        architectures=["Qwen3ForCausalLM"], vocab_size=V, hidden_size=h, intermediate_size=I,
-        num_hidden_layers=layers or L, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D,
-        rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=tied, max_position_embeddings=40960)), L
+from mini_engine_amd.config.sizes import SIZES, model_config   # noqa: E402  (the named layer sizes)
 
 
 def linear_params_per_layer(cfg) -> int:

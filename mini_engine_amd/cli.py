@@ -55,8 +55,7 @@ def main(argv=None) -> int:
     tmp = None
     path = args.model
     if args.random_weights:
-        sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-        from bench import SIZES, model_config          # the sizes the repository's benchmark names
+        from .config.sizes import SIZES, model_config
         from .weights.random_init import write_random_model
         if args.random_weights not in SIZES:
             p.error(f"--random-weights must be one of {sorted(SIZES)}")
