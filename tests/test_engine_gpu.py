@@ -274,3 +274,34 @@ def test_real_layer_sizes(tmp_path_factory, dtype):
         got = d.result(r)
         err = helpers.rel_err(got, helpers.plain_logits(folder, ids)[: got.shape[0]])
         assert err <= tol, f"{r}: {err:.3g}"
+
+
+def test_wide_layer_sizes_take_the_products_with_partial_sums(tmp_path_factory):
+    """One layer of Qwen3-8B's width (hidden 4096, 32 query / 8 key heads of 128, intermediate 12288): o and
+    down are large enough for the forms that hand float32 partial sums over slices of K to the norm that
+    follows (the library as a strided batch at 300 and 127 rows, the rows kernel at 28), which the narrow test
+    configurations never reach; then decoding; against the plain implementation."""
+    from mini_engine_amd.config.model_config import Qwen3Config
+    from mini_engine_amd.kernels import ops
+    from mini_engine_amd.weights.random_init import write_random_model
+    cfgd = dict(architectures=["Qwen3ForCausalLM"], vocab_size=1009, hidden_size=4096, intermediate_size=12288,
+                num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
+                rope_theta=1e6, tie_word_embeddings=True, max_position_embeddings=4096)
+    assert ops.library_splits(300, 4096, 4096) == 4 and ops.library_splits(127, 4096, 12288) == 8
+    assert ops.rows_takes(28, 4096, 12288) and ops.rows_takes(28, 4096, 4096)
+    folder = write_random_model(Qwen3Config.from_dict(cfgd), 5, str(tmp_path_factory.mktemp("wide")))
+    model = load_model(folder, "cuda", torch.bfloat16, 1024)
+    manager = CacheManager(64, 16, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, torch.bfloat16, "cuda", 1024, poison_cache=True, use_graphs=True)
+    a, b = helpers.random_ids(400, 1009, 1), helpers.random_ids(70, 1009, 2)
+    d = helpers.Driver(runner, manager)
+    d.step({"a": a[:300]})
+    d.step({"a": a[300:363], "b": b[:64]})
+    d.step({"a": a[363:390], "b": b[64:65]})
+    for t in range(5):
+        d.step({"a": a[390 + t:391 + t], "b": b[65 + t:66 + t]})
+    d.step({"a": a[395:]})
+    for ids, r in ((a, "a"), (b, "b")):
+        got = d.result(r)
+        err = helpers.rel_err(got, helpers.plain_logits(folder, ids)[: got.shape[0]])
+        assert err <= helpers.TOL_BF16, f"{r}: {err:.3g}"
