@@ -13,6 +13,9 @@ other); all of them reach the host inside the timed span. One JSON line is print
   prefill      one 2,048-token prompt in one step: tokens/s, ms, fraction of the bf16 MFMA peak
   roofline     bytes the decode step must read (every weight once + the live requests' cache) / time
   points       decode tokens/s at batch 1 and 64
+  offline      the reference's offline workload (256 requests) through the scheduler: output tokens/s of the
+               second of two passes, and of the first (--offline 0: skip); --mixed-lengths N: the same for N
+               requests with nine short prompts to one long under a 2,048-token budget
 Peaks: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s (MI355X, published).
 """
 from __future__ import annotations
@@ -177,7 +180,8 @@ class Bench:
 
     def serve(self, prompts, max_tokens, budget: int, max_model_len: int):
         """All requests handed to the engine at once (scheduler, sampler and step function as `LLM.generate`
-        uses them; temperature 0.6, ignore_eos, at most 256 running). Returns (output tokens / second, record)."""
+        uses them; temperature 0.6, ignore_eos, at most 256 running). Returns (output tokens / second of the
+        second of two passes, record with both)."""
         from types import SimpleNamespace
         from mini_engine_amd.engine.llm_engine import LLMEngine
         from mini_engine_amd.sampling.sampling_params import SamplingParams
@@ -187,12 +191,19 @@ class Bench:
         llm = LLMEngine.from_parts(conf, self.model, self.manager, self.runner)
         sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
         llm.generate([[1, 2, 3]], SamplingParams(max_tokens=4), use_tqdm=False)
-        self.torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        llm.generate(prompts, sps, use_tqdm=False)
-        dt = time.perf_counter() - t0
+        # The workload runs twice. The first pass, after the reference's one-prompt warm-up (its bench.py:62),
+        # still meets every shape for the first time: decode graphs are captured, the library loads its
+        # kernels and plans its products. The second pass is the engine in its steady state.
+        took = []
+        for _ in range(2):
+            self.torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            llm.generate(prompts, sps, use_tqdm=False)
+            took.append(time.perf_counter() - t0)
+        dt = took[1]
         total = sum(max_tokens)
         return total / dt, {"value": round(total / dt, 1), "unit": "output tokens/s", "seconds": round(dt, 2),
+                            "first_pass_value": round(total / took[0], 1), "first_pass_seconds": round(took[0], 2),
                             "requests": len(prompts), "input_tokens": sum(len(p) for p in prompts), "output_tokens": total,
                             "budget": budget, "preemptions": llm.scheduler.num_preemptions}
 
