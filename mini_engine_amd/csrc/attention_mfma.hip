@@ -641,6 +641,54 @@ __device__ __forceinline__ void pf_commit(const StagedBlock& st, int tid, unsign
   }
 }
 
+// Blocks start at multiples of 32 keys, so most of a thread's address arithmetic is the same for every
+// block: which table entry beyond the block's first its pieces use (pages below 32 keys), and where in
+// a page they lie. For blocks that lie wholly inside the context (pf_lookup<true>, pf_fetch<true> in
+// meaning) only the block's own part is added: its first table entry, its offset in a page of 32 keys
+// or more, the page's base.
+struct StagedInvariants {
+  int kidx[PF_PIECES], vidx[PF_PIECES];   // table entries beyond (t0 >> page_shift)
+  int koff[PF_PIECES], voff[PF_PIECES];   // element offsets inside a page, without the block's own part
+};
+__device__ __forceinline__ void pf_invariants(const AttnArgs& a, int kvh, int tid, StagedInvariants& iv) {
+  const bool small = a.page < 32;
+#pragma unroll
+  for (int j = 0; j < PF_PIECES; ++j) {
+    const int p = tid + 256 * j;
+    const bool in = p < 4 * HD;
+    const int row = p / (HD / 8), ch = p - row * (HD / 8);
+    const int krow = small ? (row & (a.page - 1)) : row;
+    iv.kidx[j] = (in && small) ? row >> a.page_shift : 0;
+    iv.koff[j] = in ? (kvh * a.page + krow) * HD + 8 * ch : 0;
+    const int d = in ? p >> 2 : 0, k8 = 8 * (p & 3);
+    iv.vidx[j] = (in && small) ? k8 >> a.page_shift : 0;
+    iv.voff[j] = in ? (kvh * HD + d) * a.page + (small ? (k8 & (a.page - 1)) : k8) : 0;
+  }
+}
+__device__ __forceinline__ void pf_lookup_inside(const AttnArgs& a, const int32_t* __restrict__ bt, int t0,
+                                                 const StagedInvariants& iv, StagedPages& pg) {
+  const int32_t* first = bt + (t0 >> a.page_shift);
+#pragma unroll
+  for (int j = 0; j < PF_PIECES; ++j) {
+    pg.k[j] = first[iv.kidx[j]];
+    pg.v[j] = first[iv.vidx[j]];
+  }
+}
+__device__ __forceinline__ void pf_fetch_inside(const AttnArgs& a, const StagedPages& pg, int t0,
+                                                const StagedInvariants& iv, StagedBlock& st) {
+  const int64_t page_stride = (int64_t)a.Hkv * a.page * HD;
+  const int in_page = a.page >= 32 ? (t0 & (a.page - 1)) : 0;      // the same for every thread
+  const bf16_t* kbase = a.k_cache + in_page * HD;
+  const bf16_t* vbase = a.v_cache + in_page;
+#pragma unroll
+  for (int j = 0; j < PF_PIECES; ++j) {
+    st.kok[j] = true;
+    st.vkeys[j] = 8;
+    st.k[j] = ld8(kbase + ((int64_t)pg.k[j] * page_stride + iv.koff[j]));
+    st.v[j] = ld8(vbase + ((int64_t)pg.v[j] * page_stride + iv.voff[j]));
+  }
+}
+
 // the LDS writes of this wave done, every wave at the same point, nothing moved across by the compiler
 __device__ __forceinline__ void pf_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -673,6 +721,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int last = min(tr.pos_last, seg_hi - 1);   // the same key range for every wave of the workgroup
   const float c = a.scale * 1.4426950408889634f;
   (void)c;
+  StagedInvariants inv;
+  pf_invariants(a, kvh, tid, inv);
 
   // every wave runs every round (a wave without columns in a round masks everything and writes nothing)
   for (int c_base = 0; c_base < ncols; c_base += 4 * 16 * CT) {
@@ -722,9 +772,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       pf_barrier();                                  // block t0 is in buffer cur
       // the next block, into registers; the page ids of the one after it
       const bool inside1 = a.window == 0 && t0 + 64 <= L, inside2 = a.window == 0 && t0 + 96 <= L;
-      if (inside1) pf_fetch<true>(a, pg, kvh, t0 + 32, L, tile_lo, tid, stg);
+      if (inside1) pf_fetch_inside(a, pg, t0 + 32, inv, stg);
       else pf_fetch<false>(a, pg, kvh, t0 + 32, L, tile_lo, tid, stg);
-      if (inside2) pf_lookup<true>(a, bt, t0 + 64, L, tile_lo, tid, pg);
+      if (inside2) pf_lookup_inside(a, bt, t0 + 64, inv, pg);
       else pf_lookup<false>(a, bt, t0 + 64, L, tile_lo, tid, pg);
       const unsigned char* kb = pf_lds + cur * PF_BUF;
       const unsigned char* vb = kb + 32 * PF_KROW;
