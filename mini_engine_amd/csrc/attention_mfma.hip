@@ -1120,11 +1120,7 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   return 0;
 }
 
-// Bytes of scratch the decode path needs for (num_seqs, Hq, num_parts): out, m, l.
-extern "C" int64_t me_attn_decode_scratch_floats(int num_seqs, int Hq, int num_parts) {
-  return (int64_t)num_seqs * Hq * num_parts * (HD + 2);
-}
-
+// Scratch of the split decode path: num_seqs * Hq * num_parts * (HD + 2) floats (out, m, l per partition).
 extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                               const void* k_cache, const void* v_cache, const int32_t* block_tables,
                               int bt_stride, const int32_t* context_lens, int num_seqs, int Hq, int Hkv,

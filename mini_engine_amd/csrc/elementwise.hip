@@ -5,6 +5,7 @@
 // Here each is one kernel; the residual stream is kept in float32 and the sum, the
 // mean of squares and the scaling are computed in float32.
 #include "common.h"
+#include "errors.inc"   // the core library's error channel lives in this file
 
 
 // ------------------------------------------------------------------ gather rows

@@ -79,17 +79,17 @@ sample_merge_kernel(const float* __restrict__ part_v, const int32_t* __restrict_
   if (threadIdx.x == 0) out[row] = best_i == 0x7fffffff ? 0 : best_i;
 }
 
-// Scratch floats needed for S rows: (value, index) per chunk.
-extern "C" int me_sample_chunks(int V) { return V >= 16384 ? 32 : (V >= 2048 ? 4 : 1); }
+// Workgroups that share a row's vocabulary; the scratch holds (value, index) per row and chunk.
+static int sample_chunks(int V) { return V >= 16384 ? 32 : (V >= 2048 ? 4 : 1); }
 
 // keys: [S, 2] uint32 per row; temperatures: [S] float32 (0 = greedy); out: [S] int32;
-// scratch: 2 * S * me_sample_chunks(V) 4-byte words.
+// scratch: 2 * S * 32 4-byte words suffice for any vocabulary.
 extern "C" int me_sample(const float* logits, int64_t ld, const float* temperatures, const uint32_t* keys,
                          int32_t* out, void* scratch, int S, int V, hipStream_t stream) {
   if (S == 0) return 0;
   ME_CHECK(V >= 1 && ld >= V, "sample: bad vocabulary size or row stride");
   ME_CHECK(S <= 65535, "sample: too many rows (%d)", S);
-  const int chunks = me_sample_chunks(V);
+  const int chunks = sample_chunks(V);
   const int chunk = (V + chunks - 1) / chunks;
   float* pv = (float*)scratch;
   int32_t* pi = (int32_t*)scratch + (int64_t)S * chunks;

@@ -28,7 +28,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
-CORE_SOURCES = ["core_runtime.hip", "elementwise.hip", "rope_kv.hip", "attention_simple.hip",
+CORE_SOURCES = ["elementwise.hip", "rope_kv.hip", "attention_simple.hip",
                 "gemm.hip", "gemm_library.hip", "sampling.hip"]
 ATTN_SOURCE = "attention_mfma.hip"
 HEADERS = ["common.h", "errors.inc"]
@@ -80,16 +80,37 @@ def _writable_dir(path: str) -> bool:
         return False
 
 
+def _own_private_dir(path: str) -> bool:
+    """Whether `path` is a real folder of this user that nobody else can write to or read."""
+    try:
+        st = os.lstat(path)
+    except OSError:
+        return False
+    import stat
+    return stat.S_ISDIR(st.st_mode) and st.st_uid == os.getuid() and (st.st_mode & 0o077) == 0
+
+
+_fallback: str | None = None
+
+
 def _fallback_dir() -> str:
-    base = os.path.join(tempfile.gettempdir(), f"mini_engine_amd-{os.getuid()}")
-    os.makedirs(base, mode=0o700, exist_ok=True)
-    return base
+    """A per-user folder under the temp directory. A folder of that name that is someone else's, a link,
+    or open to others is never used (a library planted there would be loaded): a fresh one is made."""
+    global _fallback
+    if _fallback is None:
+        base = os.path.join(tempfile.gettempdir(), f"mini_engine_amd-{os.getuid()}")
+        try:
+            os.mkdir(base, 0o700)
+        except FileExistsError:
+            pass
+        _fallback = base if _own_private_dir(base) else tempfile.mkdtemp(prefix=f"mini_engine_amd-{os.getuid()}-")
+    return _fallback
 
 
 def _lib_dirs() -> list:
     dirs = [PKG_LIB]
-    fb = os.path.join(tempfile.gettempdir(), f"mini_engine_amd-{os.getuid()}")
-    if os.path.isdir(fb):
+    fb = _fallback or os.path.join(tempfile.gettempdir(), f"mini_engine_amd-{os.getuid()}")
+    if _own_private_dir(fb):
         dirs.append(fb)
     return dirs
 

@@ -96,7 +96,6 @@ def mixed_with_reuse(env, name):
         parts, ended = {}, []
         for r in live:
             plan = portions[r]
-            k = len([1 for _ in range(0)])
             if plan:
                 c = plan.pop(0)
             else:
