@@ -6,6 +6,8 @@
 // on which other requests share the step (the reference draws from the global generator for the
 // whole [S, V] matrix).
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
 
 __device__ __forceinline__ uint32_t fmix32(uint32_t h) {
   h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
@@ -82,11 +84,8 @@ sample_merge_kernel(const float* __restrict__ part_v, const int32_t* __restrict_
 // Workgroups that share a row's vocabulary; the scratch holds (value, index) per row and chunk.
 static int sample_chunks(int V) { return V >= 16384 ? 32 : (V >= 2048 ? 4 : 1); }
 
-// keys: [S, 2] uint32 per row; temperatures: [S] float32 (0 = greedy); out: [S] int32;
-// scratch: 2 * S * 32 4-byte words suffice for any vocabulary.
-extern "C" int me_sample(const float* logits, int64_t ld, const float* temperatures, const uint32_t* keys,
+static int launch_sample(const float* logits, int64_t ld, const float* temperatures, const uint32_t* keys,
                          int32_t* out, void* scratch, int S, int V, hipStream_t stream) {
-  if (S == 0) return 0;
   ME_CHECK(V >= 1 && ld >= V, "sample: bad vocabulary size or row stride");
   ME_CHECK(S <= 65535, "sample: too many rows (%d)", S);
   const int chunks = sample_chunks(V);
@@ -98,4 +97,48 @@ extern "C" int me_sample(const float* logits, int64_t ld, const float* temperatu
   sample_merge_kernel<<<dim3(S), dim3(64), 0, stream>>>(pv, pi, out, chunks);
   ME_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int me_sample(const float* logits, int64_t ld, const float* temperatures, const uint32_t* keys,
+                         int32_t* out, void* scratch, int S, int V, hipStream_t stream) {
+  if (S == 0) return 0;
+  ME_CHECK(scratch != nullptr, "sample: no scratch memory given");
+  return launch_sample(logits, ld, temperatures, keys, out, scratch, S, V, stream);
+}
+
+// ---- the form that allocates nothing: its partial results live in this array.
+// In host code the array's name is only a stand-in; the address that kernels and copies may use is
+// asked for once per device (each GPU holds its own copy at its own address) and kept here.
+static __device__ __align__(256) uint32_t g_sample_scratch[2 * ME_SAMPLE_STATIC_MAX_ROWS * 32];
+
+#define ME_MAX_DEVICES 64
+static void* g_sample_scratch_ptr[ME_MAX_DEVICES];      // per device; nullptr: not asked yet
+static std::mutex g_sample_scratch_guard;
+
+static int sample_scratch_of_current_device(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  ME_CHECK(e == hipSuccess, "sample_static: hipGetDevice: %s", hipGetErrorString(e));
+  ME_CHECK(dev >= 0 && dev < ME_MAX_DEVICES, "sample_static: device %d beyond the %d this library keeps scratch for",
+           dev, ME_MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(g_sample_scratch_guard);
+  if (g_sample_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_sample_scratch));
+    ME_CHECK(e == hipSuccess && p != nullptr, "sample_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_sample_scratch_ptr[dev] = p;
+  }
+  *ptr = g_sample_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int me_sample_static(const float* logits, int64_t ld, const float* temperatures, const uint32_t* keys,
+                                int32_t* out, int S, int V, hipStream_t stream) {
+  if (S == 0) return 0;
+  ME_CHECK(S > 0 && S <= ME_SAMPLE_STATIC_MAX_ROWS,
+           "sample_static: %d rows, the built-in scratch holds %d at most (use me_sample with a workspace)",
+           S, ME_SAMPLE_STATIC_MAX_ROWS);
+  void* scratch = nullptr;
+  if (int rc = sample_scratch_of_current_device(&scratch)) return rc;
+  return launch_sample(logits, ld, temperatures, keys, out, scratch, S, V, stream);
 }

@@ -31,7 +31,7 @@ HIPCC_FLAGS = [
 CORE_SOURCES = ["elementwise.hip", "rope_kv.hip", "attention_simple.hip",
                 "gemm.hip", "gemm_library.hip", "sampling.hip"]
 ATTN_SOURCE = "attention_mfma.hip"
-HEADERS = ["common.h", "errors.inc"]
+HEADERS = ["common.h", "errors.inc", "sampling.h"]
 # Head sizes built by build_all(): the sizes of the benchmark models and of the test configurations.
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 128)
 
