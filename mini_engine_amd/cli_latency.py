@@ -61,15 +61,15 @@ def apply_setting(engine, name: str) -> None:
     """`pf`: whole prompts first, 16,384 tokens a step. `c<N>`: chunked prefill under N tokens a step."""
     sched = engine.scheduler
     if name == "pf":
-        sched.enable_chunked_prefill, sched.max_num_batched_tokens = False, ENGINE_BUDGET
+        sched.chunked, sched.token_budget = False, ENGINE_BUDGET
     elif name.startswith("c") and name[1:].isdigit() and 0 < int(name[1:]) <= ENGINE_BUDGET:
-        sched.enable_chunked_prefill, sched.max_num_batched_tokens = True, int(name[1:])
+        sched.chunked, sched.token_budget = True, int(name[1:])
     else:
         raise ValueError(f"setting {name!r}: expected 'pf' or 'c<tokens>' with at most {ENGINE_BUDGET} tokens")
     if name == "pf" and ENGINE_BUDGET < sched.max_model_len:
         raise ValueError(f"setting 'pf' needs a whole prompt in one step: max_model_len {sched.max_model_len} > {ENGINE_BUDGET}")
-    if sched.max_num_batched_tokens < sched.max_num_seqs:
-        raise ValueError(f"setting {name!r}: the budget must cover one token for each of {sched.max_num_seqs} requests")
+    if sched.token_budget < sched.max_live:
+        raise ValueError(f"setting {name!r}: the budget must cover one token for each of {sched.max_live} requests")
     engine.manager.forget_prefixes()
 
 

@@ -2,13 +2,13 @@
 
 Added beside the reference's fields: ``dtype`` (bfloat16 or a true float32 path),
 ``seed`` (sampling noise is a function of seed, request and output index),
-``enable_prefix_caching``, ``use_graphs`` and ``run_ahead``; ``num_kvcache_blocks`` may be given
+``enable_prefix_caching``, ``use_graphs``, ``run_ahead`` and ``random_weights``; ``num_kvcache_blocks`` may be given
 (the reference always sizes the pool itself, ``engine/model_runner.py:46-48``).
 """
 from __future__ import annotations
 
 import os
-from dataclasses import dataclass, field
+from dataclasses import dataclass, field, fields
 
 from .model_config import ConfigError, load_model_config
 
@@ -33,7 +33,15 @@ class EngineConfig:
     enable_prefix_caching: bool = True
     use_graphs: bool = True
     run_ahead: bool = True                # launch the next plain decode step before this one's tokens are fetched
+    random_weights: int | None = None     # a seed: the folder needs only config.json, weights are drawn on the device
     model_config: object = field(default=None, repr=False)
+
+    @classmethod
+    def from_options(cls, model: str, options: dict) -> "EngineConfig":
+        """The options this class knows, out of a mapping that may hold others (the reference's entry
+        point takes any keyword and passes on what its config knows, engine/llm_engine.py:13-16)."""
+        known = {f.name for f in fields(cls)} - {"model"}
+        return cls(model, **{name: options[name] for name in options.keys() & known})
 
     def __post_init__(self):
         self.model = os.path.expanduser(self.model)

@@ -61,7 +61,7 @@ def _pad4(n: int) -> int:
 
 class ModelRunner:
     def __init__(self, model, manager: CacheManager, dtype: torch.dtype, device, max_positions: int,
-                 poison_cache: bool = False, use_graphs: bool = False):
+                 poison_cache: bool = False, use_graphs: bool = False, max_decode_rows: int = 256):
         self.model = model
         self.manager = manager
         self.dtype = dtype
@@ -79,7 +79,7 @@ class ModelRunner:
         self.graphs = None
         if use_graphs:
             from .graphs import DecodeGraphs
-            self.graphs = DecodeGraphs(self, capture=self.device.type == "cuda")
+            self.graphs = DecodeGraphs(self, max_bucket=max_decode_rows, capture=self.device.type == "cuda")
         self._host = [None, None]
         self._events = [None, None]
         self._dev = None
@@ -127,7 +127,6 @@ class ModelRunner:
         through the cache manager for positions up to start + len(tokens)."""
         if not entries:
             return None
-        ps = self.manager.page_size
         if len({e.req for e in entries}) != len(entries):
             seen = set()
             for e in entries:
@@ -162,19 +161,28 @@ class ModelRunner:
         # decodes (one new token) first, the others after, each kept in the caller's order
         order = [i for i, e in enumerate(entries) if len(e.tokens) == 1] + \
                 [i for i, e in enumerate(entries) if len(e.tokens) != 1]
-        Dn = sum(1 for e in entries if len(e.tokens) == 1)
-        B = len(entries)
-        q_lens = [len(entries[i].tokens) for i in order]
-        starts = [entries[i].start for i in order]
+        G = self.manager.num_groups if self.plan.group_needs else 0
+        tables = [[self.manager.block_table(entries[i].req, g) for i in order] for g in range(G)]
+        slots_of = [self.manager.state_slot(entries[i].req) for i in order]
+        lens = [len(entries[i].tokens) for i in order]
+        cu = np.concatenate(([0], np.cumsum(lens)))
+        offset_of = {order[j]: int(cu[j]) for j in range(len(order))}
+        rows = [offset_of[i] + w for i, e in enumerate(entries) for w in e.want]      # in the caller's order
+        return self._run([entries[i].tokens for i in order], [entries[i].start for i in order], tables, slots_of, rows,
+                         names=[entries[i].req for i in order])
+
+    def _run(self, token_lists: list, starts: list, tables: list, slots_of: list, rows: list, names: list | None = None):
+        """One eager pass. Requests in step order (single tokens first): their tokens, first positions,
+        per group their block tables, their state slots; `rows`: token rows that want logits."""
+        ps = self.manager.page_size
+        B = len(token_lists)
+        q_lens = [len(t) for t in token_lists]
+        Dn = sum(1 for q in q_lens if q == 1)
         T = sum(q_lens)
         cu = np.zeros(B + 1, dtype=np.int64)
         np.cumsum(q_lens, out=cu[1:])
-        G = self.manager.num_groups if self.plan.group_needs else 0
-        tables = [[self.manager.block_table(entries[i].req, g) for i in order] for g in range(G)]
+        G = len(tables)
         MB = [max(1, max(len(t) for t in tables[g])) for g in range(G)]
-        # rows that want logits, in the caller's order
-        offset_of = {order[j]: int(cu[j]) for j in range(B)}
-        rows = [offset_of[i] + w for i, e in enumerate(entries) for w in e.want]
         R = len(rows)
 
         # ---- one packed int32 array: offsets (each segment padded to 16 bytes)
@@ -194,7 +202,7 @@ class ModelRunner:
             o, size = seg[name]
             a[o:o + size] = values
 
-        tok = np.concatenate([np.asarray(entries[i].tokens, dtype=np.int64) for i in order])
+        tok = np.concatenate([np.asarray(t, dtype=np.int64) for t in token_lists])
         if self.vocab_size is not None and (tok.min() < 0 or tok.max() >= self.vocab_size):
             raise ValueError(f"token id outside 0..{self.vocab_size - 1}")
         pos = np.concatenate([np.arange(s, s + q, dtype=np.int64) for s, q in zip(starts, q_lens)])
@@ -204,7 +212,6 @@ class ModelRunner:
         put("context_lens", [s + q for s, q in zip(starts, q_lens)])
         put("cu", cu)
         put("prefill_cu", cu[Dn:] - cu[Dn])
-        slots_of = [self.manager.state_slot(entries[i].req) for i in order]
         put("state_slots", slots_of)
         put("first_chunk", [1 if s == 0 else 0 for s in starts])
         if R:
@@ -218,7 +225,8 @@ class ModelRunner:
                 p = pos[cu[j]:cu[j + 1]]
                 pages = bt[j, p // ps] if p[-1] // ps < MB[g] else np.array([-1])
                 if (pages < 0).any():
-                    raise RuntimeError(f"request {entries[order[j]].req!r} has no page for a position it is "
+                    who = names[j] if names is not None else j
+                    raise RuntimeError(f"request {who!r} has no page for a position it is "
                                        f"about to write (group {g}); allocate before stepping")
                 slot[cu[j]:cu[j + 1]] = pages * ps + p % ps
             put(f"slots{g}", slot)
@@ -259,6 +267,41 @@ class ModelRunner:
         if not R:
             return None
         return self.model.logits(h, residual, view("rows")[:R])
+
+    # -- sizing by measurement -------------------------------------------------------------
+    @torch.inference_mode()
+    def measure_working_set(self, max_step_tokens: int, max_seqs: int, max_len: int) -> tuple:
+        """(bytes the largest step needs beyond what is allocated now, the same for the largest decode step).
+
+        Runs the two largest steps the engine's limits allow, a step of `max_step_tokens` prompt tokens
+        and a step in which `max_seqs` requests of `max_len` tokens decode, and reads the allocator's peak
+        (reference engine/model_runner.py:59-80 sizes its pool the same way). Every table entry names
+        page 0, so one page per group is all the cache this needs; what the steps write and read there
+        means nothing."""
+        if self.device.type != "cuda":
+            return 0, 0
+        ps = self.manager.page_size
+        G = len(self.plan.group_needs)
+        nslots = max(1, self.manager.num_state_slots)
+
+        def run(q_lens, starts, want_last):
+            cu = np.concatenate(([0], np.cumsum(q_lens)))
+            tables = [[[0] * -(-(s + q) // ps) for s, q in zip(starts, q_lens)] for _ in range(G)]
+            rows = [int(cu[j + 1]) - 1 for j in range(len(q_lens))] if want_last else []
+            torch.cuda.synchronize(self.device)
+            torch.cuda.reset_peak_memory_stats(self.device)
+            before = torch.cuda.memory_allocated(self.device)
+            out = self._run([[0] * q for q in q_lens], starts, tables, [j % nslots for j in range(len(q_lens))], rows)
+            torch.cuda.synchronize(self.device)
+            del out
+            return torch.cuda.max_memory_allocated(self.device) - before
+
+        m = max(1, min(max_len, max_step_tokens))
+        n = max(1, min(max_step_tokens // m, max_seqs))
+        prompt_peak = run([m] * n, [0] * n, True)
+        decode_peak = run([1] * max_seqs, [max_len - 1] * max_seqs, True)
+        torch.cuda.empty_cache()
+        return max(prompt_peak, decode_peak), decode_peak
 
     # -- sampling --------------------------------------------------------------------------
     @torch.inference_mode()

@@ -1,30 +1,87 @@
-"""Admission, chunked prefill under a token budget, decoding, finishing and freeing
-(reference engine/scheduler.py:7-173; the policies and their order are the reference's).
+"""Which requests run how many tokens in the next step, and what becomes of them afterwards.
 
-What happens when pages run out: a running request that cannot get the pages for its next
-tokens makes the scheduler preempt another running request that is not yet part of the step
-(FCFS: the one admitted last; priority: the least urgent), i.e. free everything it holds and
-put it back at the head of the waiting queue, from where it is later recomputed (prompt and
-generated tokens as one prompt, possibly hitting its own still-cached pages). If the
-requester is the only candidate left, it is preempted itself. A step in which anything was
-preempted admits nothing new. A waiting request that does not fit simply waits
-(head-of-line: nothing overtakes it).
+The policy is the reference's (engine/scheduler.py:97-155): under chunked prefill a step is filled
+from three sources in turn, while the token budget lasts: live requests that owe one token (they
+decode), live requests that owe more (their prompt is partly done), and the head of the queue;
+without chunked prefill whole prompts are admitted first and only a step that admits nothing
+decodes. Under FCFS the queue is served in order of arrival, under "priority" by (priority, arrival).
+
+When pages run out (reference engine/scheduler.py:57-78): a live request that cannot get pages for
+its next tokens makes another live request, one not yet in the step, give back everything it holds;
+that one returns to the queue (FCFS: to its head) and is later fed again from its first token, its
+generated tokens included, possibly finding its own pages still cached. FCFS evicts whoever was
+admitted last, "priority" the least urgent. A requester that is the last candidate evicts itself and
+the step goes on without it. A step in which anyone was evicted admits nobody. A queued request that
+does not fit waits, and nobody overtakes it. A step that could take nobody raises.
+
+After a step is launched its requests are moved on (`advance`) before their sampled tokens are known,
+so that the next step can be planned and launched meanwhile; `settle` puts the tokens in when they
+arrive, and `release_finished` gives back what ended requests hold once no launched step writes there.
 """
 from __future__ import annotations
 
 from collections import deque
 
 from ..cache.manager import CacheManager
-from .sequence import Sequence, SequenceStatus
+from .request import Phase, Request
+
+UNKNOWN = -1       # stands in a request's tokens for a sampled token that has not reached the host yet
+
+
+class ArrivalOrder:
+    """First come, first served; an evicted request goes back to the head of the queue."""
+
+    def enqueue(self, queue: deque, req: Request, returning: bool) -> None:
+        if returning:
+            queue.appendleft(req)
+        else:
+            queue.append(req)
+
+    def evict_from(self, candidates: list) -> Request:
+        return candidates[-1]                  # live requests are kept in order of admission: the newest
+
+
+class UrgencyOrder:
+    """Lower priority value first, earlier arrival first among equals; the least urgent is evicted."""
+
+    @staticmethod
+    def rank(req: Request) -> tuple:
+        return req.priority, req.arrived
+
+    def enqueue(self, queue: deque, req: Request, returning: bool) -> None:
+        at = sum(1 for other in queue if self.rank(other) <= self.rank(req))     # the queue is kept sorted
+        queue.insert(at, req)
+
+    def evict_from(self, candidates: list) -> Request:
+        return max(candidates, key=self.rank)
+
+
+ORDERS = {"fcfs": ArrivalOrder, "priority": UrgencyOrder}
+
+
+class _Plan:
+    """The step being put together."""
+
+    def __init__(self, room: int):
+        self.room = room                   # tokens the budget still allows
+        self.taken: list = []              # requests, in the order they were taken
+        self.members: set = set()          # their ids
+        self.evictions = 0
+
+    def take(self, req: Request, n: int) -> None:
+        req.portion = n
+        self.room -= n
+        self.taken.append(req)
+        self.members.add(req.id)
 
 
 class Scheduler:
     def __init__(self, config, manager: CacheManager):
-        self.max_num_seqs = config.max_num_seqs
-        self.max_num_batched_tokens = config.max_num_batched_tokens
-        self.long_prefill_token_threshold = config.long_prefill_token_threshold
-        self.enable_chunked_prefill = config.enable_chunked_prefill
-        self.policy = config.scheduling_policy
+        self.max_live = config.max_num_seqs
+        self.token_budget = config.max_num_batched_tokens
+        self.portion_cap = config.long_prefill_token_threshold      # 0: prompts are cut by the budget only
+        self.chunked = bool(config.enable_chunked_prefill)
+        self.order = ORDERS[config.scheduling_policy]()
         self.eos = config.eos
         self.max_model_len = config.max_model_len
         self.manager = manager
@@ -33,228 +90,155 @@ class Scheduler:
         self.running: list = []
         self.num_preemptions = 0
 
-    def is_finished(self) -> bool:
-        return not self.waiting and not self.running
-
-    def next_step_is_plain_decoding(self) -> bool:
-        """Whether the next schedule() can only be: every running request decodes one token, nobody
-        waits, and pages cannot run out (one new page per request at most). Such a step needs no
-        token value and no request's pages back, so it may be launched before the step in flight
-        has delivered its tokens."""
-        if self.waiting or not self.running or len(self.running) > self.max_num_batched_tokens:
-            return False
-        need = len(self.running)
-        if any(self.manager.num_free_pages(g) < need for g in range(self.manager.num_groups)):
-            return False
-        return all(len(s.token_ids) - s.num_computed_tokens == 1 for s in self.running)
-
-    # -- admission ---------------------------------------------------------------------------
-    def add(self, seq: Sequence) -> None:
-        total = seq.num_prompt_tokens + seq.sampling_params.max_tokens
-        if total > self.max_model_len:
-            raise ValueError(f"prompt+max_tokens={total} exceeds max_model_len={self.max_model_len}")
-        need = self.manager.pages_needed(total)
+    # -- requests in ---------------------------------------------------------------------------
+    def add(self, req: Request) -> None:
+        """Queue a request, or refuse one that could never finish (reference engine/scheduler.py:26-33)."""
+        most = req.prompt_len + req.params.max_tokens
+        if most > self.max_model_len:
+            raise ValueError(f"prompt+max_tokens={most} exceeds max_model_len={self.max_model_len}")
         for g in range(self.manager.num_groups):
-            if need > self.manager.num_pages(g):
-                raise ValueError(f"needs {need} cache pages, the pool has {self.manager.num_pages(g)}")
-        self._push_waiting(seq)
+            need, have = self.manager.pages_needed(most, g), self.manager.num_pages(g)
+            if need > have:
+                raise ValueError(f"needs {need} cache pages, the pool has {have}")
+        self.order.enqueue(self.waiting, req, returning=False)
 
-    @staticmethod
-    def _key(seq: Sequence):
-        return (seq.priority, seq.arrival_time)
+    def is_finished(self) -> bool:
+        return not (self.waiting or self.running)
 
-    def _push_waiting(self, seq: Sequence, front: bool = False) -> None:
-        if self.policy == "priority":
-            i = 0
-            while i < len(self.waiting) and self._key(self.waiting[i]) <= self._key(seq):
-                i += 1
-            self.waiting.insert(i, seq)
-        elif front:
-            self.waiting.appendleft(seq)
+    # -- planning a step -----------------------------------------------------------------------
+    def schedule(self) -> list:
+        """The requests of the next step; each one's `portion` says how many of its tokens run."""
+        plan = _Plan(self.token_budget)
+        if self.chunked:
+            self._continue_live(plan)
+            if not plan.evictions:
+                self._admit(plan, whole_prompts=False)
         else:
-            self.waiting.append(seq)
+            self._admit(plan, whole_prompts=True)
+            if not plan.taken:
+                self._continue_live(plan)
+        if not plan.taken:
+            raise RuntimeError("nothing schedulable: the cache pool or the token budget is too small "
+                               "for the request at the head of the queue")
+        return plan.taken
 
-    def _cap(self, owed: int, budget: int) -> int:
-        n = owed
-        if 0 < self.long_prefill_token_threshold < n:
-            n = self.long_prefill_token_threshold
-        return min(n, budget)
+    def _portion(self, owed: int, room: int) -> int:
+        """How much of `owed` tokens runs now (reference engine/scheduler.py:51-55)."""
+        if self.portion_cap and owed > self.portion_cap:
+            owed = self.portion_cap
+        return owed if owed < room else room
 
-    # -- running out of pages ----------------------------------------------------------------
-    def _pick_victim(self, scheduled_ids: set) -> Sequence:
-        cands = [s for s in self.running if s.seq_id not in scheduled_ids]
-        if self.policy == "priority":
-            return max(cands, key=self._key)
-        return cands[-1]
+    def _continue_live(self, plan: _Plan) -> None:
+        """Live requests, those that decode before those whose prompt is under way."""
+        turn = sorted(self.running, key=lambda r: r.owed != 1)            # stable: admission order within each kind
+        for req in turn:
+            if plan.room <= 0:
+                return
+            if req.phase is not Phase.LIVE:                               # evicted a moment ago by one before it
+                continue
+            n = self._portion(req.owed, plan.room)
+            if not self._pages_for(req, n, plan):
+                return
+            plan.take(req, n)
 
-    def _preempt(self, seq: Sequence) -> None:
-        self.running.remove(seq)
-        seq.status = SequenceStatus.WAITING
-        seq.num_scheduled_tokens = 0
-        self._release(seq)
-        self._push_waiting(seq, front=True)
-        self.num_preemptions += 1
-
-    def _release(self, seq: Sequence) -> None:
-        if self.manager.holds(seq.seq_id):
-            self.manager.free(seq.seq_id)
-        seq.num_computed_tokens = 0
-        seq.num_cached_tokens = 0
-
-    def _allocate_or_preempt(self, seq: Sequence, n: int, scheduled_ids: set) -> bool:
-        while not self.manager.allocate(seq.seq_id, seq.num_computed_tokens, n):
-            victim = self._pick_victim(scheduled_ids)
-            self._preempt(victim)
-            if victim is seq:
+    def _pages_for(self, req: Request, n: int, plan: _Plan) -> bool:
+        """Pages for the next n tokens of a live request, evicting others if that is what it takes.
+        False: it had to evict itself."""
+        while not self.manager.allocate(req.id, req.in_cache, n):
+            loser = self.order.evict_from([r for r in self.running if r.id not in plan.members])
+            self._evict(loser)
+            plan.evictions += 1
+            if loser is req:
                 return False
         return True
 
-    def _try_start(self, seq: Sequence, budget: int, whole: bool) -> int:
-        """Admit the head of the waiting queue with as many tokens as fit; 0 if it has to wait."""
-        hit = self.manager.find_prefix_hit(seq.token_ids)
-        cached = hit.num_pages * self.page_size
-        owed = seq.num_tokens - cached
-        n = owed if whole else self._cap(owed, budget)
-        if n > budget or n < 1:
-            return 0
-        if not self.manager.allocate(seq.seq_id, 0, n, hit):
-            return 0
-        seq.num_computed_tokens = cached
-        seq.num_cached_tokens = cached
-        return n
+    def _evict(self, req: Request) -> None:
+        self.running.remove(req)
+        self._give_back(req)
+        req.phase = Phase.QUEUED
+        req.portion = 0
+        self.order.enqueue(self.waiting, req, returning=True)
+        self.num_preemptions += 1
 
-    def _start(self, seq: Sequence, n: int, scheduled: list, ids: set) -> None:
-        self.waiting.popleft()
-        seq.status = SequenceStatus.RUNNING
-        seq.num_scheduled_tokens = n
-        self.running.append(seq)
-        scheduled.append(seq)
-        ids.add(seq.seq_id)
+    def _give_back(self, req: Request) -> None:
+        if self.manager.holds(req.id):
+            self.manager.free(req.id)
+        req.in_cache = req.from_prefix = 0
 
-    # -- one step's batch --------------------------------------------------------------------
-    def schedule(self) -> list:
-        scheduled = self._schedule_chunked() if self.enable_chunked_prefill else self._schedule_prefill_first()
-        if not scheduled:
-            raise RuntimeError("nothing schedulable: the cache pool or the token budget is too small "
-                               "for the request at the head of the queue")
-        return scheduled
+    def _admit(self, plan: _Plan, whole_prompts: bool) -> None:
+        """The head of the queue, again and again, until one does not fit (nobody overtakes it)."""
+        while self.waiting and plan.room > 0 and len(self.running) < self.max_live:
+            req = self.waiting[0]
+            hit = self.manager.find_prefix_hit(req.tokens)
+            reused = hit.num_pages * self.page_size
+            owed = len(req.tokens) - reused
+            n = owed if whole_prompts else self._portion(owed, plan.room)
+            if n < 1 or n > plan.room or not self.manager.allocate(req.id, 0, n, hit):
+                return
+            self.waiting.popleft()
+            req.in_cache = req.from_prefix = reused
+            req.phase = Phase.LIVE
+            self.running.append(req)
+            plan.take(req, n)
 
-    def _schedule_chunked(self) -> list:
-        budget = self.max_num_batched_tokens
-        scheduled, ids = [], set()
-        preempted = False
-        decodes, partials = [], []
-        for s in self.running:
-            (decodes if len(s.token_ids) - s.num_computed_tokens == 1 else partials).append(s)
-        allocate = self.manager.allocate
-        for seq in decodes + partials:
-            if budget == 0:
-                break
-            if seq.status != SequenceStatus.RUNNING:     # preempted earlier in this loop
-                continue
-            owed = len(seq.token_ids) - seq.num_computed_tokens
-            n = 1 if owed == 1 else self._cap(owed, budget)
-            if not allocate(seq.seq_id, seq.num_computed_tokens, n):     # pages ran out: the slow way
-                before = self.num_preemptions
-                ok = self._allocate_or_preempt(seq, n, ids)
-                preempted |= self.num_preemptions > before
-                if not ok:
-                    break
-            seq.num_scheduled_tokens = n
-            budget -= n
-            scheduled.append(seq)
-            ids.add(seq.seq_id)
-        if preempted:
-            return scheduled
-        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
-            seq = self.waiting[0]
-            n = self._try_start(seq, budget, whole=False)
-            if n == 0:
-                break
-            self._start(seq, n, scheduled, ids)
-            budget -= n
-        return scheduled
+    def next_step_is_plain_decoding(self) -> bool:
+        """Whether the next schedule() can only be: every live request decodes one token, nobody is
+        queued, and pages cannot run out (one new page per request at most). Such a step needs no
+        token value and no request's pages back, so it may be launched before the step in flight
+        has delivered its tokens."""
+        live = len(self.running)
+        if self.waiting or not live or live > self.token_budget:
+            return False
+        if any(self.manager.num_free_pages(g) < live for g in range(self.manager.num_groups)):
+            return False
+        return all(r.owed == 1 for r in self.running)
 
-    def _schedule_prefill_first(self) -> list:
-        budget = self.max_num_batched_tokens
-        scheduled, ids = [], set()
-        while self.waiting and len(self.running) < self.max_num_seqs:
-            seq = self.waiting[0]
-            n = self._try_start(seq, budget, whole=True)
-            if n == 0:
-                break
-            self._start(seq, n, scheduled, ids)
-            budget -= n
-        if scheduled:
-            return scheduled
-        for seq in list(self.running):
-            if seq.status != SequenceStatus.RUNNING:
-                continue
-            if not self._allocate_or_preempt(seq, seq.num_uncomputed_tokens, ids):
-                break
-            seq.num_scheduled_tokens = seq.num_uncomputed_tokens
-            scheduled.append(seq)
-            ids.add(seq.seq_id)
-        return scheduled
-
-    # -- after the step ----------------------------------------------------------------------
-    PLACEHOLDER = -1       # stands in a request's tokens for a sampled token that has not reached the host yet
-
-    def advance(self, seqs: list) -> list:
-        """Bookkeeping of a step that has been launched, before its tokens are known: the scheduled
-        tokens count as computed; a request whose step reached the end of what is known gets a
-        placeholder for the token being sampled, and leaves `running` if that token is its last by
-        max_tokens. Returns the requests that sample, in order."""
-        samplers = []
+    # -- after a step --------------------------------------------------------------------------
+    def advance(self, reqs: list) -> list:
+        """Bookkeeping of a step that has been launched, before its tokens are known: the portions
+        count as cached; a request whose portion reached the end of what is known gets a placeholder
+        for the token being sampled, and leaves `running` if that token is its last by max_tokens.
+        Returns the requests that sample, in order."""
+        sampling = []
         publish = self.manager.publish_full_pages if self.manager.prefix_caching else None
-        for seq in seqs:
-            seq.num_computed_tokens += seq.num_scheduled_tokens
-            seq.num_scheduled_tokens = 0
-            if publish is not None:                      # pages whose tokens are all computed and all known
-                known = len(seq.token_ids) - (seq.token_ids[-1] == self.PLACEHOLDER)
-                publish(seq.seq_id, seq.token_ids, min(seq.num_computed_tokens, known))
-            if seq.num_computed_tokens != len(seq.token_ids):
+        for req in reqs:
+            req.in_cache += req.portion
+            req.portion = 0
+            if publish is not None:                      # pages whose tokens are all cached and all known
+                known = len(req.tokens) - (req.tokens[-1] == UNKNOWN)
+                publish(req.id, req.tokens, min(req.in_cache, known))
+            if req.owed:
                 continue
-            seq.token_ids.append(self.PLACEHOLDER)
-            samplers.append(seq)
-            if len(seq.token_ids) - seq.num_prompt_tokens == seq.sampling_params.max_tokens:
-                seq.status = SequenceStatus.FINISHED
-                self.running.remove(seq)            # its pages are given back when its token is settled
-        return samplers
+            req.tokens.append(UNKNOWN)
+            sampling.append(req)
+            if req.num_generated == req.params.max_tokens:
+                req.phase = Phase.DONE
+                self.running.remove(req)                 # its pages are given back when its token is settled
+        return sampling
 
-    def settle(self, samplers: list, token_ids: list, index_of: list) -> list:
-        """The sampled tokens have arrived: index_of[i] is where samplers[i]'s placeholder stands.
-        Puts them in, publishes full pages, finishes on the end token and frees what finished
-        requests hold. A request that an earlier token already finished (it ran one step ahead of
-        its end token) is skipped. Returns the requests that got a token."""
-        emitted = []
+    def settle(self, sampling: list, token_ids: list, places: list) -> list:
+        """The sampled tokens have arrived: places[i] is where sampling[i]'s placeholder stands.
+        Puts them in, publishes pages that are now full, ends requests on the end token. A request
+        that an earlier token already ended (it ran one step ahead of its end token) is skipped.
+        Returns the requests that got a token."""
+        got = []
         publish = self.manager.publish_full_pages if self.manager.prefix_caching else None
-        for seq, token_id, at in zip(samplers, token_ids, index_of):
-            if at >= len(seq.token_ids):                 # cut off behind its end token: this token is not wanted
+        for req, token, at in zip(sampling, token_ids, places):
+            if at >= len(req.tokens):                    # cut off behind its end token: this token is not wanted
                 continue
-            seq.token_ids[at] = int(token_id)
-            emitted.append(seq)
-            if publish is not None and self.manager.holds(seq.seq_id):
-                publish(seq.seq_id, seq.token_ids, min(seq.num_computed_tokens, at + 1))
-            if token_id == self.eos and not seq.sampling_params.ignore_eos:
-                del seq.token_ids[at + 1:]               # a placeholder of a step that ran ahead
-                if seq.status != SequenceStatus.FINISHED:
-                    seq.status = SequenceStatus.FINISHED
-                    self.running.remove(seq)
-        return emitted
+            req.tokens[at] = int(token)
+            got.append(req)
+            if publish is not None and self.manager.holds(req.id):
+                publish(req.id, req.tokens, min(req.in_cache, at + 1))
+            if token == self.eos and not req.params.ignore_eos:
+                del req.tokens[at + 1:]                  # a placeholder of a step that ran ahead
+                if req.phase is not Phase.DONE:
+                    req.phase = Phase.DONE
+                    self.running.remove(req)
+        return got
 
-    def release_finished(self, seqs: list) -> None:
-        """Give back what finished requests among `seqs` hold (once no step that writes to their pages is in flight)."""
-        for seq in seqs:
-            if seq.status == SequenceStatus.FINISHED and self.manager.holds(seq.seq_id):
-                self._release(seq)
-
-    def postprocess(self, seqs: list, token_ids: list) -> list:
-        """token_ids[i] is the token sampled for seqs[i], or None if it did not sample."""
-        at = {id(s): len(s.token_ids) for s in seqs}
-        samplers = self.advance(seqs)
-        wanted = {id(s) for s in samplers}
-        tokens = [t for s, t in zip(seqs, token_ids) if id(s) in wanted]
-        emitted = self.settle(samplers, tokens, [at[id(s)] for s in samplers])
-        self.release_finished(samplers)
-        return emitted
+    def release_finished(self, reqs: list) -> None:
+        """Give back what ended requests among `reqs` hold (once no step that writes to their pages is in flight)."""
+        for req in reqs:
+            if req.phase is Phase.DONE and self.manager.holds(req.id):
+                self._give_back(req)

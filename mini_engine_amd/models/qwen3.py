@@ -14,10 +14,12 @@ from .model import DecoderModel, WeightSource
 
 
 @register_architecture("Qwen3ForCausalLM")
-def build_qwen3(cfg: Qwen3Config, tied: bool | None = None) -> DecoderModel:
-    """`tied` resolves a config without `tie_word_embeddings` (the loader passes whether the
-    checkpoint stores `lm_head.weight`)."""
-    tie = cfg.tie_word_embeddings if cfg.tie_word_embeddings is not None else bool(tied)
+def build_qwen3(cfg: Qwen3Config, checkpoint_names=None) -> DecoderModel:
+    """A config without `tie_word_embeddings` is resolved by the checkpoint: the head is the embedding
+    matrix exactly when no `lm_head.weight` is stored (untied when there is no checkpoint at all)."""
+    tie = cfg.tie_word_embeddings
+    if tie is None:
+        tie = checkpoint_names is not None and "lm_head.weight" not in checkpoint_names
     h, D = cfg.hidden_size, cfg.head_dim
     Hq, Hkv = cfg.num_attention_heads, cfg.num_key_value_heads
     rotary = make_part("position_encoding", "rotary", head_dim=D, theta=cfg.rope_theta)   # one for all layers

@@ -36,9 +36,16 @@ def architectures() -> list:
     return sorted(_BUILDERS)
 
 
-def build_model(model_config, **kwargs):
-    """Build the (unloaded) model of a typed config."""
-    return builder_for(type(model_config).architecture_name)(model_config, **kwargs)
+def build_model(model_config, checkpoint_names=None):
+    """Build the (unloaded) model of a typed config. A builder that has a parameter `checkpoint_names`
+    is told which tensors the checkpoint stores (None: there is no checkpoint, weights will be drawn),
+    for architectures whose shape depends on it (a head that is stored or not)."""
+    import inspect
+
+    builder = builder_for(type(model_config).architecture_name)
+    if "checkpoint_names" in inspect.signature(builder).parameters:
+        return builder(model_config, checkpoint_names=checkpoint_names)
+    return builder(model_config)
 
 
 def _load_builtin() -> None:

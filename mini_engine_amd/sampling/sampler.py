@@ -30,15 +30,15 @@ class Sampler:
         self.runner = runner
         self.seed = seed
 
-    def __call__(self, logits, seqs: list) -> list:
-        """One token per row of float32 logits [S, V]; seqs[s] gives temperature, seed, identity
+    def __call__(self, logits, requests: list) -> list:
+        """One token per row of float32 logits [S, V]; requests[s] gives temperature, seed, identity
         and how many tokens the request has generated so far."""
-        return self.launch(logits, seqs).tokens()
+        return self.launch(logits, requests).tokens()
 
-    def launch(self, logits, seqs: list):
+    def launch(self, logits, requests: list):
         """The same, not waiting for the tokens: returns the runner's handle, whose tokens() fetches
         them. The next decode step of these requests may be started before that."""
-        temps = [s.sampling_params.temperature for s in seqs]
-        keys = [row_key(self.seed if s.sampling_params.seed is None else s.sampling_params.seed,
-                        s.sample_stream, s.num_completion_tokens) for s in seqs]
-        return self.runner.sample_async(logits, temps, keys, [s.seq_id for s in seqs])
+        temps = [r.params.temperature for r in requests]
+        keys = [row_key(self.seed if r.params.seed is None else r.params.seed, r.noise_stream, r.num_generated)
+                for r in requests]
+        return self.runner.sample_async(logits, temps, keys, [r.id for r in requests])

@@ -136,14 +136,16 @@ def load_weights(model, model_dir: str, device, dtype: torch.dtype, index: dict 
         handles.clear()
 
 
-def load_model(model_dir: str, device, dtype: torch.dtype, max_positions: int, model_config=None):
-    """config.json -> registry -> model -> weights -> finalize. Returns the ready model."""
+def load_model(model_dir: str, device, dtype: torch.dtype, max_positions: int, model_config=None,
+               random_weights: int | None = None):
+    """config.json -> registry -> model -> weights -> finalize. Returns the ready model.
+    `random_weights` (a seed): no checkpoint is read, every tensor is drawn on the device."""
     cfg = model_config or load_model_config(model_dir)
+    if random_weights is not None:
+        from .random_init import fill_random
+        return fill_random(build_model(cfg), random_weights, device, dtype, max_positions, on_device=True)
     index = checkpoint_index(model_dir)
-    kwargs = {}
-    if getattr(cfg, "tie_word_embeddings", True) is None:
-        kwargs["tied"] = "lm_head.weight" not in index
-    model = build_model(cfg, **kwargs)
+    model = build_model(cfg, checkpoint_names=set(index))
     load_weights(model, model_dir, device, dtype, index)
     model.finalize_all(device, dtype, max_positions)
     return model

@@ -27,29 +27,49 @@ def _checkpoint_tensor_specs(model) -> list:
     return sorted((n, s, k, d) for n, (s, k, d) in out.items())
 
 
+def _draw(shape, kind: str, gen, device) -> torch.Tensor:
+    if kind == "matrix":
+        return torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * 0.02
+    if kind == "norm":
+        return 1.0 + (torch.rand(shape, generator=gen, dtype=torch.float32, device=device) * 0.2 - 0.1)
+    raise ValueError(f"unknown init kind {kind!r}")
+
+
 def random_tensors(model, seed: int):
     """Yield (checkpoint name, float32 cpu tensor, dtype policy) in sorted name order."""
     gen = torch.Generator(device="cpu")
     gen.manual_seed(int(seed))
     for name, shape, kind, policy in _checkpoint_tensor_specs(model):
-        if kind == "matrix":
-            t = torch.randn(shape, generator=gen, dtype=torch.float32) * 0.02
-        elif kind == "norm":
-            t = 1.0 + (torch.rand(shape, generator=gen, dtype=torch.float32) * 0.2 - 0.1)
-        else:
-            raise ValueError(f"{name}: unknown init kind {kind!r}")
-        yield name, t, policy
+        yield name, _draw(shape, kind, gen, "cpu"), policy
 
 
-def fill_random(model, seed: int, device, dtype: torch.dtype, max_positions: int, round_to=torch.bfloat16):
+def fill_random(model, seed: int, device, dtype: torch.dtype, max_positions: int, round_to=torch.bfloat16,
+                on_device: bool = False):
     """Bind random weights without a folder. Values are first rounded to `round_to` (what a
-    written folder would store) so both routes give the same model."""
+    written folder would store) so both routes give the same model.
+
+    on_device: every tensor is drawn where it will live, by a generator of that device seeded with
+    (seed, the tensor's place in the sorted name order), one tensor at a time: no host copy of the
+    model exists at any moment (a 32B model is 65 GB). The values then depend on (config, seed) and
+    the kind of device, and differ from those of the host route."""
     from .loader import fill_model
 
-    store = {}
-    for name, t, _ in random_tensors(model, seed):
-        store[name] = t.to(round_to) if round_to is not None else t
-    fill_model(model, store.__getitem__, lambda n: store[n].dtype, device, dtype)
+    if on_device and torch.device(device).type != "cpu":
+        specs = {name: (i, shape, kind) for i, (name, shape, kind, _) in enumerate(_checkpoint_tensor_specs(model))}
+        gen = torch.Generator(device=device)
+
+        def draw(name):
+            i, shape, kind = specs[name]
+            gen.manual_seed((int(seed) << 20) + i)
+            t = _draw(shape, kind, gen, device)
+            return t.to(round_to) if round_to is not None else t
+
+        fill_model(model, draw, lambda n: round_to or torch.float32, device, dtype)
+    else:
+        store = {}
+        for name, t, _ in random_tensors(model, seed):
+            store[name] = t.to(round_to) if round_to is not None else t
+        fill_model(model, store.__getitem__, lambda n: store[n].dtype, device, dtype)
     model.finalize_all(device, dtype, max_positions)
     return model
 

@@ -53,9 +53,9 @@ def _engine(folder, **kw):
 def test_settings_switch_the_scheduler_and_refuse_what_it_cannot_do(folders, plain_backend):
     llm = _engine(folders("B"))
     cli_latency.apply_setting(llm, "c16")
-    assert llm.scheduler.enable_chunked_prefill and llm.scheduler.max_num_batched_tokens == 16
+    assert llm.scheduler.chunked and llm.scheduler.token_budget == 16
     cli_latency.apply_setting(llm, "pf")
-    assert not llm.scheduler.enable_chunked_prefill and llm.scheduler.max_num_batched_tokens == cli_latency.ENGINE_BUDGET
+    assert not llm.scheduler.chunked and llm.scheduler.token_budget == cli_latency.ENGINE_BUDGET
     for bad in ("c0", "c99999", "x12", "c", "c2"):     # c2: fewer tokens than requests that may decode
         with pytest.raises(ValueError):
             cli_latency.apply_setting(llm, bad)
