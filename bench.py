@@ -4,16 +4,17 @@
 
 The default run has the layer sizes of Qwen3-0.6B (28 layers, hidden 1024, 16 query / 8 key heads
 of 128, intermediate 3072, vocabulary 151936, tied head) with seeded random weights, bfloat16, a
-batch of 8 requests each holding a 2,048-token context. A "step" is one decode step of the whole
-batch: the engine's own step function, cache manager and sampler (greedy), from token ids to the
-next token ids on the host. As in LLMEngine.step, a step is launched with its input tokens still on
-the device while the host fetches the tokens of the step before (--no-run-ahead: one after the
-other); all of them reach the host inside the timed span. One JSON line is printed:
+batch of 8 requests each holding a 2,048-token context. Everything measured goes through the engine's
+entry point: a model folder is written, `LLM(folder, ...)` loads it and sizes its cache pool, requests
+are added with `add_request` and run with `step` (scheduler, step function, cache manager, sampler,
+decode graphs, steps launched one ahead: what `generate` uses). A "step" is one decode step of the whole
+batch; every step's tokens reach the host inside the timed span. One JSON line is printed:
   value        decoded tokens per second at the default batch
   prefill      one 2,048-token prompt in one step: tokens/s, ms, fraction of the bf16 MFMA peak
   roofline     bytes the decode step must read (every weight once + the live requests' cache) / time
   points       decode tokens/s at batch 1 and 64
-  offline      the reference's offline workload (256 requests) through the scheduler: output tokens/s of the
+  8b           the same figures at the Qwen3-8B layer sizes (random weights drawn on the device; --second-size '' skips)
+  offline      the reference's offline workload (256 requests) through `generate`: output tokens/s of the
                second of two passes, and of the first (--offline 0: skip); --mixed-lengths N: the same for N
                requests with nine short prompts to one long under a 2,048-token budget
 Peaks: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 157.3 TFLOP/s (MI355X, published).
@@ -22,13 +23,19 @@ from __future__ import annotations
 
 import argparse
 import json
+import os
 import sys
+import tempfile
 import time
 
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
 from mini_engine_amd.config.sizes import SIZES, model_config   # noqa: E402  (the named layer sizes)
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
 def linear_params_per_layer(cfg) -> int:
@@ -53,159 +60,176 @@ def prefill_flops(cfg, T: int) -> float:
 
 
 class Bench:
-    def __init__(self, cfg, dtype: str, page: int, max_batch: int, context: int, gen: int, seed: int = 0,
-                 graphs: bool = True, min_pages: int = 0, max_len: int = 0, run_ahead: bool = True):
+    """An engine built by `LLM(folder)` and the workloads run on it."""
+
+    def __init__(self, cfg, folder: str, dtype: str, page: int, max_seqs: int, max_len: int, budget: int, seed: int,
+                 graphs: bool, run_ahead: bool, random_weights: int | None):
         import torch
-        from mini_engine_amd.cache.manager import CacheManager
-        from mini_engine_amd.engine.runner import ModelRunner
-        from mini_engine_amd.registry import build_model
-        from mini_engine_amd.weights.random_init import fill_random
+        from mini_engine_amd import LLM
 
-        self.torch = torch
-        self.cfg, self.page, self.context, self.gen = cfg, page, context, gen
-        self.run_ahead = run_ahead
-        self.dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
-        self.max_len = max(context + gen + 64, max_len)
+        self.torch, self.cfg = torch, cfg
         t0 = time.time()
-        self.model = fill_random(build_model(cfg), seed, "cuda", self.dtype, self.max_len)
-        print(f"[bench] random weights ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
-        pages = max(max_batch * -(-self.max_len // page), min_pages)
-        self.manager = CacheManager(pages, page, ModelRunner.windows_of(self.model), enable_prefix_caching=False)
-        self.runner = ModelRunner(self.model, self.manager, self.dtype, "cuda", self.max_len, use_graphs=graphs)
-        self.gen_ids = torch.Generator().manual_seed(seed)
+        self.llm = LLM(folder, dtype=dtype, kvcache_block_size=page, max_num_seqs=max_seqs, max_model_len=max_len,
+                       max_num_batched_tokens=budget, seed=seed, use_graphs=graphs, run_ahead=run_ahead,
+                       random_weights=random_weights, eos=-1)
+        log(f"engine ready in {time.time() - t0:.1f}s: {self.llm.config.num_kvcache_blocks} pages of {page} tokens, "
+            f"{self.llm.reserved_bytes >> 20} MiB kept free for the steps' working set")
+        self.ids = torch.Generator().manual_seed(seed)
 
-    def _ids(self, n):
-        return self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen_ids).tolist()
+    def _prompt(self, n: int) -> list:
+        return self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.ids).tolist()
 
-    def prefill(self, rid, n, want_last=True, ids=None):
-        from mini_engine_amd.engine.runner import StepEntry
-        assert self.manager.allocate(rid, 0, n)
-        return self.runner.step([StepEntry(rid, ids if ids is not None else self._ids(n), 0, [n - 1] if want_last else [])])
+    def _drain(self) -> None:
+        while not self.llm.is_finished():
+            self.llm.step()
 
-    def time_prefill(self, T: int, reps: int = 3):
-        torch = self.torch
-        best = None
-        for i in range(reps + 1):                          # the first run warms up
-            ids = self._ids(T)                             # drawing the prompt is not the engine's work
+    def time_prefill(self, T: int, reps: int = 3) -> float:
+        """One prompt of T tokens, one generated token: add_request + step, best of `reps` (after a warm-up)."""
+        from mini_engine_amd import SamplingParams
+        torch, best = self.torch, None
+        for i in range(reps + 1):
+            prompt = self._prompt(T)                       # drawing the prompt is not the engine's work
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            self.prefill(("p", i), T, ids=ids)
+            self.llm.add_request(prompt, SamplingParams(temperature=0, max_tokens=1, ignore_eos=True))
+            finished, num_prefill, _, _ = self.llm.step()
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
-            self.manager.free(("p", i))
+            assert num_prefill == T and len(finished) == 1, "the prompt did not run as one step"
             if i and (best is None or dt < best):
                 best = dt
         return best
 
-    def time_decode(self, batch: int, steps: int, warmup: int):
-        """`batch` requests with `context` tokens each in the cache, then warmup + steps decode steps.
-
-        With run_ahead (the engine's default way of decoding, LLMEngine.step) a step is launched with its
-        tokens still on the device and the tokens of the step before are fetched behind it; every step's
-        tokens reach the host inside the timed span, the last ones before the clock stops."""
-        from mini_engine_amd.engine.runner import PENDING, StepEntry
-        torch = self.torch
-        reqs = [("d", batch, i) for i in range(batch)]
-        last = []
-        for r in reqs:                                     # real prefill, one request per step
-            logits = self.prefill(r, self.context)
-            last.append(int(self.runner.sample(logits, [0.0], [(0, 0)])[0]))
-        pos = self.context
-        temps, keys = [0.0] * batch, [(0, 0)] * batch
-        ahead = self.run_ahead and self.runner.graphs is not None and self.runner.graphs.takes(batch)
-        in_flight = None
-
-        def one():
-            nonlocal last, pos, in_flight
-            entries = []
-            for r, tok in zip(reqs, last):
-                assert self.manager.allocate(r, pos, 1)
-                entries.append(StepEntry(r, [PENDING if in_flight is not None else tok], pos, [0]))
-            logits = self.runner.step(entries)
-            if not ahead:
-                last = self.runner.sample(logits, temps, keys)  # token ids on the host: the step is complete
-            else:
-                launched = self.runner.sample_async(logits, temps, keys, reqs)
-                if in_flight is not None:
-                    last = in_flight.tokens()              # the tokens of the step before, on the host
-                in_flight = launched
-            pos += 1
-
-        def drain():
-            nonlocal last, in_flight
-            if in_flight is not None:
-                last = in_flight.tokens()
-                in_flight = None
-
+    def time_decode(self, batch: int, context: int, steps: int, warmup: int):
+        """`batch` requests of `context` prompt tokens each; once all decode, `warmup` untimed steps, then
+        `steps` timed ones. Returns (seconds per step, mean context length over the timed steps)."""
+        from mini_engine_amd import SamplingParams
+        torch, llm = self.torch, self.llm
+        slack = 16 + batch * context // max(1, llm.scheduler.token_budget)     # requests admitted early decode while others go in
+        sp = SamplingParams(temperature=0, max_tokens=warmup + steps + slack, ignore_eos=True)
+        for _ in range(batch):
+            llm.add_request(self._prompt(context), sp)
+        while True:                                         # prompts go in under the token budget
+            _, num_prefill, num_decode, _ = llm.step()
+            if num_prefill == 0 and num_decode == batch and not llm.scheduler.waiting:
+                break
         for _ in range(warmup):
-            one()
-        drain()
+            llm.step()
         torch.cuda.synchronize()
+        live = llm.scheduler.running
+        first_ctx = sum(r.in_cache for r in live) / len(live) + 1     # keys a request reads in the first timed step
         t0 = time.perf_counter()
         for _ in range(steps):
-            one()
-        drain()
+            _, num_prefill, num_decode, got = llm.step()
+            assert num_prefill == 0 and num_decode == batch and len(got) == batch
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        ctx_mid = pos - steps / 2.0                        # mean context length over the timed steps
-        for r in reqs:
-            self.manager.free(r)
-        return dt / steps, ctx_mid
+        self._drain()
+        return dt / steps, first_ctx + (steps - 1) / 2.0
 
-
-    def offline(self, num_seqs: int, budget: int = 16384, max_model_len: int = 2048):
+    def offline(self, num_seqs: int):
         """The reference's offline workload (its bench.py:38-48,60-66): `random.seed(0)`, prompts of 100-1024
-        random ids below 10000, max_tokens 100-1024, temperature 0.6, ignore_eos, max_num_seqs 256,
-        max_model_len 2048, chunked prefill under a 16k budget. Returns (sum of max_tokens / seconds, record)."""
+        random ids below 10000, max_tokens 100-1024, temperature 0.6, ignore_eos, chunked prefill under the
+        engine's budget. Returns the record."""
         from random import randint, seed
         seed(0)
         prompts = [[randint(0, 10000) % self.cfg.vocab_size for _ in range(randint(100, 1024))] for _ in range(num_seqs)]
         max_tokens = [randint(100, 1024) for _ in range(num_seqs)]
-        rate, record = self.serve(prompts, max_tokens, budget, max_model_len)
+        record = self.serve(prompts, max_tokens)
         record["reference_a100_tok_s"] = 4205.0
-        return rate, record
+        return record
 
-    def mixed_lengths(self, num_seqs: int, budget: int = 2048, max_model_len: int = 8192):
-        """Nine short prompts (128-512 tokens) to one long (4,096-7,680), 128-256 output tokens each, chunked
-        prefill under a 2,048 budget: long prompts go through the cache in portions while the others decode
-        beside them, so most steps are mixed ones. Same sampling and engine settings as `offline`."""
+    def mixed_lengths(self, num_seqs: int):
+        """Nine short prompts (128-512 tokens) to one long (4,096-7,680), 128-256 output tokens each: long
+        prompts go through the cache in portions while the others decode beside them, so most steps are mixed."""
         from random import randint, random, seed
         seed(0)
         lengths = [randint(4096, 7680) if random() < 0.1 else randint(128, 512) for _ in range(num_seqs)]
         prompts = [[randint(0, 10000) % self.cfg.vocab_size for _ in range(n)] for n in lengths]
         max_tokens = [randint(128, 256) for _ in range(num_seqs)]
-        rate, record = self.serve(prompts, max_tokens, budget, max_model_len)
+        record = self.serve(prompts, max_tokens)
         record["long_prompts"] = sum(n >= 4096 for n in lengths)
-        return rate, record
+        return record
 
-    def serve(self, prompts, max_tokens, budget: int, max_model_len: int):
-        """All requests handed to the engine at once (scheduler, sampler and step function as `LLM.generate`
-        uses them; temperature 0.6, ignore_eos, at most 256 running). Returns (output tokens / second of the
-        second of two passes, record with both)."""
-        from types import SimpleNamespace
-        from mini_engine_amd.engine.llm_engine import LLMEngine
-        from mini_engine_amd.sampling.sampling_params import SamplingParams
-        conf = SimpleNamespace(max_num_seqs=256, max_num_batched_tokens=budget, long_prefill_token_threshold=0,
-                               enable_chunked_prefill=True, scheduling_policy="fcfs", eos=-1, max_model_len=max_model_len,
-                               seed=0, run_ahead=self.run_ahead)
-        llm = LLMEngine.from_parts(conf, self.model, self.manager, self.runner)
+    def serve(self, prompts, max_tokens):
+        """All requests handed to `generate` at once (temperature 0.6, ignore_eos). The workload runs twice: the
+        first pass, after the reference's one-prompt warm-up (its bench.py:62), still meets every shape for the
+        first time (decode graphs are captured, the library plans its products); the second is the steady state."""
+        from mini_engine_amd import SamplingParams
+        llm = self.llm
         sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
         llm.generate([[1, 2, 3]], SamplingParams(max_tokens=4), use_tqdm=False)
-        # The workload runs twice. The first pass, after the reference's one-prompt warm-up (its bench.py:62),
-        # still meets every shape for the first time: decode graphs are captured, the library loads its
-        # kernels and plans its products. The second pass is the engine in its steady state.
         took = []
         for _ in range(2):
+            llm.manager.forget_prefixes()                  # the second pass must not find the first one's pages
             self.torch.cuda.synchronize()
             t0 = time.perf_counter()
             llm.generate(prompts, sps, use_tqdm=False)
             took.append(time.perf_counter() - t0)
-        dt = took[1]
         total = sum(max_tokens)
-        return total / dt, {"value": round(total / dt, 1), "unit": "output tokens/s", "seconds": round(dt, 2),
-                            "first_pass_value": round(total / took[0], 1), "first_pass_seconds": round(took[0], 2),
-                            "requests": len(prompts), "input_tokens": sum(len(p) for p in prompts), "output_tokens": total,
-                            "budget": budget, "preemptions": llm.scheduler.num_preemptions}
+        return {"value": round(total / took[1], 1), "unit": "output tokens/s", "seconds": round(took[1], 2),
+                "first_pass_value": round(total / took[0], 1), "first_pass_seconds": round(took[0], 2),
+                "requests": len(prompts), "input_tokens": sum(len(p) for p in prompts), "output_tokens": total,
+                "budget": llm.scheduler.token_budget, "preemptions": llm.scheduler.num_preemptions}
+
+
+def folder_for(cfg, seed: int, root: str, on_device: bool) -> tuple:
+    """(model folder, random_weights option). on_device: the folder holds config.json only and the engine draws
+    the weights where they live; otherwise config.json and model.safetensors are written and loaded."""
+    from mini_engine_amd.weights.random_init import write_random_model
+    os.makedirs(root, exist_ok=True)
+    if on_device:
+        with open(os.path.join(root, "config.json"), "w") as f:
+            json.dump(cfg.to_dict(), f)
+        return root, seed
+    t0 = time.time()
+    write_random_model(cfg, seed, root)
+    log(f"model folder written in {time.time() - t0:.1f}s")
+    return root, None
+
+
+def measure(args, size: str, layers, tmp: str, points: list, steps: int, warmup: int, serve: bool) -> dict:
+    """Prefill, decode at the default batch and at `points`, and the served workloads, at one model size."""
+    cfg, full_layers = model_config(size, layers)
+    params = cfg.num_hidden_layers * linear_params_per_layer(cfg) + cfg.vocab_size * cfg.hidden_size
+    on_device = args.weights == "device" or (args.weights == "auto" and params > 2e9)
+    folder, random_weights = folder_for(cfg, args.seed, os.path.join(tmp, size), on_device)
+    gen = max(args.gen, steps + warmup + 2)
+    max_len = max(args.context + gen + 128, 4096, 8192 if (serve and args.mixed_lengths) else 0)
+    batches = [args.batch] + points
+    max_seqs = max(batches + ([256] if serve and (args.offline or args.mixed_lengths) else []))
+    budget = max(args.prefill_tokens, 2048 if (serve and args.mixed_lengths) else 16384, max_seqs)
+    bench = Bench(cfg, folder, args.dtype, args.page, max_seqs, max_len, budget, args.seed, not args.no_graphs,
+                  not args.no_run_ahead, random_weights)
+    item = 2 if args.dtype == "bfloat16" else 4
+    out = {"cfg": cfg, "full_layers": full_layers, "weights": "drawn on the device" if on_device else "written folder"}
+
+    T = args.prefill_tokens
+    pre = bench.time_prefill(T)
+    out["prefill"] = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
+                      "frac": round(prefill_flops(cfg, T) / pre / FLOP_PEAK[args.dtype], 4)}
+    log(f"{size}: prefill {T} tokens: {pre * 1e3:.2f} ms")
+
+    out["decode"] = {}
+    for b in batches:
+        k, w = (steps, warmup) if b == args.batch else (min(steps, 64), min(warmup, 8))
+        step_s, ctx = bench.time_decode(b, args.context, k, w)
+        need = decode_bytes(cfg, item, [ctx] * b)
+        out["decode"][b] = {"step_s": step_s, "tok_s": round(b / step_s, 1), "hbm_frac": round(need / step_s / HBM_PEAK, 4),
+                            "gbps": round(need / step_s / 1e9, 1)}
+        log(f"{size}: decode batch {b}: {step_s * 1e3:.3f} ms/step, {need / step_s / HBM_PEAK:.1%} of HBM")
+    if serve and args.offline:
+        out["offline"] = bench.offline(args.offline)
+        log(f"{size}: reference offline workload: {out['offline']['value']} output tokens/s")
+    if serve and args.mixed_lengths:
+        out["mixed_lengths"] = bench.mixed_lengths(args.mixed_lengths)
+        log(f"{size}: short and long prompts mixed: {out['mixed_lengths']['value']} output tokens/s")
+    del bench
+    import gc
+    import torch
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
 
 
 def main(argv=None) -> int:
@@ -215,6 +239,8 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--model-size", default="0.6b", choices=sorted(SIZES))
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the size has (both numbers are reported)")
+    ap.add_argument("--second-size", default="8b", help="a second size whose figures go into an object of its own ('' for none)")
+    ap.add_argument("--second-layers", type=int, default=None)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
@@ -223,6 +249,9 @@ def main(argv=None) -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="extra decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--weights", default="auto", choices=["auto", "folder", "device"],
+                    help="folder: write model.safetensors and load it; device: draw the weights on the GPU; "
+                         "auto: a folder up to 2 G parameters, the device beyond")
     ap.add_argument("--offline", type=int, default=256,
                     help="also run the reference's offline workload with this many requests (0: skip)")
     ap.add_argument("--mixed-lengths", type=int, default=0,
@@ -234,65 +263,49 @@ def main(argv=None) -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
-    if args.steps + args.warmup > args.gen:
-        args.gen = args.steps + args.warmup
 
-    import torch
-    cfg, full_layers = model_config(args.model_size, args.layers)
-    points = [int(p) for p in args.points.split(",") if p]
-    off_pages = args.offline * -(-2048 // args.page) if args.offline else 0
-    if args.mixed_lengths:      # room for every request at its full length (a tenth of them long): no preemption
-        off_pages = max(off_pages, args.mixed_lengths * -(-(768 + 8192 // 8) // args.page))
-    bench = Bench(cfg, args.dtype, args.page, max([args.batch] + points), args.context, args.gen, args.seed,
-                  graphs=not args.no_graphs, min_pages=off_pages, max_len=8192 if args.mixed_lengths else 2048 if args.offline else 0,
-                  run_ahead=not args.no_run_ahead)
-    item = 2 if args.dtype == "bfloat16" else 4
+    points = [int(p) for p in args.points.split(",") if p and int(p) != args.batch]
+    with tempfile.TemporaryDirectory() as tmp:
+        main_run = measure(args, args.model_size, args.layers, tmp, points, args.steps, args.warmup, serve=True)
+        second = None
+        if args.second_size and args.second_size != args.model_size:
+            second = measure(args, args.second_size, args.second_layers, tmp, points, min(args.steps, 32),
+                             min(args.warmup, 4), serve=False)
 
-    T = args.prefill_tokens
-    pre = bench.time_prefill(T)
-    prefill = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
-               "frac": round(prefill_flops(cfg, T) / pre / FLOP_PEAK[args.dtype], 4)}
-    print(f"[bench] prefill {T} tokens: {pre * 1e3:.2f} ms", file=sys.stderr, flush=True)
-
-    step_s, ctx_mid = bench.time_decode(args.batch, args.steps, args.warmup)
-    need = decode_bytes(cfg, item, [ctx_mid] * args.batch)
-    roofline = {"bound": "hbm", "achieved": round(need / step_s / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                "frac": round(need / step_s / HBM_PEAK, 4)}
-    print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
-    pts = {}
-    for b in points:
-        s, _ = bench.time_decode(b, min(args.steps, 64), min(args.warmup, 8))
-        pts[f"decode_b{b}"] = round(b / s, 1)
-        print(f"[bench] decode batch {b}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
-
-    offline = None
-    if args.offline:
-        _, offline = bench.offline(args.offline)
-        print(f"[bench] reference offline workload: {offline['value']} output tokens/s", file=sys.stderr, flush=True)
-
-    mixed = None
-    if args.mixed_lengths:
-        _, mixed = bench.mixed_lengths(args.mixed_lengths)
-        print(f"[bench] short and long prompts mixed: {mixed['value']} output tokens/s", file=sys.stderr, flush=True)
-
+    cfg = main_run["cfg"]
+    head = main_run["decode"][args.batch]
     line = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens; % roofline",
-        "value": round(args.batch / step_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "value": head["tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(head["step_s"] * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic: seeded random token ids, seeded random weights",
-        "config": {"model": f"Qwen3-{args.model_size} sizes", "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+        "data": f"synthetic: seeded random token ids, seeded random weights ({main_run['weights']})",
+        "config": {"model": f"Qwen3-{args.model_size} sizes", "layers": cfg.num_hidden_layers, "layers_of_model": main_run["full_layers"],
                    "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "tied": bool(cfg.tie_word_embeddings), "page": args.page, "global_batch": args.batch,
                    "seq_len": args.context, "gen": args.gen, "parallelism": "single GPU",
-                   "hip_graphs": not args.no_graphs, "run_ahead": not args.no_run_ahead and not args.no_graphs},
-        "prefill": prefill, "roofline": roofline, "points": pts,
+                   "hip_graphs": not args.no_graphs, "run_ahead": not args.no_run_ahead and not args.no_graphs,
+                   "entry": "LLM.add_request/step"},
+        "prefill": main_run["prefill"],
+        "roofline": {"bound": "hbm", "achieved": head["gbps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head["hbm_frac"]},
+        "points": {f"decode_b{b}": main_run["decode"][b]["tok_s"] for b in points},
     }
-    if offline is not None:
-        line["offline"] = offline
-    if mixed is not None:
-        line["mixed_lengths"] = mixed
+    if second is not None:
+        c2 = second["cfg"]
+        obj = {"model": f"Qwen3-{args.second_size} sizes", "layers": c2.num_hidden_layers, "layers_of_model": second["full_layers"],
+               "hidden": c2.hidden_size, "q_heads": c2.num_attention_heads, "kv_heads": c2.num_key_value_heads,
+               "head_dim": c2.head_dim, "intermediate": c2.intermediate_size, "vocab": c2.vocab_size,
+               "tied": bool(c2.tie_word_embeddings), "weights": second["weights"], "seq_len": args.context,
+               "prefill": second["prefill"]}
+        for b, d in second["decode"].items():
+            obj[f"decode_b{b}"] = d["tok_s"]
+            obj[f"decode_b{b}_ms"] = round(d["step_s"] * 1e3, 4)
+            obj[f"decode_b{b}_hbm_frac"] = d["hbm_frac"]
+        line[args.second_size] = obj
+    for name in ("offline", "mixed_lengths"):
+        if name in main_run:
+            line[name] = main_run[name]
     print(json.dumps(line), flush=True)
     return 0
 

@@ -10,6 +10,11 @@ Options the reference has keep its names and meanings: --model, --num-seqs, --ou
 `random.seed(0)`, prompts of 100-1024 random ids below 10000, max_tokens 100-1024, temperature 0.6,
 ignore_eos, max_num_seqs 256, max_model_len 2048, one warm-up generate; the figure is the sum of
 max_tokens over the wall time. One JSON row is printed and appended to --out.
+
+With --prompts FILE the workload is the file's instead: one request a line, either a JSON list of token
+ids or an object {"prompt": [ids], "max_tokens": n, "temperature": t} (missing fields: --max-output and
+--temperature). --tokens-out FILE writes what was generated, one JSON list of token ids a line in the order
+of the prompts ("-": standard output, before the row). Ids in, ids out: a model folder needs no tokenizer.
 Not taken over: --engine (other engines), --attn unified (this engine has one attention path),
 --expect-gpu.
 """
@@ -45,6 +50,12 @@ def main(argv=None) -> int:
     p.add_argument("--policy", default="fcfs", choices=["fcfs", "priority"])
     p.add_argument("--max-prompt", type=int, default=1024)
     p.add_argument("--max-output", type=int, default=1024)
+    p.add_argument("--device", default="cuda")
+    p.add_argument("--num-kv-blocks", type=int, default=-1, help="num_kvcache_blocks (-1: sized from free memory)")
+    p.add_argument("--prompts", default=None, metavar="FILE", help="requests to run instead of the random workload (JSON lines)")
+    p.add_argument("--tokens-out", default=None, metavar="FILE", help="write the generated token ids here, a JSON list a line ('-': stdout)")
+    p.add_argument("--temperature", type=float, default=0.6, help="0: greedy")
+    p.add_argument("--stop-at-eos", action="store_true", help="end a request at the model's end token (default: ignore it, as the reference's workload)")
     args = p.parse_args(argv)
     if (args.model is None) == (args.random_weights is None):
         p.error("give exactly one of --model and --random-weights")
@@ -64,28 +75,57 @@ def main(argv=None) -> int:
         path = write_random_model(cfg, args.seed, tmp.name)
     path = os.path.expanduser(path)
 
-    seed(0)
-    N = args.num_seqs
     vocab_cap = 10000
-    prompt_token_ids = [[randint(0, vocab_cap) for _ in range(randint(min(100, args.max_prompt), args.max_prompt))] for _ in range(N)]
-    max_tokens = [randint(min(100, args.max_output), args.max_output) for _ in range(N)]
+    if args.prompts:
+        prompt_token_ids, max_tokens, temperatures = [], [], []
+        with open(args.prompts) as f:
+            for number, text in enumerate(f, 1):
+                if not text.strip():
+                    continue
+                rec = json.loads(text)
+                if isinstance(rec, list):
+                    rec = {"prompt": rec}
+                if not (isinstance(rec, dict) and isinstance(rec.get("prompt"), list) and rec["prompt"]
+                        and all(isinstance(t, int) for t in rec["prompt"])):
+                    p.error(f"{args.prompts}:{number}: expected a list of token ids or an object with one under 'prompt'")
+                prompt_token_ids.append(rec["prompt"])
+                max_tokens.append(int(rec.get("max_tokens", args.max_output)))
+                temperatures.append(float(rec.get("temperature", args.temperature)))
+        N = len(prompt_token_ids)
+        vocab_cap = None
+    else:
+        seed(0)
+        N = args.num_seqs
+        prompt_token_ids = [[randint(0, vocab_cap) for _ in range(randint(min(100, args.max_prompt), args.max_prompt))] for _ in range(N)]
+        max_tokens = [randint(min(100, args.max_output), args.max_output) for _ in range(N)]
+        temperatures = [args.temperature] * N
 
     llm = LLM(path, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len, max_num_batched_tokens=args.budget,
               enable_chunked_prefill=bool(args.chunked), long_prefill_token_threshold=args.threshold, dtype=args.dtype,
-              seed=args.seed, kvcache_block_size=args.block_size, scheduling_policy=args.policy)
+              seed=args.seed, kvcache_block_size=args.block_size, scheduling_policy=args.policy, device=args.device,
+              num_kvcache_blocks=args.num_kv_blocks)
     vocab = llm.model.embedding.vocab_size
-    if vocab <= vocab_cap:
+    if vocab_cap is not None and vocab <= vocab_cap:
         prompt_token_ids = [[t % vocab for t in ids] for ids in prompt_token_ids]
-    sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
+    sps = [SamplingParams(temperature=temp, ignore_eos=not args.stop_at_eos, max_tokens=m)
+           for temp, m in zip(temperatures, max_tokens)]
 
     llm.generate([[1, 2, 3]], SamplingParams(max_tokens=4), use_tqdm=False)      # warm-up
     t = time.time()
-    llm.generate(prompt_token_ids, sps, use_tqdm=False)
+    results = llm.generate(prompt_token_ids, sps, use_tqdm=False)
     t = time.time() - t
+    if args.tokens_out:
+        lines = "".join(json.dumps(r["token_ids"]) + "\n" for r in results)
+        if args.tokens_out == "-":
+            sys.stdout.write(lines)
+        else:
+            os.makedirs(os.path.dirname(args.tokens_out) or ".", exist_ok=True)
+            with open(args.tokens_out, "w") as f:
+                f.write(lines)
 
-    total = sum(max_tokens)
+    total = sum(len(r["token_ids"]) for r in results)
     row = {
-        "engine": "mini_engine_amd", "label": args.label, "gpu": torch.cuda.get_device_name(0), "torch": torch.__version__,
+        "engine": "mini_engine_amd", "label": args.label, "gpu": torch.cuda.get_device_name(0) if args.device.startswith("cuda") else args.device, "torch": torch.__version__,
         "model": args.random_weights or path, "dtype": args.dtype, "num_seqs": N,
         "input_tokens": sum(len(x) for x in prompt_token_ids), "output_tokens": total, "time_s": round(t, 2),
         "throughput_tok_s": round(total / t, 1), "chunked": bool(args.chunked), "budget": args.budget,

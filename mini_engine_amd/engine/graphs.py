@@ -6,7 +6,7 @@ token, the whole forward pass is captured once per (batch bucket, context cap, c
 long or not) and replayed:
 the step's metadata lives in one device array of fixed layout that is rewritten before each
 replay. Rows beyond the real batch are padding: context length 0, slot -1 (nothing is
-written to the cache), token 0.
+written to any request's page: their slot lies in the pool's spare page, their state row is the spare one), token 0.
 
 The captured work is the same model code and kernels as the eager step; only the launch
 mechanism differs. Nothing is cleared with memset nodes inside the graph.
@@ -24,8 +24,15 @@ from .context import GroupStep, StepContext
 
 PENDING = -1      # the runner's marker for a token that is still on the device (runner.PENDING)
 
-BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 CONTEXT_STEP = 1024      # the context cap of a captured graph is a multiple of this
+
+
+def bucket_of(rows: int) -> int:
+    """Rows of the captured layout that holds a step of `rows` requests: powers of two up to 256,
+    multiples of 128 beyond."""
+    if rows <= 256:
+        return 1 << max(0, rows - 1).bit_length()
+    return -(-rows // 128) * 128
 
 
 def _pad4(n: int) -> int:
@@ -36,7 +43,7 @@ class _Captured:
     def __init__(self, runner, bucket: int, ctx_cap: int, even: bool = False):
         self.bucket, self.ctx_cap, self.even = bucket, ctx_cap, even
         ps = runner.manager.page_size
-        self.G = runner.manager.num_groups
+        self.G = len(runner.plan.group_needs)
         self.MB = -(-ctx_cap // ps)
         B = bucket
         self.seg, n = {}, 0
@@ -52,9 +59,12 @@ class _Captured:
         self.put("seq_of_token", np.arange(B))
         self.put("cu", np.arange(B + 1))
         self.put("rows", np.arange(B))
-        self.put("state_slots", -1)
+        self.spare_state = runner.pool.spare_state_slot
+        self.spare_slot = [runner.pool.spare_page(g) * ps for g in range(self.G)]
+        self.put("state_slots", self.spare_state)
         for g in range(self.G):
             self.put(f"bt{g}", -1)
+            self.put(f"slots{g}", self.spare_slot[g])
         self.row_req = [None] * B                            # which request's table a row holds
         self.row_len = [[0] * B for _ in range(self.G)]      # how many of its entries are written
         self.row_tab = [[None] * B for _ in range(self.G)]   # the manager's table they were copied from
@@ -66,7 +76,6 @@ class _Captured:
         self.flip = 0
         self.dev = torch.zeros(n, dtype=torch.int32, device=runner.device)
         self.graph = None
-        self.logits = None
 
     def put(self, name, values):
         o, size = self.seg[name]
@@ -102,26 +111,28 @@ class _Captured:
 
 class DecodeGraphs:
     def __init__(self, runner, max_bucket: int = 256, capture: bool = True, max_graphs: int = 64):
-        """capture=False runs the padded, fixed-layout step eagerly every time (no graph): the same
-        metadata path without the capture, for machines without a GPU."""
+        """Steps of up to `max_bucket` requests go through here. capture=False runs the padded,
+        fixed-layout step eagerly every time (no graph): the same metadata path without the capture,
+        for machines without a GPU."""
         self.runner = weakref.proxy(runner)      # the runner owns this object: no cycle, so that an engine that
         self.max_bucket = max_bucket             # goes out of use is freed at once, not by a later collection
         self.max_graphs = max(4, max_graphs)     # (bucket, context cap) pairs kept; the one unused for longest goes first
         self.capture = capture
         self.captured: dict = {}
-        # One memory pool for all captured graphs: they replay one after the other on one stream and a
-        # step's logits are sampled before the next graph is launched, so a graph may reuse what the
-        # others' activations and logits occupy (else every (bucket, context cap) keeps its own, and a
-        # batch of 256 holds 150 MB of logits alone per context cap).
+        # One memory pool for all captured graphs: they replay one after the other on one stream, so a
+        # graph may reuse what the others' activations occupy. Nothing a graph allocates outlives its
+        # capture: the logits, the one result that is read afterwards, go into `self.logits`, one buffer
+        # for all layouts (a layout that kept its own would pin 150 MB of the pool at 256 rows).
         self.pool = torch.cuda.graph_pool_handle() if (capture and runner.device.type == "cuda") else None
+        self.logits = None
         self.replays = 0
         self.advances = 0        # of those, steps whose tables and slots were carried on from the step before
 
     def takes(self, num_entries: int) -> bool:
         """Whether a step of this many single-token entries goes through here."""
         r = self.runner
-        return ((r.device.type == "cuda" or not self.capture) and not r.pool.has_state and bool(r.plan.group_needs)
-                and num_entries <= self.max_bucket)
+        return ((r.device.type == "cuda" or not self.capture) and num_entries <= self.max_bucket
+                and r.vocab_size is not None)
 
     def eligible(self, entries) -> bool:
         return self.takes(len(entries)) and all(len(e.tokens) == 1 for e in entries)
@@ -130,7 +141,7 @@ class DecodeGraphs:
         """Logits [len(entries), vocab] for a step in which every request brings one token."""
         r = self.runner
         B = len(entries)
-        bucket = next(b for b in BUCKETS if b >= B)
+        bucket = bucket_of(B)
         need_ctx = max(e.start for e in entries) + 1
         ctx_cap = min(-(-need_ctx // CONTEXT_STEP) * CONTEXT_STEP, -(-r.max_positions // 8) * 8)
         # whether the contexts are equally long is part of the layout: the decode kernel's grid depends on it
@@ -161,6 +172,16 @@ class DecodeGraphs:
         cap.put("tokens", tok); cap.put("positions", pos); cap.put("context_lens", ctx)
         cap.put("first_chunk", (pos == 0) & (ctx > 0))
         reqs = [e.req for e in entries]
+        if r.pool.has_state:
+            state = np.full(bucket, cap.spare_state, dtype=np.int64)
+            state[:B] = [r.manager.state_slot(q) for q in reqs]
+            cap.put("state_slots", state)
+            fresh = state[:B][pos[:B] == 0]
+            if fresh.size:              # a request whose first token this is starts from empty state (outside the graph)
+                idx = torch.tensor(fresh.tolist(), dtype=torch.long, device=r.device)
+                for st in r.pool.states:
+                    if st is not None:
+                        st.index_fill_(0, idx, 0)
         continues = self._continues(cap, reqs, pos, B)
         cap.last_starts = None                       # stays so if what follows raises
         if continues:
@@ -182,7 +203,7 @@ class DecodeGraphs:
         if cap.graph is None:
             self._capture(cap)
         cap.graph.replay()
-        return cap.logits[:B]
+        return self.logits[:B]
 
     def _take_pending(self, cap: _Captured, take, B: int) -> None:
         """Copy the tokens that the last sampling call left on the device into the step's token rows
@@ -242,7 +263,7 @@ class DecodeGraphs:
         for g in range(cap.G):
             o, _ = cap.seg[f"bt{g}"]
             bt = cap.master[o:o + bucket * cap.MB].reshape(bucket, cap.MB)
-            slots = np.full(bucket, -1, dtype=np.int64)
+            slots = np.full(bucket, cap.spare_slot[g], dtype=np.int64)
             windowed = r.manager.groups[g].window is not None
             for j, e in enumerate(entries):
                 t = r.manager.block_table(e.req, g)
@@ -268,15 +289,26 @@ class DecodeGraphs:
                     cap.row_tab[g][j] = None
             cap.put(f"slots{g}", slots)
 
-    def _forward(self, cap: _Captured):
+    def _forward(self, cap: _Captured, out=None):
         r = self.runner
         h, residual = r.model.forward(cap.view("tokens"), cap.context(), r.pool.views, r.pool.states)
-        return r.model.logits(h, residual, cap.view("rows"))
+        return r.model.logits(h, residual, cap.view("rows"), out=out)
 
     def _capture(self, cap: _Captured) -> None:
         # one eager run first: libraries load, scratch buffers get their size, the caching allocator warms up
         # (it rewrites this step's cache entries with the same values the replay will write)
-        self._forward(cap)
+        if self.logits is None:
+            r = self.runner
+            self.logits = torch.empty((bucket_of(self.max_bucket), r.vocab_size), dtype=torch.float32, device=r.device)
+        out = self.logits[:cap.bucket]
+        # Cache writes can be repeated, state updates cannot: what the eager run does to the requests'
+        # state is taken back, the replay that follows does it for good.
+        states = [st for st in self.runner.pool.states if st is not None]
+        kept = [st.clone() for st in states]
+        self._forward(cap, out)
+        for st, was in zip(states, kept):
+            st.copy_(was)
+        del kept
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         # No garbage collection while the stream is capturing: a collector run that finds an old
@@ -286,7 +318,7 @@ class DecodeGraphs:
         gc.disable()
         try:
             with torch.cuda.graph(graph, pool=self.pool):
-                cap.logits = self._forward(cap)
+                self._forward(cap, out)
         finally:
             if collecting:
                 gc.enable()

@@ -153,7 +153,8 @@ def library_is_direct() -> bool:
     return _library_direct
 
 
-def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, splits: int = 1) -> torch.Tensor:
+def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, splits: int = 1,
+                    out: torch.Tensor | None = None) -> torch.Tensor:
     """x [M, K] . w[N, K]^T through hipBLASLt, bfloat16 operands, float32 accumulation (reference
     layers/linear.py:25-26: its F.linear is a library product too).
 
@@ -174,7 +175,7 @@ def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, sp
     if _library_direct and _library_workspace is not None:
         M, K = x.shape
         N = w.shape[0]
-        y = torch.empty((M, N) if splits == 1 else (splits, M, N), dtype=out_dtype, device=x.device)
+        y = out if out is not None else torch.empty((M, N) if splits == 1 else (splits, M, N), dtype=out_dtype, device=x.device)
         rc = core().fns["me_gemm_library_bf16"](x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                                                _code(out_dtype), _library_workspace.data_ptr(),
                                                LIBRARY_WORKSPACE_BYTES, M, N, K, splits, _stream())
@@ -184,9 +185,11 @@ def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, sp
             raise KernelError(f"me_gemm_library_bf16: {core().cdll.me_last_error().decode()}")
     if splits > 1:
         return None                 # partial sums over slices of K only through the direct call
-    if out_dtype == torch.float32:
-        return torch.mm(x, w.t(), out_dtype=torch.float32)
-    return torch.matmul(x, w.t())
+    y = torch.mm(x, w.t(), out_dtype=torch.float32) if out_dtype == torch.float32 else torch.matmul(x, w.t())
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y
 
 
 class HipBackend:
@@ -287,7 +290,7 @@ class HipBackend:
     def paged_attention(self, q, k_cache, v_cache, page: int, block_tables, context_lens, seq_of_token,
                         positions, prefill_cu, num_decodes: int, max_decode_context: int, scale: float,
                         window: int | None, Hq: int, Hkv: int, D: int, force_simple: bool = False,
-                        max_prefill_context: int = 0, even_contexts: bool = False):
+                        max_prefill_context: int = 0, even_contexts: bool = False, decode_as_prefill: bool = False):
         """Causal attention of this step's tokens over the paged keys of their requests.
 
         q: [T, Hq*D] (a strided view is fine). Rows are ordered decode requests first (one token
@@ -296,9 +299,12 @@ class HipBackend:
         after this step's write; `block_tables` int32 [B, MB]. `max_prefill_context`: the largest
         context among the others (a hint for cutting long key ranges; 0 = unknown). `even_contexts`: the
         decode requests' contexts are equally long (decode_contexts_even), which lets the decode kernel
-        keep each request on one XCD. Returns [T, Hq*D].
+        keep each request on one XCD. `decode_as_prefill` (or the module's DECODE_AS_PREFILL): the
+        single-token rows go through the prefill kernel too, as prompts of one token: a second
+        implementation of decoding to check the first against. Returns [T, Hq*D].
         (reference layers/attention.py:63-76: decode rows to the decode kernel, the rest to the
-        prefill kernel; csrc/paged_decode.cu, csrc/paged_prefill.cu.)"""
+        prefill kernel, or all rows to the prefill kernel in its `unified` mode; csrc/paged_decode.cu,
+        csrc/paged_prefill.cu.)"""
         T = q.shape[0]
         B = context_lens.numel()
         _check(q.dim() == 2 and q.shape[1] == Hq * D and q.stride(1) == 1, "attention: q must be [T, Hq*D], unit inner stride")
@@ -320,6 +326,11 @@ class HipBackend:
             return out
         lib = attn_lib(D)
         es = q.element_size()
+        if (decode_as_prefill or DECODE_AS_PREFILL) and num_decodes > 0:
+            ones = torch.arange(num_decodes + 1, dtype=torch.int32, device=q.device)
+            prefill_cu = ones if prefill_cu is None else torch.cat((ones[:-1], prefill_cu[:B - num_decodes + 1] + num_decodes))
+            max_prefill_context = max(max_prefill_context, max_decode_context)
+            num_decodes = 0
         if num_decodes > 0:
             part_size, num_parts = decode_partitions(num_decodes, Hq, Hkv, max_decode_context)
             scratch = _scratch(num_decodes * Hq * num_parts * (D + 2), q.device) if num_parts > 1 else None
@@ -342,7 +353,7 @@ class HipBackend:
 
     # -- matrix products -----------------------------------------------------------------
     def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
-               allow_partials: bool = False):
+               allow_partials: bool = False, out: torch.Tensor | None = None):
         """x [M, K] . w[N, K]^T (reference layers/linear.py:25-26: F.linear, no bias).
 
         float32: plain FMA kernel. bfloat16: the skinny MFMA kernel for up to 32 rows (64 for
@@ -352,23 +363,28 @@ class HipBackend:
         With allow_partials the result may be float32 partial sums [S, M, N] over slices of K for a
         consumer that adds them: from the skinny kernel when the output features are few
         (choose_ksplit), from the rows kernel for 17-32 rows over large weights (rows_takes), from the
-        library as a strided batch for 33-1,024 rows over large weights (library_splits)."""
+        library as a strided batch for 33-1,024 rows over large weights (library_splits).
+        `out` (not with allow_partials): a contiguous [M, N] tensor of the output dtype to write into."""
         _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: {tuple(x.shape)} x {tuple(w.shape)}^T")
         _check(x.dtype == w.dtype, f"linear: activation {x.dtype} and weight {w.dtype} differ")
         _check(x.stride(1) == 1 and w.stride(1) == 1, "linear: rows must be contiguous")
         M, K = x.shape
         N = w.shape[0]
         out_dtype = out_dtype or x.dtype
+        if out is not None:
+            _check(not allow_partials and out.shape == (M, N) and out.dtype == out_dtype and out.is_contiguous()
+                   and out.device == x.device, "linear: `out` must be a contiguous [M, N] tensor of the output dtype")
+        new = (lambda: out) if out is not None else (lambda: torch.empty((M, N), dtype=out_dtype, device=x.device))
         if x.dtype == torch.float32:
             _check(out_dtype == torch.float32, "linear: float32 inputs give float32 outputs")
-            y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+            y = new()
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_F32, ME_F32, M, N, K, _stream())
             return y
         aligned = (K % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
                    and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
         if not aligned:
-            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            y = new()
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
             return y
@@ -391,13 +407,13 @@ class HipBackend:
                         ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, _stream())
             return parts
         if skinny_takes(M, N, K):
-            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            y = new()
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), None, 1, M, N, K, 0, _stream())
             return y
         # many rows, or the head over a large vocabulary: the library product (float32 accumulation; the
         # float32 output form keeps the logits unrounded)
-        return library_product(x, w, out_dtype)
+        return library_product(x, w, out_dtype, out=out)
 
     def silu_mul_linear(self, gu: torch.Tensor, w: torch.Tensor, allow_partials: bool = False):
         """(silu(gu[:, :I]) * gu[:, I:]) . w[N, I]^T: the gating fused into the product for few
@@ -472,6 +488,7 @@ ROWS_MIN_WEIGHT = 16 * 1024 * 1024
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS wherever it fits (0: never)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
+DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
 # The fused form evaluates the gate in every workgroup (N/16 of them), which is free while the
 # product waits for its weights but not over a long K: at 4096x12288, one row, fused 63 us against
 # 27 us for the plain product after a separate gating kernel (3 us).

@@ -53,6 +53,7 @@ class DecoderModel(Part):
         self.optional_sources = set(optional_sources or ())
         self.device = None
         self.dtype = None
+        self._head_takes_out = None
         for i, call in enumerate(self.order):
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"run order entry {i} names layer {call.layer}, the model has {len(self.layers)}")
@@ -76,9 +77,8 @@ class DecoderModel(Part):
                 src = call.cache_of
                 if call_group[src] is None or not call_writes[src]:
                     raise ValueError(f"run order entry {i} reads the cache of entry {src}, which owns none")
-                src_need = needs[call_group[src]]
-                if (need.num_kv_heads, need.head_dim) != (src_need.num_kv_heads, src_need.head_dim):
-                    raise ValueError(f"run order entry {i} and entry {src} disagree on the cache's head layout")
+                if need.tensors != needs[call_group[src]].tensors:
+                    raise ValueError(f"run order entry {i} and entry {src} disagree on what a page of the cache holds")
                 call_group.append(call_group[src]); call_idx.append(call_idx[src]); call_writes.append(False)
                 continue
             g = keys.setdefault(need.group_key(), len(needs))
@@ -104,10 +104,19 @@ class DecoderModel(Part):
             h, residual = self.layers[call.layer].forward(h, residual, step, caches[i], states[i])
         return h, residual
 
-    def logits(self, h, residual, rows: torch.Tensor) -> torch.Tensor:
+    def logits(self, h, residual, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """Final norm of (h + residual), then the rows that want logits, then the head: float32
-        [len(rows), vocab] (reference models/qwen3.py:91,116-117; layers/embed_head.py:19-23)."""
+        [len(rows), vocab] (reference models/qwen3.py:91,116-117; layers/embed_head.py:19-23).
+        `out`: where to put them, for a head whose forward takes `out`; any other head's result is copied there."""
+        import inspect
         from ..kernels import ops
         x, _ = norm_of(self.final_norm, h, residual)
         x = ops.gather_rows(x, rows)
-        return self.head.forward(x)
+        if out is None:
+            return self.head.forward(x)
+        if self._head_takes_out is None:
+            self._head_takes_out = "out" in inspect.signature(self.head.forward).parameters
+        if self._head_takes_out:
+            return self.head.forward(x, out=out)
+        out.copy_(self.head.forward(x))
+        return out

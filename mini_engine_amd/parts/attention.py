@@ -51,7 +51,7 @@ class Attention(Mixer):
             self.position = None
 
     def cache_need(self):
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window)
 
     def forward(self, x, step, cache, state):
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim

@@ -31,26 +31,56 @@ class ParamSpec:
     dtype: str = "compute"
 
 
+PAGE = "page"      # stands in a PageTensor's shape for the axis that counts a page's tokens
+
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One tensor a mixer keeps per cached token. `shape` is what one page of one layer call looks
+    like, with PAGE where the page's tokens are counted: keys stored token by token under their head
+    are (heads, PAGE, head size); values transposed inside a page are (heads, head size, PAGE); one
+    latent vector per token is (PAGE, width). The pool allocates [pages, *shape] with PAGE replaced by
+    the engine's page size. `dtype`: "compute" (the engine's), "float32", "bfloat16" or "int32"."""
+
+    name: str
+    shape: tuple
+    dtype: str = "compute"
+
+    def __post_init__(self):
+        if sum(1 for d in self.shape if d == PAGE) != 1:
+            raise ValueError(f"page tensor {self.name!r}: exactly one axis of {self.shape} must be PAGE")
+
+    def sized(self, page_size: int) -> tuple:
+        return tuple(page_size if d == PAGE else int(d) for d in self.shape)
+
+
 @dataclass(frozen=True)
 class CacheNeed:
-    """What a mixer wants from the paged key/value cache.
+    """What a mixer wants from the paged cache: which tensors per token, and for how long.
 
-    ``window``: None keeps every key; n keeps the last n positions (pages that
+    ``window``: None keeps every token; n keeps the last n positions (pages that
     the window has passed are given back). Layers with equal needs share one
     group of pages and one block table per request.
     """
 
-    num_kv_heads: int
-    head_dim: int
+    tensors: tuple                     # of PageTensor
     window: int | None = None
 
+    @classmethod
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int | None = None) -> "CacheNeed":
+        """The layout of the attention kernels: K [pages, heads, page, head size], V [pages, heads, head
+        size, page] (V transposed inside a page: the P.V operand of the matrix cores is then one load)."""
+        return cls((PageTensor("k", (num_kv_heads, PAGE, head_dim)), PageTensor("v", (num_kv_heads, head_dim, PAGE))),
+                   window)
+
     def group_key(self) -> tuple:
-        return (self.num_kv_heads, self.head_dim, self.window)
+        return (self.tensors, self.window)
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Fixed-size per-request state of a mixer: one tensor ``[num_slots, *shape]``."""
+    """Fixed-size per-request state of a mixer: one tensor ``[num_slots + 1, *shape]``; the last row is
+    a spare that belongs to no request (padding rows of a step with a fixed layout name it)."""
 
     shape: tuple
     dtype: str = "float32"
@@ -147,7 +177,7 @@ class Mixer(Part):
 
         ``step``: the `StepContext` of this step. ``cache``: a `CacheView` (pages of this
         call's layer, or of the layer it reads) or None. ``state``: this call's state
-        tensor ``[num_slots, *shape]`` or None; rows are ``step.state_slots``.
+        tensor ``[num_slots + 1, *shape]`` or None; rows are ``step.state_slots``.
         """
         raise NotImplementedError
 
@@ -173,13 +203,22 @@ class LayerCall:
 
 @dataclass
 class CacheView:
-    """The pages one layer call reads and writes."""
+    """The pages one layer call reads and writes: per tensor of its CacheNeed, [num_pages + 1, *shape
+    of a page]. The last page is a spare that belongs to no request: padding rows of a step with a fixed
+    layout write there."""
 
     group: int                 # index of the page group (selects block table and slot mapping)
-    k: torch.Tensor            # [num_pages, Hkv, page, D]
-    v: torch.Tensor            # [num_pages, Hkv, D, page]  (transposed within a page)
+    tensors: dict              # PageTensor name -> tensor
     page_size: int
     write: bool = True
+
+    @property
+    def k(self) -> torch.Tensor:           # [pages, Hkv, page, D] of a keys-and-values layout
+        return self.tensors["k"]
+
+    @property
+    def v(self) -> torch.Tensor:           # [pages, Hkv, D, page]
+        return self.tensors["v"]
 
 
 # ---------------------------------------------------------------- registries

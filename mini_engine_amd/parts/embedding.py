@@ -33,5 +33,7 @@ class LMHead(Part):
     def matrix(self) -> torch.Tensor:
         return self.tied_to.weight if self.tied_to is not None else self.weight
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.linear(x, self.matrix(), torch.float32)
+    def forward(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """`out`: a float32 [rows, vocab] tensor to write the logits into (a step with a fixed layout
+        keeps one)."""
+        return ops.linear(x, self.matrix(), torch.float32, out=out)

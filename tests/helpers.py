@@ -126,3 +126,21 @@ def cuts_schedule(lengths: dict, pattern: list) -> list:
         if step:
             steps.append(step)
     return steps
+
+
+def assert_greedy_like_plain(folder: str, prompts: list, outputs: list, exact: bool, what: str = "") -> None:
+    """outputs[i]: the token ids generated greedily after prompts[i]. Each token must be the plain
+    implementation's best next token given what came before it; with exact=False (bfloat16) another
+    token passes only where the plain model's logits of the two lie within bfloat16's tolerance."""
+    if folder not in _plain_cache:
+        _plain_cache[folder] = plain_qwen3.read_model_folder(folder, torch.float64)
+    cfg, w = _plain_cache[folder]
+    for i, (prompt, out) in enumerate(zip(prompts, outputs)):
+        ids = list(prompt)
+        for tok in out:
+            z = plain_qwen3.logits(cfg, w, ids)[-1]
+            best = int(torch.argmax(z))
+            if tok != best:
+                assert not exact and float(z[best] - z[tok]) <= TOL_BF16 * float(z.abs().max()), \
+                    f"{what}: request {i} generated {tok} at position {len(ids)}, the plain implementation gives {best}"
+            ids.append(tok)

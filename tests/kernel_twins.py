@@ -56,9 +56,9 @@ def write_pages(k, v, slots, k_cache, v_cache, page):
 def qk_norm_rope_store(qkv, q_weight, k_weight, eps, table, positions, slots, k_cache, v_cache,
                        Hq, Hkv, D, page, store=True):
     T = qkv.shape[0]
-    q = _norm_rope(qkv[:, :Hq * D].float().view(T, Hq, D), q_weight, eps, table, positions)
+    q = _norm_rope(qkv[:, :Hq * D].float().clone().view(T, Hq, D), q_weight, eps, table, positions)
     if Hkv:
-        k = _norm_rope(qkv[:, Hq * D:(Hq + Hkv) * D].float().view(T, Hkv, D), k_weight, eps, table, positions)
+        k = _norm_rope(qkv[:, Hq * D:(Hq + Hkv) * D].float().clone().view(T, Hkv, D), k_weight, eps, table, positions)
     qkv[:, :Hq * D] = q.reshape(T, Hq * D).to(qkv.dtype)
     if store:
         v = qkv[:, (Hq + Hkv) * D:].view(T, Hkv, D)
@@ -102,8 +102,12 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
     return out
 
 
-def linear(x, w, out_dtype=None, allow_partials=False):
-    return (x.float() @ w.float().t()).to(out_dtype or x.dtype)
+def linear(x, w, out_dtype=None, allow_partials=False, out=None):
+    y = (x.float() @ w.float().t()).to(out_dtype or x.dtype)
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y
 
 
 def silu_mul_linear(gu, w, allow_partials=False):

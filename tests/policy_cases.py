@@ -1,0 +1,104 @@
+"""Scheduling policies and engine options run with a model through `LLM.generate`, each compared with the
+plain implementation's greedy tokens. `make(folder, **options)` builds the engine (on the GPU, or on the CPU
+with the plain kernel twins); `exact`: float32 (tokens must be equal) or bfloat16 (near-ties may differ)."""
+import helpers
+
+
+def _greedy(n):
+    from mini_engine_amd import SamplingParams
+    return SamplingParams(temperature=0, max_tokens=n, ignore_eos=True)
+
+
+def priority_policy(make, folders, exact):
+    """Mixed priorities under a pool so small that the least urgent request is evicted and fed again."""
+    folder = folders("B")
+    prompts = [helpers.random_ids(n, 384, 300 + n) for n in (24, 9, 40, 17, 33)]
+    llm = make(folder, scheduling_policy="priority", kvcache_block_size=8, num_kvcache_blocks=13, max_num_seqs=4,
+               max_num_batched_tokens=32, max_model_len=64, enable_prefix_caching=False)
+    outs = llm.generate(prompts, _greedy(10), use_tqdm=False, priorities=[2, 0, 1, 0, 2])
+    assert llm.scheduler.num_preemptions > 0, "the pool was large enough that nobody was evicted"
+    helpers.assert_greedy_like_plain(folder, prompts, [o["token_ids"] for o in outs], exact, "priority")
+    llm.manager.check_invariants()
+    assert llm.manager.num_free_pages() == 13
+
+
+def priority_order(make, folders, exact):
+    """With room for one request at a time, requests finish in the order of (priority, arrival)."""
+    from mini_engine_amd import SamplingParams
+    folder = folders("A")
+    llm = make(folder, scheduling_policy="priority", kvcache_block_size=16, num_kvcache_blocks=8, max_num_seqs=1,
+               max_num_batched_tokens=64, max_model_len=64)
+    prompts = [helpers.random_ids(6, 256, 40 + i) for i in range(5)]
+    ranks = [3, 1, 2, 1, 0]
+    ids = [llm.add_request(p, SamplingParams(temperature=0, max_tokens=3, ignore_eos=True), priority=r)
+           for p, r in zip(prompts, ranks)]
+    finished, outs = [], {}
+    while not llm.is_finished():
+        for rid, toks in llm.step()[0]:
+            finished.append(rid); outs[rid] = toks
+    assert finished == [ids[i] for i in (4, 1, 3, 2, 0)]
+    helpers.assert_greedy_like_plain(folder, prompts, [outs[i] for i in ids], exact, "priority order")
+
+
+def long_prefill_threshold(make, folders, exact):
+    """Prompts go in five tokens at a time beside requests that already decode."""
+    folder = folders("B")
+    prompts = [helpers.random_ids(n, 384, 310 + n) for n in (3, 23, 41, 12)]
+    llm = make(folder, long_prefill_token_threshold=5, kvcache_block_size=8, num_kvcache_blocks=40, max_num_seqs=4,
+               max_num_batched_tokens=32, max_model_len=64)
+    sizes = []
+    step = llm.step
+
+    def counting():
+        out = step()
+        sizes.append(out[1])
+        return out
+    llm.step = counting
+    outs = llm.generate(prompts, _greedy(9), use_tqdm=False)
+    assert max(sizes) <= 4 * 5 and any(0 < s <= 5 for s in sizes), sizes       # no request ran more than 5 prompt tokens a step
+    helpers.assert_greedy_like_plain(folder, prompts, [o["token_ids"] for o in outs], exact, "threshold")
+
+
+def prefill_first(make, folders, exact):
+    """Whole prompts first, decoding only in steps that admit nobody; a pool that forces evictions."""
+    folder = folders("A")
+    prompts = [helpers.random_ids(n, 256, 320 + n) for n in (15, 31, 16, 47, 14, 30)]
+    llm = make(folder, enable_chunked_prefill=False, kvcache_block_size=16, num_kvcache_blocks=6, max_num_seqs=3,
+               max_num_batched_tokens=64, max_model_len=64, enable_prefix_caching=False)
+    outs = llm.generate(prompts, _greedy(12), use_tqdm=False)
+    assert llm.scheduler.num_preemptions > 0
+    helpers.assert_greedy_like_plain(folder, prompts, [o["token_ids"] for o in outs], exact, "prefill first")
+    assert llm.manager.num_free_pages() == 6
+
+
+def many_live_requests(make, folders, exact):
+    """300 requests decoding together: more rows than any power-of-two layout up to 256 holds."""
+    folder = folders("A")
+    prompts = [helpers.random_ids(2 + i % 7, 256, 1000 + i) for i in range(300)]
+    llm = make(folder, kvcache_block_size=16, num_kvcache_blocks=300, max_num_seqs=300, max_num_batched_tokens=4096,
+               max_model_len=16)
+    outs = llm.generate(prompts, _greedy(4), use_tqdm=False)
+    assert len(llm.scheduler.running) == 0 and llm.runner.graphs.replays >= 3
+    assert any(c.bucket == 384 for c in llm.runner.graphs.captured.values())
+    helpers.assert_greedy_like_plain(folder, prompts[::13], [o["token_ids"] for o in outs][::13], exact, "300 live")
+
+
+def windowed_model(make, folders, exact):
+    """Tiny C (sliding windows on two of four layers: two page groups) through the scheduler: pages behind the
+    window given back while requests run, evictions and feeding again, steps run ahead or not."""
+    folder = folders("C")
+    prompts = [helpers.random_ids(n, 300, 330 + n) for n in (5, 50, 33, 70, 18)]
+    for options in (dict(num_kvcache_blocks=40, max_num_batched_tokens=64),
+                    dict(num_kvcache_blocks=11, max_num_batched_tokens=16, run_ahead=True),
+                    dict(num_kvcache_blocks=11, max_num_batched_tokens=16, run_ahead=False),
+                    dict(num_kvcache_blocks=14, max_num_batched_tokens=128, enable_chunked_prefill=False)):
+        llm = make(folder, kvcache_block_size=16, max_num_seqs=4, max_model_len=128, **options)
+        outs = llm.generate(prompts, _greedy(16), use_tqdm=False)
+        if options["num_kvcache_blocks"] == 11:
+            assert llm.scheduler.num_preemptions > 0, "nobody was evicted"
+        helpers.assert_greedy_like_plain(folder, prompts, [o["token_ids"] for o in outs], exact, f"windowed {options}")
+        llm.manager.check_invariants()
+        assert all(llm.manager.num_free_pages(g) == options["num_kvcache_blocks"] for g in range(2))
+
+
+ALL = [priority_policy, priority_order, long_prefill_threshold, prefill_first, many_live_requests, windowed_model]

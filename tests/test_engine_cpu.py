@@ -119,6 +119,7 @@ def test_running_one_step_ahead_changes_no_token(folders, plain_backend):
     eos = free_run[1][11]                                     # request 1 meets its end token in mid-flight
     want = [o[:o.index(eos) + 1] if eos in o else o for o in free_run]
     assert len(want[1]) < 30
+    helpers.assert_greedy_like_plain(folder, prompts[0::2], want[0::2], True, "run ahead")          # the greedy ones
     for caching in (False, True):
         plain = _llm(folder, run_ahead=False, eos=eos, enable_prefix_caching=caching, **kw)
         assert [o["token_ids"] for o in plain.generate(prompts, sps, use_tqdm=False)] == want
@@ -190,6 +191,7 @@ def test_prefix_hits_give_the_same_tokens(folders, plain_backend):
         for _, t in warm.step()[0]:
             second = t
     assert [first, second] == want
+    helpers.assert_greedy_like_plain(folder, prompts, want, True, "prefix hits")
 
 
 def test_replay_program_on_cpu(folders, plain_backend, tmp_path, monkeypatch, capsys):
@@ -311,3 +313,18 @@ def test_toy_architecture_on_cpu(plain_backend):
     position encoding, registered from tests/toy_arch.py, stepped through the real runner."""
     import toy_arch
     toy_arch.run_toy("cpu", torch.float32, 1e-5)
+
+
+def test_toy_architecture_through_the_engine_on_cpu(plain_backend):
+    """The same toy architecture from a written folder through `LLM.generate`: scheduler, state slots and a
+    second page group under admission, eviction and finish, the decode steps' fixed layout, steps run ahead."""
+    import toy_arch
+    toy_arch.run_toy_engine("cpu", "float32", capture=False)
+
+
+import policy_cases
+
+
+@pytest.mark.parametrize("case", policy_cases.ALL, ids=lambda c: c.__name__)
+def test_policies_with_a_model_on_cpu(folders, plain_backend, case):
+    case(_llm, folders, exact=True)

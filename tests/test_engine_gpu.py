@@ -163,6 +163,7 @@ def test_running_one_step_ahead_changes_no_token(folders, dtype):
     ahead = _llm(folder, dtype, run_ahead=True, eos=eos, **kw)
     assert [o["token_ids"] for o in ahead.generate(prompts, sps, use_tqdm=False)] == want
     assert one_by_one.steps_run_ahead == 0 and ahead.steps_run_ahead >= 15
+    helpers.assert_greedy_like_plain(folder, prompts[0::2], want[0::2], dtype == "float32", "run ahead")      # the greedy ones
     ahead.manager.check_invariants()
     assert ahead.manager.num_free_pages() == 40 and not ahead.manager.held
 
@@ -184,6 +185,7 @@ def test_prefix_hits_give_the_same_tokens(folders, dtype):
     assert warm.manager.find_prefix_hit(prompts[1]).num_pages == 2          # 32 of the 40 shared tokens
     second = warm.generate(prompts[1:], sp, use_tqdm=False)[0]["token_ids"]
     assert [first, second] == want
+    helpers.assert_greedy_like_plain(folder, prompts, want, dtype == "float32", "prefix hits")
 
 
 def test_float32_logits_do_not_depend_on_the_cut_bitwise(folders):
@@ -276,19 +278,21 @@ def test_real_layer_sizes(tmp_path_factory, dtype):
         assert err <= tol, f"{r}: {err:.3g}"
 
 
-def test_wide_layer_sizes_take_the_products_with_partial_sums(tmp_path_factory):
-    """One layer of Qwen3-8B's width (hidden 4096, 32 query / 8 key heads of 128, intermediate 12288): o and
-    down are large enough for the forms that hand float32 partial sums over slices of K to the norm that
-    follows (the library as a strided batch at 300 and 127 rows, the rows kernel at 28), which the narrow test
-    configurations never reach; then decoding; against the plain implementation."""
+@pytest.mark.parametrize("hidden,Hq,Hkv,inter", [(4096, 32, 8, 12288), (5120, 64, 8, 25600)], ids=["8b_width", "32b_width"])
+def test_wide_layer_sizes_take_the_products_with_partial_sums(tmp_path_factory, hidden, Hq, Hkv, inter):
+    """One layer of Qwen3-8B's width (hidden 4096, 32 query / 8 key heads of 128, intermediate 12288) and of
+    Qwen3-32B's (hidden 5120, 64 query / 8 key heads: groups of 8, intermediate 25600): o and down are large
+    enough for the forms that hand float32 partial sums over slices of K to the norm that follows (the library
+    as a strided batch at 300 and 127 rows, the rows kernel at 28), which the narrow test configurations never
+    reach; then decoding; against the plain implementation."""
     from mini_engine_amd.config.model_config import Qwen3Config
     from mini_engine_amd.kernels import ops
     from mini_engine_amd.weights.random_init import write_random_model
-    cfgd = dict(architectures=["Qwen3ForCausalLM"], vocab_size=1009, hidden_size=4096, intermediate_size=12288,
-                num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
+    cfgd = dict(architectures=["Qwen3ForCausalLM"], vocab_size=1009, hidden_size=hidden, intermediate_size=inter,
+                num_hidden_layers=1, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=128, rms_norm_eps=1e-6,
                 rope_theta=1e6, tie_word_embeddings=True, max_position_embeddings=4096)
-    assert ops.library_splits(300, 4096, 4096) == 4 and ops.library_splits(127, 4096, 12288) == 8
-    assert ops.rows_takes(28, 4096, 12288) and ops.rows_takes(28, 4096, 4096)
+    assert ops.library_splits(300, hidden, Hq * 128) > 1 and ops.library_splits(127, hidden, inter) == 8
+    assert ops.rows_takes(28, hidden, inter) and ops.rows_takes(28, hidden, Hq * 128)
     folder = write_random_model(Qwen3Config.from_dict(cfgd), 5, str(tmp_path_factory.mktemp("wide")))
     model = load_model(folder, "cuda", torch.bfloat16, 1024)
     manager = CacheManager(64, 16, ModelRunner.windows_of(model), enable_prefix_caching=False)
@@ -305,3 +309,26 @@ def test_wide_layer_sizes_take_the_products_with_partial_sums(tmp_path_factory):
         got = d.result(r)
         err = helpers.rel_err(got, helpers.plain_logits(folder, ids)[: got.shape[0]])
         assert err <= helpers.TOL_BF16, f"{r}: {err:.3g}"
+
+
+def test_single_token_rows_through_the_prefill_kernel_in_the_engine(folders, monkeypatch):
+    """The mixed case of every configuration with the step's single-token rows sent through the prefill kernel
+    instead of the decode kernel: a second implementation of decoding under the same cuts, against the plain
+    implementation (the reference's `unified` mode, layers/attention.py:66-68)."""
+    from mini_engine_amd.kernels import ops
+    monkeypatch.setattr(ops, "DECODE_AS_PREFILL", True)
+    env = Env(folders, torch.bfloat16)
+    for name in ("A", "B", "C"):
+        engine_cases.mixed_with_reuse(env, name)
+        engine_cases.tail_one_by_one(env, name)
+        engine_cases.batch_of_decodes(env, name)
+
+import policy_cases
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", policy_cases.ALL, ids=lambda c: c.__name__)
+def test_policies_with_a_model(folders, dtype, case):
+    """Priority scheduling, a cap on prompt portions, whole prompts first, 300 requests decoding together and a
+    windowed model, each through `LLM.generate` against the plain implementation's greedy tokens."""
+    case(lambda folder, **kw: _llm(folder, dtype, **kw), folders, exact=dtype == "float32")

@@ -215,7 +215,8 @@ def prefill_form(request, monkeypatch):
 
 
 SHAPES = [(4, 2, 16, 16), (6, 2, 32, 8), (4, 1, 48, 16), (16, 8, 128, 16), (8, 8, 64, 32), (32, 1, 64, 16), (2, 2, 128, 64),
-          (80, 1, 32, 16)]      # the last: more heads in a group than one round of a workgroup's columns
+          (80, 1, 32, 16),      # more heads in a group than one round of a workgroup's columns
+          (40, 8, 128, 16), (64, 8, 128, 16)]      # groups of 5 and of 8 at head size 128 (Qwen3-14B and 32B)
 
 
 @pytest.mark.parametrize("Hq,Hkv,D,page", SHAPES)
@@ -268,6 +269,35 @@ def test_attention_far_key_stands_out(prefill_form, dtype):
         close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(40, 8), (64, 8)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_attention_wide_groups_at_head_size_128(prefill_form, monkeypatch, Hq, Hkv, window):
+    """Groups of 5 and 8 query heads at head size 128: a far key, a window's edge and long tiles cut into
+    segments, decode and prompt rows in one step."""
+    seqs = [(1024, 1), (150, 1), (700, 130), (1024, 40), (33, 33)]
+    for peak, seg_keys in ((None, None), (0, None), (1023 if window is None else 950, None), (600 if window is None else 1000, 96)):
+        monkeypatch.setattr(ops, "PREFILL_SEGMENT_KEYS", seg_keys)
+        args = _attention_case(torch.bfloat16, Hq, Hkv, 128, 16, seqs, window=window, seed=Hq, peak=peak)
+        close(hip().paged_attention(*args, max_prefill_context=1024), twin.paged_attention(*args), 1.5e-2)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(4, 2, 16, 16), (6, 2, 32, 8), (16, 8, 128, 16), (40, 8, 128, 16)])
+@pytest.mark.parametrize("window", [None, 50])
+def test_decode_rows_through_the_prefill_kernel(prefill_form, Hq, Hkv, D, page, window):
+    """Two implementations of decoding cross-checked: the same step with its single-token rows sent to the
+    decode kernel, and with every row sent to the prefill kernel (`decode_as_prefill`), each against the
+    plain twin (the reference's `unified` mode: layers/attention.py:66-68)."""
+    for seqs in ([(7, 1), (130, 1), (2, 1), (1, 1)], [(700, 1), (33, 1), (900, 1), (128, 1), (129, 1)],
+                 [(40, 1), (300, 1), (50, 50), (90, 7), (2, 2)]):
+        args = _attention_case(torch.bfloat16, Hq, Hkv, D, page, seqs, window=window, seed=len(seqs) + D, peak=0)
+        want = twin.paged_attention(*args)
+        split = hip().paged_attention(*args)
+        unified = hip().paged_attention(*args, decode_as_prefill=True)
+        close(split, want, 1.5e-2)
+        close(unified, want, 1.5e-2)
+        close(unified, split, 2e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [1, 7, 16, 24, 100])
 def test_attention_window_edges(prefill_form, dtype, window):
@@ -310,6 +340,7 @@ def test_attention_generic_path_takes_odd_sizes():
     args = _attention_case(torch.bfloat16, 4, 2, 32, 24, [(100, 1), (50, 50), (30, 3)], seed=3)   # page 24: no power of two
     close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
     args = _attention_case(torch.bfloat16, 4, 2, 64, 16, [(300, 1), (70, 70)], seed=2)
+    close(hip().paged_attention(*args, force_simple=True), twin.paged_attention(*args), 1.5e-2)
     close(hip().paged_attention(*args, force_simple=True), hip().paged_attention(*args), 1.5e-2)
 
 

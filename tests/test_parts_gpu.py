@@ -74,7 +74,7 @@ def test_attention_part_alone(dtype, tol, window):
     k_cache = torch.full((6, Hkv, page, D), float("nan"), device=DEV, dtype=dtype)
     v_cache = torch.full((6, Hkv, D, page), float("nan"), device=DEV, dtype=dtype)
     from mini_engine_amd.parts import CacheView
-    view = CacheView(0, k_cache, v_cache, page)
+    view = CacheView(0, {"k": k_cache, "v": v_cache}, page)
     table = [4, 1, 5, 0, 2]
     outs = []
     for a, b in ((0, 20), (20, T)):
@@ -103,3 +103,11 @@ def test_toy_architecture_registers_builds_and_steps(dtype, tol):
     architecture, all defined in tests/toy_arch.py and registered from there: no framework file changes."""
     import toy_arch
     toy_arch.run_toy(DEV, dtype, tol)
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_toy_architecture_through_the_engine_and_captured_graphs(dtype_name):
+    """The toy architecture (state of its own, a cache of one tensor per token) from a written folder through
+    `LLM.generate`: its decode steps are captured as graphs and launched one ahead, with no framework file changed."""
+    import toy_arch
+    toy_arch.run_toy_engine(DEV, dtype_name, capture=True)

@@ -50,37 +50,78 @@ def steps_from_schedule(ids, schedule, ends=True):
     return steps
 
 
+def most_live_tokens(steps) -> int:
+    """The --max-tokens a trace needs: the most tokens live requests hold at any time, each request's count
+    rounded up to a multiple of 64 (a request is live from its first step to the step that ends it)."""
+    fed, most = {}, 0
+    for s in steps:
+        for e in s["entries"]:
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+        most = max(most, sum(-(-n // 64) * 64 for n in fed.values()))
+        for r in s["end"]:
+            fed.pop(r)
+    return most
+
+
+def pages_used_again(folder, steps, max_tokens, page) -> dict:
+    """Replays the trace's allocations on a cache manager of the program's size (it hands out pages in a fixed
+    order): per request, how many of its pages had belonged to a request that ended before."""
+    from mini_engine_amd.cache.manager import CacheManager
+    from mini_engine_amd.config.model_config import load_model_config
+    from mini_engine_amd.engine.runner import ModelRunner
+    from mini_engine_amd.registry import build_model
+    manager = CacheManager(max_tokens // page, page, ModelRunner.windows_of(build_model(load_model_config(folder))),
+                           enable_prefix_caching=False)
+    fed, given_back, again = {}, set(), {}
+    for s in steps:
+        for e in s["entries"]:
+            assert manager.allocate(e["id"], fed.get(e["id"], 0), len(e["tokens"]))
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+            again[e["id"]] = len(given_back & {p for p in manager.block_table(e["id"]) if p >= 0})
+        for r in s["end"]:
+            given_back |= {p for p in manager.block_table(r) if p >= 0}
+            manager.free(r)
+            fed.pop(r)
+    return again
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_replay_cuts(folders, tmp_path, dtype, name):
     folder = folders(name)
     V = helpers.CONFIGS[name]["vocab_size"]
+    page = helpers.PAGE[name]
     tol = helpers.TOL_F32 if dtype == "float32" else helpers.TOL_BF16
-    lens = {"a": 100, "b": 61, "c": 40, "d": 77, "e": 90}
+    lens = {"a": 128, "b": 64, "c": 62, "d": 126, "e": 120}
     ids = {r: helpers.random_ids(n, V, 40 + i) for i, (r, n) in enumerate(lens.items())}
     cases = {
         "whole": [{r: (0, lens[r])} for r in ("a", "b")],
-        "tail": [{"a": (0, 68)}] + [{"a": (t, t + 1)} for t in range(68, 100)],
-        "portions": helpers.cuts_schedule({"a": 100}, [2, 3, 31, 2, 17, 1, 8]),
-        # five requests, at most four live, in a pool of 4 x 128 tokens less one request: later ones reuse pages
+        "tail": [{"a": (0, 96)}] + [{"a": (t, t + 1)} for t in range(96, 128)],
+        "portions": helpers.cuts_schedule({"a": 128}, [2, 3, 31, 2, 17, 1, 8]),
+        # five requests, at most four live, in a pool of exactly what they hold at most: e, which starts when
+        # c has ended, cannot be served from pages nobody has used
         "mixed": helpers.cuts_schedule({r: lens[r] for r in ("a", "b", "c", "d")}, [19, 1, 1, 2, 33, 1, 7, 1]),
     }
     for case, schedule in cases.items():
         steps = steps_from_schedule(ids, schedule)
         if case == "mixed":      # e starts once c (the shortest) has ended, taking over its pages
             last_c = max(i for i, st in enumerate(schedule) if "c" in st)
-            extra = helpers.cuts_schedule({"e": 90}, [5, 1, 40, 1])
+            extra = helpers.cuts_schedule({"e": lens["e"]}, [5, 1, 40, 1])
             for j, st in enumerate(extra):
                 i = last_c + 1 + j
                 a, b = st["e"]
                 entry = {"id": "e", "tokens": ids["e"][a:b], "want": list(range(b - a))}
                 if i < len(steps):
                     steps[i]["entries"].append(entry)
-                    if b == 90: steps[i]["end"].append("e")
+                    if b == lens["e"]: steps[i]["end"].append("e")
                 else:
-                    steps.append({"step": i, "entries": [entry], "end": ["e"] if b == 90 else []})
+                    steps.append({"step": i, "entries": [entry], "end": ["e"] if b == lens["e"] else []})
+        max_tokens = most_live_tokens(steps)
+        if case == "mixed":
+            assert max(len(s["entries"]) for s in steps) == 4
+            assert pages_used_again(folder, steps, max_tokens, page)["e"] >= 2, "e was served from pages nobody had used"
         out = str(tmp_path / f"{case}")
-        replay(folder, dtype, steps, out, max_tokens=128 * 3 + 64, page=helpers.PAGE[name])
+        replay(folder, dtype, steps, out, max_tokens=max_tokens, page=page)
         got = collect(steps, out, V)
         for r, g in got.items():
             err = helpers.rel_err(g, helpers.plain_logits(folder, ids[r]))
