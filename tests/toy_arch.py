@@ -95,8 +95,9 @@ class ToyLinear(FeedForward):
 @register_part("feed_forward", "toy_top1_experts")
 class ToyExperts(FeedForward):
     """Every token goes to the expert with the largest router logit and is scaled by that expert's softmax
-    weight: y = p_e . W_e x, e = argmax(R x). The router works in float32 whatever the compute dtype; the
-    tokens are grouped by expert, so each expert sees its tokens as one matrix."""
+    weight: y = p_e . W_e x, e = argmax(R x). The router works in float32 whatever the compute dtype. Each
+    token picks its expert's matrix on the device (no value travels to the host, so a decode step with this
+    feed-forward can be captured as a graph)."""
 
     def __init__(self, hidden_size, num_experts, router_scale):
         super().__init__()
@@ -107,13 +108,8 @@ class ToyExperts(FeedForward):
     def forward(self, x):
         logits = (x.float() @ self.router.T) * self.router_scale
         weight, chosen = torch.softmax(logits, -1).max(-1)
-        out = torch.empty_like(x)
-        for e in range(self.num_experts):
-            rows = (chosen == e).nonzero().flatten()
-            if rows.numel():
-                y = (x[rows] @ self.experts[e].T).float() * weight[rows, None]
-                out[rows] = y.to(x.dtype)
-        return out
+        y = torch.bmm(self.experts[chosen], x.unsqueeze(-1)).squeeze(-1)        # [T, n, k] x [T, k, 1]
+        return (y.float() * weight[:, None]).to(x.dtype)
 
 
 @register_part("position_encoding", "toy_interleaved_rotary")
