@@ -21,6 +21,7 @@ import torch
 
 from ..kernels import ops
 from .context import GroupStep, StepContext
+from .packing import StepLayout, context_of, pack_step, views_of
 
 PENDING = -1      # the runner's marker for a token that is still on the device (runner.PENDING)
 
@@ -123,7 +124,7 @@ class DecodeGraphs:
         # graph may reuse what the others' activations occupy. Nothing a graph allocates outlives its
         # capture: the logits, the one result that is read afterwards, go into `self.logits`, one buffer
         # for all layouts (a layout that kept its own would pin 150 MB of the pool at 256 rows).
-        self.pool = torch.cuda.graph_pool_handle() if (capture and runner.device.type == "cuda") else None
+        self.pool = runner.graph_pool() if capture else None
         self.logits = None
         self.replays = 0
         self.advances = 0        # of those, steps whose tables and slots were carried on from the step before
@@ -297,29 +298,162 @@ class DecodeGraphs:
     def _capture(self, cap: _Captured) -> None:
         # one eager run first: libraries load, scratch buffers get their size, the caching allocator warms up
         # (it rewrites this step's cache entries with the same values the replay will write)
-        if self.logits is None:
-            r = self.runner
-            self.logits = torch.empty((bucket_of(self.max_bucket), r.vocab_size), dtype=torch.float32, device=r.device)
+        self.logits = self.runner.graph_logits()
         out = self.logits[:cap.bucket]
-        # Cache writes can be repeated, state updates cannot: what the eager run does to the requests'
-        # state is taken back, the replay that follows does it for good.
-        states = [st for st in self.runner.pool.states if st is not None]
-        kept = [st.clone() for st in states]
-        self._forward(cap, out)
-        for st, was in zip(states, kept):
-            st.copy_(was)
-        del kept
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        # No garbage collection while the stream is capturing: a collector run that finds an old
-        # engine's graphs, events or pinned buffers frees them with calls that a capturing stream
-        # refuses, and the process aborts inside a destructor. (torch collects once on entering.)
-        collecting = gc.isenabled()
-        gc.disable()
-        try:
-            with torch.cuda.graph(graph, pool=self.pool):
-                self._forward(cap, out)
-        finally:
-            if collecting:
-                gc.enable()
-        cap.graph = graph
+        cap.graph = capture_graph(self.runner, self.pool, lambda: self._forward(cap, out))
+
+
+def capture_graph(runner, pool, forward):
+    """Run `forward` once eagerly, then capture it. The eager run comes first so that libraries load, scratch
+    buffers get their size and the caching allocator warms up outside the capture."""
+    # Cache writes can be repeated, state updates cannot: what the eager run does to the requests'
+    # state is taken back, the replay that follows does it for good.
+    states = [st for st in runner.pool.states if st is not None]
+    kept = [st.clone() for st in states]
+    forward()
+    for st, was in zip(states, kept):
+        st.copy_(was)
+    del kept
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    # No garbage collection while the stream is capturing: a collector run that finds an old
+    # engine's graphs, events or pinned buffers frees them with calls that a capturing stream
+    # refuses, and the process aborts inside a destructor. (torch collects once on entering.)
+    collecting = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph, pool=pool):
+            forward()
+    finally:
+        if collecting:
+            gc.enable()
+    return graph
+
+
+# ------------------------------------------------------------------------------------------------
+# Steps that are not plain decoding: portions of prompts, alone or beside single tokens.
+
+def _round_up(n: int, to: int) -> int:
+    return -(-n // to) * to
+
+
+def token_bucket(tokens: int) -> int:
+    """Tokens of the padded layout that holds `tokens` prompt tokens and at least one of padding: steps of 32
+    up to 512 tokens, of 64 up to 4,096, of 256 beyond (at most a sixteenth more work than the step has)."""
+    need = tokens + 1
+    if need <= 512:
+        return _round_up(need, 32)
+    if need <= 4096:
+        return _round_up(need, 64)
+    return _round_up(need, 256)
+
+
+class _CapturedStep:
+    def __init__(self, runner, layout: StepLayout):
+        self.layout = layout
+        self.n = layout.segments()[1]
+        on_gpu = runner.device.type == "cuda"
+        self.pinned = [torch.empty(self.n, dtype=torch.int32, pin_memory=on_gpu) for _ in range(2)]
+        self.events = [None, None]
+        self.flip = 0
+        self.dev = torch.zeros(self.n, dtype=torch.int32, device=runner.device)
+        self.graph = None
+        self.replays = 0
+
+    def staging(self):
+        i = self.flip
+        self.flip ^= 1
+        if self.events[i] is not None:
+            self.events[i].synchronize()           # the copy that last used this buffer has finished
+        return i, self.pinned[i]
+
+
+class MixedGraphs:
+    """Steps with prompt portions, padded to a layout shared by many steps and replayed as a graph.
+
+    Launched kernel by kernel from Python, such a step costs the host a few milliseconds whatever its size,
+    which for small models and short portions is more than the GPU needs. A step's shape is rounded up to a
+    layout (single-token rows to a bucket, prompt tokens to a bucket through one padding request, block-table
+    columns, context caps, rows that want logits); a layout that has come up `capture_after` times is captured
+    on its next appearance and replayed from then on. Layouts that come up once (the ramp of a workload) stay
+    eager, exactly sized. The captured work is the model's own forward pass over the padded step."""
+
+    def __init__(self, runner, max_rows: int, capture: bool = True, capture_after: int = 2, max_graphs: int = 48):
+        self.runner = weakref.proxy(runner)
+        self.max_rows = max_rows
+        self.capture = capture
+        self.capture_after = capture_after
+        self.max_graphs = max_graphs
+        self.captured: dict = {}
+        self.sightings: dict = {}
+        self.pool = runner.graph_pool() if capture else None
+        self.replays = 0
+
+    def padded(self, exact: StepLayout) -> StepLayout | None:
+        r = self.runner
+        if (exact.prefill_reqs == 0 or exact.rows > self.max_rows or r.vocab_size is None
+                or not (r.device.type == "cuda" or not self.capture)):
+            return None
+        most_ctx = -(-r.max_positions // 8) * 8
+        return StepLayout(
+            decode_rows=bucket_of(exact.decode_rows) if exact.decode_rows else 0,
+            prefill_reqs=exact.prefill_reqs + 1, prefill_tokens=token_bucket(exact.prefill_tokens),
+            rows=bucket_of(exact.rows) if exact.rows else 0,
+            max_blocks=tuple(_round_up(mb, 64) for mb in exact.max_blocks),
+            decode_ctx=min(_round_up(exact.decode_ctx, CONTEXT_STEP), most_ctx) if exact.decode_rows else 0,
+            prefill_ctx=_round_up(exact.prefill_ctx, CONTEXT_STEP), even=exact.even)
+
+    def lookup(self, exact: StepLayout):
+        """The captured (or about to be captured) layout that takes this step, or None: run it eagerly."""
+        layout = self.padded(exact)
+        if layout is None:
+            return None
+        cap = self.captured.pop(layout, None)
+        if cap is None:
+            seen = self.sightings.get(layout, 0) + 1
+            if seen <= self.capture_after:
+                if len(self.sightings) > 4096:
+                    self.sightings.clear()
+                self.sightings[layout] = seen
+                return None
+            self.sightings.pop(layout, None)
+            cap = _CapturedStep(self.runner, layout)
+            while len(self.captured) >= self.max_graphs:        # the one unused for longest goes
+                del self.captured[next(iter(self.captured))]
+        self.captured[layout] = cap                               # most recently used last
+        return cap
+
+    def run(self, cap: _CapturedStep, token_lists, starts, tables, state_slots, rows, names):
+        r = self.runner
+        layout = cap.layout
+        i, host = cap.staging()
+        q_lens, first = pack_step(layout, host.numpy(), token_lists, starts, tables, state_slots, rows, r.manager.page_size,
+                                  [r.pool.spare_page(g) for g in range(len(layout.max_blocks))], r.pool.spare_state_slot,
+                                  r.vocab_size, names)
+        cap.dev.copy_(host, non_blocking=True)
+        if r.device.type == "cuda":
+            ev = torch.cuda.Event()
+            ev.record()
+            cap.events[i] = ev
+        r.zero_fresh_state(state_slots, starts)
+        cap.replays += 1
+        self.replays += 1
+        R = len(rows)
+        if not self.capture:
+            out = self._forward(cap, None, q_lens, first)
+            return out[:R] if R else None
+        logits = r.graph_logits()
+        if cap.graph is None:
+            out = logits[:layout.rows] if layout.rows else None
+            cap.graph = capture_graph(r, self.pool, lambda: self._forward(cap, out, q_lens, first))
+        cap.graph.replay()
+        return logits[:R] if R else None
+
+    def _forward(self, cap: _CapturedStep, out, q_lens, first):
+        r = self.runner
+        layout = cap.layout
+        tokens, rows = views_of(layout, cap.dev)
+        h, residual = r.model.forward(tokens, context_of(layout, cap.dev, q_lens, first), r.pool.views, r.pool.states)
+        if not layout.rows:
+            return None
+        return r.model.logits(h, residual, rows[:layout.rows], out=out)

@@ -100,8 +100,9 @@ class LLMEngine:
         prompt step and the largest decode step, then the pool from the allocator's peak).
 
         Kept free beside the pool: the measured peak of the larger of the two steps (activations,
-        attention scratch, the library's workspace is allocated by then and counts as used), and for
-        the decode graphs their memory pool (the decode step's peak once more) and the logits buffer."""
+        attention scratch; the library's workspace is allocated by then and counts as used), and for
+        the captured graphs their memory pool (a captured step needs what the eager one needs: the same
+        peak once more) and the logits buffer."""
         cfg = self.config
         if self.device.type != "cuda":
             raise RuntimeError("the cache pool can be sized from free memory only on a GPU: give num_kvcache_blocks")
@@ -112,7 +113,7 @@ class LLMEngine:
         del probe, probe_manager
         torch.cuda.empty_cache()
         vocab = getattr(self.model.embedding, "vocab_size", 0)
-        graphs = decode_peak + min(cfg.max_num_seqs, 256) * vocab * 4 if cfg.use_graphs else 0
+        graphs = step_peak + (cfg.max_num_seqs + 128) * vocab * 4 if cfg.use_graphs else 0
         self.reserved_bytes = step_peak + graphs
         free, total = torch.cuda.mem_get_info(self.device)
         budget = int(total * cfg.gpu_memory_utilization) - (total - free) - self.reserved_bytes

@@ -16,7 +16,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.pool import CachePool, page_bytes
 from ..kernels import ops
-from .context import GroupStep, StepContext
+from .packing import context_of, exact_layout, pack_step, views_of
 
 
 @dataclass
@@ -61,7 +61,10 @@ def _pad4(n: int) -> int:
 
 class ModelRunner:
     def __init__(self, model, manager: CacheManager, dtype: torch.dtype, device, max_positions: int,
-                 poison_cache: bool = False, use_graphs: bool = False, max_decode_rows: int = 256):
+                 poison_cache: bool = False, use_graphs: bool = False, max_decode_rows: int = 256,
+                 mixed_graphs_after: int | None = 2):
+        """use_graphs: decode steps are replayed as HIP graphs, and so are steps with prompt portions whose
+        padded shape has come up more than `mixed_graphs_after` times (None: those always run eagerly)."""
         self.model = model
         self.manager = manager
         self.dtype = dtype
@@ -76,10 +79,17 @@ class ModelRunner:
         if self.pool.has_state and manager.num_state_slots < 1:
             raise ValueError("the model keeps per-request state but the cache manager has no state slots")
         self.vocab_size = model.embedding.vocab_size if hasattr(model.embedding, "vocab_size") else None
-        self.graphs = None
+        self.max_decode_rows = max_decode_rows
+        self._graph_pool = None
+        self._graph_logits = None
+        self.graphs = None              # plain decode steps
+        self.mixed_graphs = None        # steps with prompt portions
         if use_graphs:
-            from .graphs import DecodeGraphs
-            self.graphs = DecodeGraphs(self, max_bucket=max_decode_rows, capture=self.device.type == "cuda")
+            from .graphs import DecodeGraphs, MixedGraphs
+            on_gpu = self.device.type == "cuda"
+            self.graphs = DecodeGraphs(self, max_bucket=max_decode_rows, capture=on_gpu)
+            if mixed_graphs_after is not None:
+                self.mixed_graphs = MixedGraphs(self, max_rows=max_decode_rows, capture=on_gpu, capture_after=mixed_graphs_after)
         self._host = [None, None]
         self._events = [None, None]
         self._dev = None
@@ -172,101 +182,59 @@ class ModelRunner:
                          names=[entries[i].req for i in order])
 
     def _run(self, token_lists: list, starts: list, tables: list, slots_of: list, rows: list, names: list | None = None):
-        """One eager pass. Requests in step order (single tokens first): their tokens, first positions,
-        per group their block tables, their state slots; `rows`: token rows that want logits."""
-        ps = self.manager.page_size
-        B = len(token_lists)
+        """One pass. Requests in step order (single tokens first): their tokens, first positions, per group
+        their block tables, their state slots; `rows`: token rows that want logits. Steps whose padded shape
+        has come up before are replayed as graphs (`MixedGraphs`); the others run eagerly, exactly sized."""
         q_lens = [len(t) for t in token_lists]
-        Dn = sum(1 for q in q_lens if q == 1)
-        T = sum(q_lens)
-        cu = np.zeros(B + 1, dtype=np.int64)
-        np.cumsum(q_lens, out=cu[1:])
-        G = len(tables)
-        MB = [max(1, max(len(t) for t in tables[g])) for g in range(G)]
-        R = len(rows)
-
-        # ---- one packed int32 array: offsets (each segment padded to 16 bytes)
-        seg, n = {}, 0
-        for name, size in (("tokens", T), ("positions", T), ("seq_of_token", T), ("context_lens", B),
-                           ("cu", B + 1), ("prefill_cu", B - Dn + 1), ("state_slots", B), ("first_chunk", B),
-                           ("rows", max(R, 1))):
-            seg[name] = (n, size)
-            n += _pad4(size)
-        for g in range(G):
-            seg[f"slots{g}"] = (n, T); n += _pad4(T)
-            seg[f"bt{g}"] = (n, B * MB[g]); n += _pad4(B * MB[g])
+        layout = exact_layout(q_lens, starts, tables, len(rows), ops.decode_contexts_even)
+        if self.mixed_graphs is not None:
+            captured = self.mixed_graphs.lookup(layout)
+            if captured is not None:
+                return self.mixed_graphs.run(captured, token_lists, starts, tables, slots_of, rows, names)
+        n = layout.segments()[1]
         buf_i, host = self._staging(n)
-        a = host.numpy()[:n]
-
-        def put(name, values):
-            o, size = seg[name]
-            a[o:o + size] = values
-
-        tok = np.concatenate([np.asarray(t, dtype=np.int64) for t in token_lists])
-        if self.vocab_size is not None and (tok.min() < 0 or tok.max() >= self.vocab_size):
-            raise ValueError(f"token id outside 0..{self.vocab_size - 1}")
-        pos = np.concatenate([np.arange(s, s + q, dtype=np.int64) for s, q in zip(starts, q_lens)])
-        put("tokens", tok)
-        put("positions", pos)
-        put("seq_of_token", np.repeat(np.arange(B), q_lens))
-        put("context_lens", [s + q for s, q in zip(starts, q_lens)])
-        put("cu", cu)
-        put("prefill_cu", cu[Dn:] - cu[Dn])
-        put("state_slots", slots_of)
-        put("first_chunk", [1 if s == 0 else 0 for s in starts])
-        if R:
-            put("rows", rows)
-        for g in range(G):
-            bt = np.full((B, MB[g]), -1, dtype=np.int64)
-            slot = np.empty(T, dtype=np.int64)
-            for j in range(B):
-                t = tables[g][j]
-                bt[j, :len(t)] = t
-                p = pos[cu[j]:cu[j + 1]]
-                pages = bt[j, p // ps] if p[-1] // ps < MB[g] else np.array([-1])
-                if (pages < 0).any():
-                    who = names[j] if names is not None else j
-                    raise RuntimeError(f"request {who!r} has no page for a position it is "
-                                       f"about to write (group {g}); allocate before stepping")
-                slot[cu[j]:cu[j + 1]] = pages * ps + p % ps
-            put(f"slots{g}", slot)
-            put(f"bt{g}", bt.reshape(-1))
-
+        pack_step(layout, host.numpy()[:n], token_lists, starts, tables, slots_of, rows, self.manager.page_size,
+                  [self.pool.spare_page(g) for g in range(len(tables))], self.pool.spare_state_slot, self.vocab_size, names)
         dev = self._dev[:n]
         dev.copy_(host[:n], non_blocking=True)
         if self.device.type == "cuda":
             ev = torch.cuda.Event()
             ev.record()
             self._events[buf_i] = ev
-
-        def view(name):
-            o, size = seg[name]
-            return dev[o:o + size]
-
-        decode_ctx = [s + 1 for s, q in zip(starts, q_lens) if q == 1]
-        ctx = StepContext(
-            num_tokens=T, num_seqs=B, num_decodes=Dn, positions=view("positions"),
-            seq_of_token=view("seq_of_token"), context_lens=view("context_lens"), cu_seqlens=view("cu"),
-            prefill_cu=view("prefill_cu") if Dn < B else None,
-            max_decode_context=max(decode_ctx, default=0),
-            decode_contexts_even=bool(decode_ctx) and ops.decode_contexts_even(len(decode_ctx), min(decode_ctx), max(decode_ctx)),
-            max_prefill_context=max((s + q for s, q in zip(starts, q_lens) if q != 1), default=0),
-            groups=[GroupStep(view(f"bt{g}").view(B, MB[g]), view(f"slots{g}")) for g in range(G)],
-            state_slots=view("state_slots"), first_chunk=view("first_chunk"), q_lens=q_lens, starts=starts)
-
-        # a request whose tokens start at position 0 starts from empty state
-        if self.pool.has_state:
-            fresh = [s for s, st in zip(slots_of, starts) if st == 0 and s >= 0]
-            if fresh:
-                idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
-                for st in self.pool.states:
-                    if st is not None:
-                        st.index_fill_(0, idx, 0)
-
-        h, residual = self.model.forward(view("tokens"), ctx, self.pool.views, self.pool.states)
-        if not R:
+        self.zero_fresh_state(slots_of, starts)
+        tokens, row_view = views_of(layout, dev)
+        h, residual = self.model.forward(tokens, context_of(layout, dev, q_lens, starts), self.pool.views, self.pool.states)
+        if not rows:
             return None
-        return self.model.logits(h, residual, view("rows")[:R])
+        return self.model.logits(h, residual, row_view[:len(rows)])
+
+    def zero_fresh_state(self, slots_of: list, starts: list) -> None:
+        """A request whose tokens start at position 0 starts from empty state."""
+        if not self.pool.has_state:
+            return
+        fresh = [s for s, st in zip(slots_of, starts) if st == 0 and s >= 0]
+        if fresh:
+            idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
+            for st in self.pool.states:
+                if st is not None:
+                    st.index_fill_(0, idx, 0)
+
+    # -- what the captured graphs share ----------------------------------------------------
+    def graph_pool(self):
+        """One memory pool for all captured graphs: they replay one after the other on one stream, so a graph
+        may reuse what the others' activations occupy."""
+        if self._graph_pool is None and self.device.type == "cuda":
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        return self._graph_pool
+
+    def graph_logits(self) -> torch.Tensor:
+        """The one buffer every captured graph writes its logits to ([rows a step can want, vocabulary]); what a
+        step returns is a view of it, valid until the next step."""
+        if self._graph_logits is None:
+            from .graphs import bucket_of
+            self._graph_logits = torch.empty((bucket_of(self.max_decode_rows), self.vocab_size), dtype=torch.float32,
+                                             device=self.device)
+        return self._graph_logits
 
     # -- sizing by measurement -------------------------------------------------------------
     @torch.inference_mode()

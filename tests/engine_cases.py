@@ -174,3 +174,24 @@ def wanted_rows_only(env, name):
 
 ALL = [whole, tail_one_by_one, changing_portions, mixed_with_reuse, long_decode, batch_of_decodes, first_tokens,
        wanted_rows_only]
+
+
+def padded_layouts_are_used(env, name, captured: bool):
+    """With `mixed_graphs_after=0` every step with a prompt portion goes through a padded layout (replayed
+    from a graph where there is a GPU), single tokens alone through the decode layouts; logits as ever."""
+    runner, manager, folder = env.runner(name, 40)
+    assert runner.mixed_graphs is not None and runner.mixed_graphs.capture_after == 0
+    V = _vocab(name)
+    a, b = helpers.random_ids(70, V, 801), helpers.random_ids(45, V, 802)
+    d = helpers.Driver(runner, manager)
+    d.step({"a": a[:33]})
+    d.step({"a": a[33:34], "b": b[:20]})
+    d.step({"a": a[34:35], "b": b[20:40]})               # the same padded layout as the step before
+    d.step({"a": a[35:36], "b": b[40:41]})               # two single tokens: the decode layouts
+    d.step({"a": a[36:70], "b": b[41:45]})
+    assert runner.mixed_graphs.replays == 4 and runner.graphs.replays == 1
+    assert len(runner.mixed_graphs.captured) == 3
+    if captured:
+        assert all(c.graph is not None for c in runner.mixed_graphs.captured.values())
+    _check(env, folder, a, d.result("a"), "a through padded layouts")
+    _check(env, folder, b, d.result("b"), "b through padded layouts")

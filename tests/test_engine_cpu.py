@@ -18,9 +18,10 @@ from mini_engine_amd.weights.loader import load_model
 class Env:
     device, dtype, tol = "cpu", torch.float32, helpers.TOL_F32
 
-    def __init__(self, folders):
+    def __init__(self, folders, graphs=False):
         self.folders = folders
         self.models = {}
+        self.graphs = graphs           # every step through the fixed layouts (padded; captured where there is a GPU)
 
     def runner(self, name, pages):
         folder = self.folders(name)
@@ -28,12 +29,27 @@ class Env:
             self.models[name] = load_model(folder, self.device, self.dtype, 512)
         model = self.models[name]
         manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
-        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True), manager, folder
+        options = dict(use_graphs=True, mixed_graphs_after=0) if self.graphs else {}
+        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True, **options), manager, folder
 
 
 @pytest.fixture(scope="module")
 def env(folders):
     return Env(folders)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("case", [c for c in engine_cases.ALL if c.__name__ not in ("long_decode",)], ids=lambda c: c.__name__)
+def test_cuts_through_padded_layouts(folders, plain_backend, case, name):
+    """The same cuts with every step rounded up to a shared layout: padding rows among the single tokens, a
+    padding request behind the prompt portions, wider block tables, more rows of logits than wanted."""
+    env = Env(folders, graphs=True)
+    case(env, name)
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_padded_layouts_are_used(folders, plain_backend, name):
+    engine_cases.padded_layouts_are_used(Env(folders, graphs=True), name, captured=False)
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])

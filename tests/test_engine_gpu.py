@@ -16,8 +16,9 @@ pytestmark = pytest.mark.gpu
 class Env:
     device = "cuda"
 
-    def __init__(self, folders, dtype):
+    def __init__(self, folders, dtype, graphs=False):
         self.folders, self.dtype = folders, dtype
+        self.graphs = graphs           # every step through a captured graph of its padded layout
         self.tol = helpers.TOL_F32 if dtype == torch.float32 else helpers.TOL_BF16
         self.models = {}
 
@@ -27,7 +28,8 @@ class Env:
             self.models[name] = load_model(folder, self.device, self.dtype, 512)
         model = self.models[name]
         manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
-        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True), manager, folder
+        options = dict(use_graphs=True, mixed_graphs_after=0) if self.graphs else {}
+        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True, **options), manager, folder
 
 
 @pytest.fixture(scope="module", params=[torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -39,6 +41,24 @@ def env(request, folders):
 @pytest.mark.parametrize("case", engine_cases.ALL, ids=lambda c: c.__name__)
 def test_cuts(env, case, name):
     case(env, name)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("case", [engine_cases.whole, engine_cases.tail_one_by_one, engine_cases.changing_portions,
+                                  engine_cases.mixed_with_reuse, engine_cases.wanted_rows_only], ids=lambda c: c.__name__)
+def test_cuts_through_captured_steps(env, case, name):
+    """The cuts again with every step, prompt portions and mixed ones too, replayed from a captured graph of its
+    padded layout (padding rows, a padding request, wider tables, spare logits rows)."""
+    graphs = Env(env.folders, env.dtype, graphs=True)
+    graphs.models = env.models
+    case(graphs, name)
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_padded_layouts_are_captured_and_replayed(env, name):
+    graphs = Env(env.folders, env.dtype, graphs=True)
+    graphs.models = env.models
+    engine_cases.padded_layouts_are_used(graphs, name, captured=True)
 
 
 def test_hip_libraries_are_the_ones_running(env):
