@@ -128,7 +128,7 @@ class ModelRunner:
         return i, self._host[i]
 
     # -- the step --------------------------------------------------------------------------
-    @torch.inference_mode()
+    @torch.no_grad()      # not inference_mode: tensors made there cannot be used by a graph capture outside it, ours or the caller's
     def step(self, entries: list) -> torch.Tensor | None:
         """Run the given tokens as one batch. Returns float32 logits [R, vocab] for the wanted
         places, in the order of `entries` and of each entry's `want`; None if nothing is wanted.
@@ -237,7 +237,7 @@ class ModelRunner:
         return self._graph_logits
 
     # -- sizing by measurement -------------------------------------------------------------
-    @torch.inference_mode()
+    @torch.no_grad()
     def measure_working_set(self, max_step_tokens: int, max_seqs: int, max_len: int) -> tuple:
         """(bytes the largest step needs beyond what is allocated now, the same for the largest decode step).
 
@@ -272,12 +272,12 @@ class ModelRunner:
         return max(prompt_peak, decode_peak), decode_peak
 
     # -- sampling --------------------------------------------------------------------------
-    @torch.inference_mode()
+    @torch.no_grad()
     def sample(self, logits: torch.Tensor, temperatures: list, keys: list) -> list:
         """Token ids for float32 logits [S, V]; keys: (k0, k1) 32-bit pairs per row."""
         return self.sample_async(logits, temperatures, keys).tokens()
 
-    @torch.inference_mode()
+    @torch.no_grad()
     def sample_async(self, logits: torch.Tensor, temperatures: list, keys: list, reqs: list | None = None) -> SampledTokens:
         """The same without waiting for the result. `reqs` names the request of every row: the next
         step may then give PENDING as the token of any of them."""

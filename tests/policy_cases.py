@@ -54,7 +54,10 @@ def long_prefill_threshold(make, folders, exact):
         sizes.append(out[1])
         return out
     llm.step = counting
-    outs = llm.generate(prompts, _greedy(9), use_tqdm=False)
+    try:
+        outs = llm.generate(prompts, _greedy(9), use_tqdm=False)
+    finally:
+        del llm.step                    # the wrapper refers to the engine: no reference cycle is left behind
     assert max(sizes) <= 4 * 5 and any(0 < s <= 5 for s in sizes), sizes       # no request ran more than 5 prompt tokens a step
     helpers.assert_greedy_like_plain(folder, prompts, [o["token_ids"] for o in outs], exact, "threshold")
 
