@@ -337,15 +337,32 @@ def _round_up(n: int, to: int) -> int:
     return -(-n // to) * to
 
 
-def token_bucket(tokens: int) -> int:
-    """Tokens of the padded layout that holds `tokens` prompt tokens and at least one of padding: steps of 32
-    up to 512 tokens, of 64 up to 4,096, of 256 beyond (at most a sixteenth more work than the step has)."""
-    need = tokens + 1
-    if need <= 512:
-        return _round_up(need, 32)
-    if need <= 4096:
-        return _round_up(need, 64)
-    return _round_up(need, 256)
+def _pow2_at_least(n: int) -> int:
+    return 1 << max(0, n - 1).bit_length()
+
+
+# What launching a layer's kernels from Python costs the host, and the rate at which small steps run on the GPU:
+# from them follows up to how many tokens a step is bound by the host rather than by the GPU. Measured at
+# Qwen3-0.6B sizes (28 layers): an eager step costs the host 3.6-4.4 ms whatever its size; replayed, a prompt of
+# 128 tokens takes 2.4 ms and one of 512 tokens 3.2 ms (the GPU's own time: products of so few rows run far below
+# the rate of large ones), and a step of 504 prompt tokens beside 8 requests with long contexts 4.1 ms, which is
+# what it takes eagerly. A capture costs 12-14 ms, so layouts that do not pay must not be captured at all.
+HOST_US_PER_LAYER = 130.0
+SMALL_STEP_FLOPS = 1.0e14
+
+
+def host_bound_tokens(model) -> int:
+    """Up to how many tokens a step of this model is worth replaying from a graph: below, the host's launches
+    take longer than the GPU's work; above, the eager step keeps the GPU busy anyway and padding only costs."""
+    per_token = 0
+    for name, _, _, spec in model.named_specs():
+        if len(spec.shape) == 2 and not name.startswith(("embedding.", "head.")):
+            per_token += 2 * spec.shape[0] * spec.shape[1]
+    per_token *= max(1, len(model.order)) / max(1, len(model.layers))
+    if per_token <= 0:
+        return 2048
+    tokens = HOST_US_PER_LAYER * 1e-6 * len(model.order) / (per_token / SMALL_STEP_FLOPS)
+    return int(min(2048, max(64, tokens)))
 
 
 class _CapturedStep:
@@ -369,21 +386,27 @@ class _CapturedStep:
 
 
 class MixedGraphs:
-    """Steps with prompt portions, padded to a layout shared by many steps and replayed as a graph.
+    """Small steps with prompt portions, padded to a layout shared by many steps and replayed as a graph.
 
-    Launched kernel by kernel from Python, such a step costs the host a few milliseconds whatever its size,
-    which for small models and short portions is more than the GPU needs. A step's shape is rounded up to a
-    layout (single-token rows to a bucket, prompt tokens to a bucket through one padding request, block-table
-    columns, context caps, rows that want logits); a layout that has come up `capture_after` times is captured
-    on its next appearance and replayed from then on. Layouts that come up once (the ramp of a workload) stay
-    eager, exactly sized. The captured work is the model's own forward pass over the padded step."""
+    Launched kernel by kernel from Python, a step costs the host a few milliseconds whatever its size, which
+    for small models and short portions is more than the GPU needs. Such a step (up to `max_tokens` tokens: see
+    host_bound_tokens) is rounded up to a layout: single-token rows to a bucket, all tokens to a power of two
+    (beyond 256 to a multiple of 64, beyond 1,024 of 128: a step that fills a token budget must not grow by half)
+    through one padding request, one power-of-two cap for every context and block table, rows that want logits
+    to a bucket. The rounding is coarse on purpose: a capture costs about three eager steps, so layouts must be
+    few, and a step that the host bounds loses nothing by the padding. A layout that has come up
+    `capture_after` times is captured on its next appearance and replayed from then on; larger steps, and
+    layouts that come up once, stay eager and exactly sized. The captured work is the model's own forward pass
+    over the padded step."""
 
-    def __init__(self, runner, max_rows: int, capture: bool = True, capture_after: int = 2, max_graphs: int = 48):
+    def __init__(self, runner, max_rows: int, capture: bool = True, capture_after: int = 4, max_graphs: int = 48,
+                 max_tokens: int | None = None):
         self.runner = weakref.proxy(runner)
         self.max_rows = max_rows
         self.capture = capture
         self.capture_after = capture_after
         self.max_graphs = max_graphs
+        self.max_tokens = host_bound_tokens(runner.model) if max_tokens is None else max_tokens
         self.captured: dict = {}
         self.sightings: dict = {}
         self.pool = runner.graph_pool() if capture else None
@@ -391,17 +414,22 @@ class MixedGraphs:
 
     def padded(self, exact: StepLayout) -> StepLayout | None:
         r = self.runner
-        if (exact.prefill_reqs == 0 or exact.rows > self.max_rows or r.vocab_size is None
+        tokens = exact.decode_rows + exact.prefill_tokens
+        if (exact.prefill_reqs == 0 or exact.rows > self.max_rows or tokens >= self.max_tokens or r.vocab_size is None
                 or not (r.device.type == "cuda" or not self.capture)):
             return None
+        decode_rows = bucket_of(exact.decode_rows) if exact.decode_rows else 0
+        need = decode_rows + exact.prefill_tokens + 1
+        total = max(32, _pow2_at_least(need)) if need <= 256 else _round_up(need, 64 if need <= 1024 else 128)
+        pad = total - decode_rows - exact.prefill_tokens
         most_ctx = -(-r.max_positions // 8) * 8
+        cap = min(max(1024, _pow2_at_least(max(exact.decode_ctx, exact.prefill_ctx, pad))), most_ctx)
+        ps = r.manager.page_size
         return StepLayout(
-            decode_rows=bucket_of(exact.decode_rows) if exact.decode_rows else 0,
-            prefill_reqs=exact.prefill_reqs + 1, prefill_tokens=token_bucket(exact.prefill_tokens),
+            decode_rows=decode_rows, prefill_reqs=exact.prefill_reqs + 1, prefill_tokens=total - decode_rows,
             rows=bucket_of(exact.rows) if exact.rows else 0,
-            max_blocks=tuple(_round_up(mb, 64) for mb in exact.max_blocks),
-            decode_ctx=min(_round_up(exact.decode_ctx, CONTEXT_STEP), most_ctx) if exact.decode_rows else 0,
-            prefill_ctx=_round_up(exact.prefill_ctx, CONTEXT_STEP), even=exact.even)
+            max_blocks=tuple(max(mb, -(-cap // ps)) for mb in exact.max_blocks),
+            decode_ctx=cap if exact.decode_rows else 0, prefill_ctx=cap, even=exact.even)
 
     def lookup(self, exact: StepLayout):
         """The captured (or about to be captured) layout that takes this step, or None: run it eagerly."""

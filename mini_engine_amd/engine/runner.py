@@ -62,9 +62,10 @@ def _pad4(n: int) -> int:
 class ModelRunner:
     def __init__(self, model, manager: CacheManager, dtype: torch.dtype, device, max_positions: int,
                  poison_cache: bool = False, use_graphs: bool = False, max_decode_rows: int = 256,
-                 mixed_graphs_after: int | None = 2):
-        """use_graphs: decode steps are replayed as HIP graphs, and so are steps with prompt portions whose
-        padded shape has come up more than `mixed_graphs_after` times (None: those always run eagerly)."""
+                 mixed_graphs_after: int | None = 4, mixed_graphs_max_tokens: int | None = None):
+        """use_graphs: decode steps are replayed as HIP graphs, and so are small steps with prompt portions
+        whose padded shape has come up more than `mixed_graphs_after` times (None: those always run eagerly);
+        `mixed_graphs_max_tokens`: up to how many tokens a step counts as small (None: by the model's size)."""
         self.model = model
         self.manager = manager
         self.dtype = dtype
@@ -89,7 +90,8 @@ class ModelRunner:
             on_gpu = self.device.type == "cuda"
             self.graphs = DecodeGraphs(self, max_bucket=max_decode_rows, capture=on_gpu)
             if mixed_graphs_after is not None:
-                self.mixed_graphs = MixedGraphs(self, max_rows=max_decode_rows, capture=on_gpu, capture_after=mixed_graphs_after)
+                self.mixed_graphs = MixedGraphs(self, max_rows=max_decode_rows, capture=on_gpu, capture_after=mixed_graphs_after,
+                                                max_tokens=mixed_graphs_max_tokens)
         self._host = [None, None]
         self._events = [None, None]
         self._dev = None

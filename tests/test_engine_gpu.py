@@ -28,7 +28,7 @@ class Env:
             self.models[name] = load_model(folder, self.device, self.dtype, 512)
         model = self.models[name]
         manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
-        options = dict(use_graphs=True, mixed_graphs_after=0) if self.graphs else {}
+        options = dict(use_graphs=True, mixed_graphs_after=0, mixed_graphs_max_tokens=4096) if self.graphs else {}
         return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True, **options), manager, folder
 
 
