@@ -85,7 +85,7 @@ class ModelRunner:
         self._graph_logits = None
         self.graphs = None              # plain decode steps
         self.mixed_graphs = None        # steps with prompt portions
-        if use_graphs:
+        if use_graphs and all(part.capturable for part in model.parts()):
             from .graphs import DecodeGraphs, MixedGraphs
             on_gpu = self.device.type == "cuda"
             self.graphs = DecodeGraphs(self, max_bucket=max_decode_rows, capture=on_gpu)

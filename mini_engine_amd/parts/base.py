@@ -89,6 +89,11 @@ class StateNeed:
 class Part:
     """Base of all parts: named parameters and named child parts."""
 
+    # Whether a step that contains this part may be captured as a graph: its forward must then use device
+    # operations only (no value may travel to the host: no .tolist(), .item(), nonzero(), ...). A part that
+    # needs the host sets this to False; the model's steps then always run eagerly.
+    capturable = True
+
     def __init__(self):
         self._specs: dict[str, ParamSpec] = {}
         self._children: dict[str, "Part"] = {}

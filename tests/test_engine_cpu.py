@@ -344,3 +344,18 @@ import policy_cases
 @pytest.mark.parametrize("case", policy_cases.ALL, ids=lambda c: c.__name__)
 def test_policies_with_a_model_on_cpu(folders, plain_backend, case):
     case(_llm, folders, exact=True)
+
+
+def test_a_part_that_needs_the_host_keeps_its_model_out_of_the_graphs(plain_backend, monkeypatch):
+    """A part may declare that its forward reads values on the host (`capturable = False`): a model that
+    contains it is never captured, whatever the engine was asked for."""
+    import toy_arch
+    from mini_engine_amd.registry import build_model
+    from mini_engine_amd.weights.random_init import fill_random
+    model = fill_random(build_model(toy_arch.ToyConfig.from_dict({"vocab_size": 50, "hidden_size": 40, "eps": 1e-5})),
+                        4, "cpu", torch.float32, 64)
+    manager = lambda: CacheManager(8, 8, ModelRunner.windows_of(model), num_state_slots=2)
+    assert ModelRunner(model, manager(), torch.float32, "cpu", 64, use_graphs=True).graphs is not None
+    monkeypatch.setattr(toy_arch.RunningMean, "capturable", False)
+    runner = ModelRunner(model, manager(), torch.float32, "cpu", 64, use_graphs=True)
+    assert runner.graphs is None and runner.mixed_graphs is None
