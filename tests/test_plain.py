@@ -187,3 +187,57 @@ def test_sampler_formula():
     e = torch.empty(50, dtype=D64).exponential_(1.0)
     assert P.sample_gumbel_reference(z, 0.7, e) == int(torch.argmax(z / 0.7 - torch.log(e)))
     assert P.sample_gumbel_reference(z, 0.0, e) == int(torch.argmax(z))
+
+
+def test_q_and_k_pass_a_norm_and_v_does_not(tmp_path):
+    """reference models/qwen3.py:34-35 norms q and k per head and leaves v alone. What that means, whatever the
+    code looks like: the block's output does not change when q_proj or k_proj is scaled (an RMS norm forgets
+    the scale of its input, up to eps) and is linear in v_proj (the output is a weighted sum of raw values)."""
+    d = _folder(tmp_path, "B")
+    cfg, w = P.read_model_folder(d, D64)
+    p = "model.layers.1.self_attn."
+    T = 13
+    x = torch.randn(T, cfg["hidden_size"], dtype=D64, generator=torch.Generator().manual_seed(2))
+    cos, sin = P.rope_tables(cfg["head_dim"], T, cfg["rope_theta"], D64)
+    run = lambda weights: P.attention_block(cfg, weights, p, x, torch.arange(T), cos, sin, None)
+    base = run(w)
+    for name in ("q_proj.weight", "k_proj.weight"):
+        scaled = run({**w, p + name: w[p + name] * 7.0})
+        assert float((scaled - base).abs().max()) <= 1e-3 * float(base.abs().max()), name   # eps keeps it from being exact
+    assert torch.allclose(run({**w, p + "v_proj.weight": w[p + "v_proj.weight"] * 7.0}), base * 7.0, rtol=1e-12)
+    assert not torch.allclose(run({**w, p + "v_proj.weight": w[p + "v_proj.weight"] * 7.0}), base, rtol=1e-2)
+
+
+def test_gate_goes_through_silu_and_up_does_not(tmp_path):
+    """reference layers/activation.py:6-7: silu(first half) * second half, the first half being gate_proj's rows
+    (layers/linear.py:29-45). So the feed-forward is linear in up_proj and not in gate_proj."""
+    d = _folder(tmp_path, "B")
+    cfg, w = P.read_model_folder(d, D64)
+    p = "model.layers.0.mlp."
+    x = torch.randn(9, cfg["hidden_size"], dtype=D64, generator=torch.Generator().manual_seed(3)) * 4
+    base = P.mlp_block(w, p, x)
+    assert torch.allclose(P.mlp_block({**w, p + "up_proj.weight": w[p + "up_proj.weight"] * 3.0}, p, x), base * 3.0, rtol=1e-12)
+    gate3 = P.mlp_block({**w, p + "gate_proj.weight": w[p + "gate_proj.weight"] * 3.0}, p, x)
+    assert not torch.allclose(gate3, base * 3.0, rtol=1e-2)
+    # silu(z) -> z for large z: where every gate value is large and positive the block becomes gate * up
+    big = {**w, p + "gate_proj.weight": torch.zeros_like(w[p + "gate_proj.weight"])}
+    assert torch.equal(P.mlp_block(big, p, x), torch.zeros_like(base))            # silu(0) = 0, whatever up is
+
+
+def test_layers_that_output_nothing_leave_the_norm_of_the_embedding(tmp_path):
+    """reference models/qwen3.py:65-74,91: every layer adds its attention and feed-forward outputs to the
+    residual stream, which starts as the embedding, and the final norm takes the last output plus the stream.
+    With every o_proj and down_proj zero the logits are therefore head(rms_norm(embedding)): library routines
+    only. (A final norm over the last layer's output alone would give zeros; a stream that did not start at the
+    embedding would give something else.)"""
+    d = _folder(tmp_path, "B")
+    cfg, w = P.read_model_folder(d, D64)
+    silent = {k: (torch.zeros_like(v) if k.endswith(("o_proj.weight", "down_proj.weight")) else v) for k, v in w.items()}
+    ids = helpers.random_ids(17, cfg["vocab_size"], 8)
+    h = F.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    want = F.linear(F.rms_norm(h, (h.shape[-1],), w["model.norm.weight"], cfg["rms_norm_eps"]), w["lm_head.weight"])
+    assert torch.allclose(P.logits(cfg, silent, ids), want, atol=1e-12)
+    # and with only the last feed-forward speaking, its output reaches the logits through the same norm
+    last = f"model.layers.{cfg['num_hidden_layers'] - 1}.mlp.down_proj.weight"
+    speaking = {**silent, last: w[last]}
+    assert not torch.allclose(P.logits(cfg, speaking, ids), want, atol=1e-6)
