@@ -63,7 +63,7 @@ class Bench:
     """An engine built by `LLM(folder)` and the workloads run on it."""
 
     def __init__(self, cfg, folder: str, dtype: str, page: int, max_seqs: int, max_len: int, budget: int, seed: int,
-                 graphs: bool, run_ahead: bool, random_weights: int | None):
+                 graphs: bool, run_ahead: bool, random_weights: int | None, kv_blocks: int = -1):
         import torch
         from mini_engine_amd import LLM
 
@@ -71,7 +71,7 @@ class Bench:
         t0 = time.time()
         self.llm = LLM(folder, dtype=dtype, kvcache_block_size=page, max_num_seqs=max_seqs, max_model_len=max_len,
                        max_num_batched_tokens=budget, seed=seed, use_graphs=graphs, run_ahead=run_ahead,
-                       random_weights=random_weights, eos=-1)
+                       random_weights=random_weights, eos=-1, num_kvcache_blocks=kv_blocks)
         log(f"engine ready in {time.time() - t0:.1f}s: {self.llm.config.num_kvcache_blocks} pages of {page} tokens, "
             f"{self.llm.reserved_bytes >> 20} MiB kept free for the steps' working set")
         self.ids = torch.Generator().manual_seed(seed)
@@ -200,7 +200,7 @@ def measure(args, size: str, layers, tmp: str, points: list, steps: int, warmup:
     max_seqs = max(batches + ([256] if serve and (args.offline or args.mixed_lengths) else []))
     budget = max(args.prefill_tokens, 2048 if (serve and args.mixed_lengths) else 16384, max_seqs)
     bench = Bench(cfg, folder, args.dtype, args.page, max_seqs, max_len, budget, args.seed, not args.no_graphs,
-                  not args.no_run_ahead, random_weights)
+                  not args.no_run_ahead, random_weights, args.kv_blocks)
     item = 2 if args.dtype == "bfloat16" else 4
     out = {"cfg": cfg, "full_layers": full_layers, "weights": "drawn on the device" if on_device else "written folder"}
 
@@ -256,6 +256,8 @@ def main(argv=None) -> int:
                     help="also run the reference's offline workload with this many requests (0: skip)")
     ap.add_argument("--mixed-lengths", type=int, default=0,
                     help="also run this many requests with nine short prompts to one long under a 2,048 budget (0: skip)")
+    ap.add_argument("--kv-blocks", type=int, default=-1,
+                    help="pages of the cache pool (-1: sized by the engine from a measured warm-up, as a user's engine is)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="fetch every decode step's tokens before the next step is launched")
