@@ -69,6 +69,17 @@ struct AttnArgs {
   float* pf_scratch;            // [tokens, Hq, max_segs, HD + 2]: unnormalised output, max (log2 domain), sum
   const int32_t* seq_of_token;  // prefill: [tokens] index of the token's sequence among the prefill sequences + seq_base
   int seq_base;
+  // decode with the step's prologue inside (attn_decode_kernel<true>): q and the new token's key and value are
+  // taken as the packed projection left them; the kernel norms and rotates q and the key itself, attends to the
+  // new key and value from LDS, and writes them to their place in the pages
+  const bf16_t* raw_k;          // token 0's first key head in the packed row (token stride q_stride)
+  const bf16_t* raw_v;
+  const float* q_w;             // per-head RMSNorm weights [HD], or both nullptr: no norm
+  const float* k_w;
+  float eps;
+  const float* rope;            // [positions, HD/2, 2] (cos, sin), or nullptr: no rotation
+  bf16_t* k_cache_w;
+  bf16_t* v_cache_w;
 };
 
 // Key range of the tile that holds new token `tl` (index within its sequence's new tokens) and the
@@ -913,8 +924,16 @@ __device__ __forceinline__ void decode_part_range(const AttnArgs& a, int L, int&
   end = max(first + 1, min(a.num_parts, (L + a.part_size - 1) / a.part_size));
 }
 
+// PROLOGUE: what precedes attention in a decode step happens here too (reference models/qwen3.py:34-36 the
+// per-head norms, layers/rotary_embedding.py:20-25 the rotation, csrc/kv_cache.cu:10-31 the cache write). The
+// new token sits at position L - 1. Every workgroup norms and rotates its own query heads (a wave per head, a
+// lane per rotation pair) into LDS, rounded to bfloat16 as the stand-alone kernel leaves them in the row. The
+// workgroups whose partition holds position L - 1 do the same for the new key and copy the new value: they
+// attend to both from LDS, in place of what the page holds there, and the first column tile's workgroup writes
+// them into the page. No workgroup reads what another one writes.
+template <bool PROLOGUE>
 __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
-  extern __shared__ float lds[];  // [4 waves][cols][HD + 2]
+  extern __shared__ float lds[];  // [4 waves][cols][HD + 2]; PROLOGUE: then bfloat16 [cols + 2][HD]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int b = a.spread_heads ? blockIdx.y : blockIdx.x;
@@ -942,18 +961,125 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
   f32x4 acc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int cmax = a.G < 16 ? a.G : 16;
+  bf16_t* q_s = reinterpret_cast<bf16_t*>(lds + 4 * cmax * (HD + 2));   // [cols][HD]
+  bf16_t* k_s = q_s + cmax * HD;                                        // [HD] the new key
+  bf16_t* v_s = k_s + HD;                                               // [HD] the new value
+  const bool holds_new = PROLOGUE && pos >= p_lo && pos < p_hi;
+  constexpr int HALF = HD / 2, PPL = (HALF + 63) / 64;   // rotation pairs of a head, pairs per lane
+  struct RawHead { float x1[PPL], x2[PPL], w1[PPL], w2[PPL], cs[PPL], sn[PPL]; };
+  const int nheads = PROLOGUE ? ncols + (holds_new ? 1 : 0) : 0;
+  const int pi = pos >> a.page_shift;
+  const int new_page = holds_new ? bt[pi] : -1;
+  const int new_off = pos - (pi << a.page_shift);
+  // a head's values, norm weights and angles as they lie in memory: only asked for here
+  auto fetch_head = [&](int h, RawHead& r) {
+    const bool is_q = h < ncols;
+    const bf16_t* src = is_q ? a.q + t * a.q_stride + (int64_t)(kvh * a.G + ctile * 16 + h) * HD
+                             : a.raw_k + t * a.q_stride + (int64_t)kvh * HD;
+    const float* w = is_q ? a.q_w : a.k_w;
+#pragma unroll
+    for (int i = 0; i < PPL; ++i) {
+      const int j = lane + 64 * i;
+      const int js = j < HALF ? j : 0;
+      r.x1[i] = static_cast<float>(src[js]);
+      r.x2[i] = static_cast<float>(src[HALF + js]);
+      r.w1[i] = w ? w[js] : 1.f;
+      r.w2[i] = w ? w[HALF + js] : 1.f;
+      // a padding row has no token (L = 0): it reads the angles of position 0 and nothing comes of them
+      const float2 c = a.rope ? *reinterpret_cast<const float2*>(a.rope + ((int64_t)(pos > 0 ? pos : 0) * HALF + js) * 2) : make_float2(1.f, 0.f);
+      r.cs[i] = c.x; r.sn[i] = c.y;
+    }
+  };
+  // norm, rotation, rounding; into LDS, and the key into its page as well
+  auto finish_head = [&](int h, const RawHead& r) {
+    const bool is_q = h < ncols;
+    const bool writes = !is_q && ctile == 0 && new_page >= 0;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PPL; ++i)
+      if (lane + 64 * i < HALF) ss += r.x1[i] * r.x1[i] + r.x2[i] * r.x2[i];
+    float inv = 1.f;
+    if (a.q_w) inv = rsqrtf(wave_sum(ss) / (float)HD + a.eps);
+    bf16_t* dst = is_q ? q_s + h * HD : k_s;
+    bf16_t* page_row = a.k_cache_w + (((int64_t)(writes ? new_page : 0) * a.Hkv + kvh) * a.page + new_off) * HD;
+#pragma unroll
+    for (int i = 0; i < PPL; ++i) {
+      const int j = lane + 64 * i;
+      float o1 = r.x1[i] * inv, o2 = r.x2[i] * inv;
+      o1 *= r.w1[i]; o2 *= r.w2[i];
+      const bf16_t r1 = static_cast<bf16_t>(o1 * r.cs[i] - o2 * r.sn[i]);
+      const bf16_t r2 = static_cast<bf16_t>(o2 * r.cs[i] + o1 * r.sn[i]);
+      if (j < HALF) {
+        dst[j] = r1; dst[HALF + j] = r2;
+        if (writes) { page_row[j] = r1; page_row[HALF + j] = r2; }
+      }
+    }
+  };
   // One block buffer only: the registers saved let several workgroups share a compute unit,
   // and it is their interleaving that hides the load latency here (partitions are short).
   int t0 = p_lo + 32 * wave;
-  if (t0 < p_hi) {
-    KVBlock A;
+  const bool has_keys = t0 < p_hi;
+  KVBlock A;
+  if (PROLOGUE) {
+    // the wave's first head is asked for before the first block of keys, and worked on while those are on
+    // their way; the heads after it (more than three query heads to a key head) one by one
+    RawHead first;
+    if (wave < nheads) fetch_head(wave, first);
+    bf16_t new_v = static_cast<bf16_t>(0.f);
+    const int vd = threadIdx.x < HD ? threadIdx.x : 0;
+    if (holds_new) new_v = a.raw_v[t * a.q_stride + (int64_t)kvh * HD + vd];
+    if (has_keys) load_block(a, bt, kvh, t0, L, lo, n, g, A);
+    if (wave < nheads) finish_head(wave, first);
+    for (int h = wave + 4; h < nheads; h += 4) {
+      RawHead r;
+      fetch_head(h, r);
+      finish_head(h, r);
+    }
+    if (holds_new) {
+      const bool writes = ctile == 0 && new_page >= 0;
+      bf16_t* page_col = a.v_cache_w + (((int64_t)(writes ? new_page : 0) * a.Hkv + kvh) * HD) * a.page + new_off;
+      for (int d = threadIdx.x; d < HD; d += 256) {
+        const bf16_t v = d == vd ? new_v : a.raw_v[t * a.q_stride + (int64_t)kvh * HD + d];
+        v_s[d] = v;
+        if (writes) page_col[(int64_t)d * a.page] = v;
+      }
+    }
+    __syncthreads();
+  } else if (has_keys) {
     load_block(a, bt, kvh, t0, L, lo, n, g, A);
+  }
+  if (has_keys) {
     bf16x8 qb[KS];
-    load_q(a.q + t * a.q_stride + (int64_t)head * HD, valid, g, qb);
+    if (PROLOGUE) load_q(q_s + (valid ? n : 0) * HD, valid, g, qb);
+    else load_q(a.q + t * a.q_stride + (int64_t)head * HD, valid, g, qb);
     const int col_hi = valid ? pos : -1;
     while (true) {
       VBlock vb;
       load_v(a, A, kvh, t0, L, n, g, vb);
+      if (holds_new && pos >= t0 && pos < t0 + 32) {
+        // the block with the new token: its key row and its value column come from LDS
+        const int rel = pos - t0;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+          if (8 * (n >> 2) + 4 * tt + (n & 3) == rel) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+              const int d0 = 32 * ks + 8 * g;
+              A.k[tt][ks] = ld8(k_s + ((HD % 32 == 0 || d0 < HD) ? d0 : 0));
+            }
+            A.kok[tt] = true;
+          }
+        if ((rel >> 3) == g) {
+          const int at = rel & 7;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const bf16_t nv = v_s[16 * dt + n];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) vb.v[dt][e] = e == at ? nv : vb.v[dt][e];
+          }
+        }
+      }
       if (t0 + 32 <= L && t0 >= lo) attend_block<true>(a, A, vb, t0, qb, lo, col_hi, m, l, acc, g);
       else attend_block<false>(a, A, vb, t0, qb, lo, col_hi, m, l, acc, g);
       t0 += 128;
@@ -1069,6 +1195,8 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
   a.scale = scale; a.window = window; a.tok_tile = 1; a.part_size = 0; a.num_parts = 1; a.spread_heads = 1;
   a.tmp_out = a.tmp_m = a.tmp_l = nullptr;
   a.seg_keys = 0; a.max_segs = 1; a.pf_scratch = nullptr; a.seq_of_token = nullptr; a.seq_base = 0;
+  a.raw_k = a.raw_v = nullptr; a.q_w = a.k_w = nullptr; a.eps = 0.f; a.rope = nullptr;
+  a.k_cache_w = a.v_cache_w = nullptr;
   return 0;
 }
 
@@ -1121,6 +1249,42 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
 }
 
 // Scratch of the split decode path: num_seqs * Hq * num_parts * (HD + 2) floats (out, m, l per partition).
+static int launch_decode(AttnArgs& a, int num_seqs, int part_size, int num_parts, float* scratch, int spread_heads,
+                         bool prologue, hipStream_t stream) {
+  ME_CHECK(num_parts >= 1 && num_parts <= RED_MAX_PARTS, "attention: %d partitions outside 1..%d", num_parts, RED_MAX_PARTS);
+  ME_CHECK(num_parts == 1 || (part_size >= 32 && part_size % 32 == 0),
+           "attention: partition size %d must be a multiple of 32", part_size);
+  ME_CHECK(num_parts == 1 || scratch != nullptr, "attention: split decode needs scratch");
+  a.part_size = num_parts == 1 ? (1 << 30) : part_size;
+  a.num_parts = num_parts;
+  a.spread_heads = spread_heads ? 1 : 0;
+  if (num_parts > 1) {
+    const int64_t rows = (int64_t)num_seqs * a.Hq * num_parts;
+    a.tmp_out = scratch; a.tmp_m = scratch + rows * HD; a.tmp_l = a.tmp_m + rows;
+  }
+  const int col_tiles = (a.G + 15) / 16;
+  ME_CHECK((int64_t)a.Hkv * col_tiles <= 65535 && num_seqs <= 65535,
+           "attention: %d sequences or %d head blocks exceed one launch", num_seqs, a.Hkv * col_tiles);
+  const int cmax = a.G < 16 ? a.G : 16;
+  const size_t lds = (size_t)4 * cmax * (HD + 2) * sizeof(float) + (prologue ? (size_t)(cmax + 2) * HD * sizeof(bf16_t) : 0);
+  static size_t lds_allowed[2] = {64 * 1024, 64 * 1024};
+  if (lds > lds_allowed[prologue]) {
+    hipError_t e = hipFuncSetAttribute(prologue ? (const void*)attn_decode_kernel<true> : (const void*)attn_decode_kernel<false>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    ME_CHECK(e == hipSuccess, "attention: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    lds_allowed[prologue] = lds;
+  }
+  const dim3 grid = a.spread_heads ? dim3(a.Hkv * col_tiles, num_seqs, num_parts) : dim3(num_seqs, a.Hkv * col_tiles, num_parts);
+  if (prologue) attn_decode_kernel<true><<<grid, dim3(256), lds, stream>>>(a);
+  else attn_decode_kernel<false><<<grid, dim3(256), lds, stream>>>(a);
+  ME_LAUNCH_CHECK();
+  if (num_parts > 1) {
+    attn_reduce_kernel<<<dim3(num_seqs, a.Hq), dim3(128), 0, stream>>>(a);
+    ME_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
 extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                               const void* k_cache, const void* v_cache, const int32_t* block_tables,
                               int bt_stride, const int32_t* context_lens, int num_seqs, int Hq, int Hkv,
@@ -1130,34 +1294,33 @@ extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_
   AttnArgs a;
   if (fill_common(a, q, q_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
                   num_seqs, Hq, Hkv, page, scale, window)) return -1;
-  ME_CHECK(num_parts >= 1 && num_parts <= RED_MAX_PARTS, "attention: %d partitions outside 1..%d", num_parts, RED_MAX_PARTS);
-  ME_CHECK(num_parts == 1 || (part_size >= 32 && part_size % 32 == 0),
-           "attention: partition size %d must be a multiple of 32", part_size);
-  ME_CHECK(num_parts == 1 || scratch != nullptr, "attention: split decode needs scratch");
-  a.part_size = num_parts == 1 ? (1 << 30) : part_size;
-  a.num_parts = num_parts;
-  a.spread_heads = spread_heads ? 1 : 0;
-  if (num_parts > 1) {
-    const int64_t rows = (int64_t)num_seqs * Hq * num_parts;
-    a.tmp_out = scratch; a.tmp_m = scratch + rows * HD; a.tmp_l = a.tmp_m + rows;
-  }
-  const int col_tiles = (a.G + 15) / 16;
-  ME_CHECK((int64_t)Hkv * col_tiles <= 65535 && num_seqs <= 65535,
-           "attention: %d sequences or %d head blocks exceed one launch", num_seqs, Hkv * col_tiles);
-  const size_t lds = (size_t)4 * (a.G < 16 ? a.G : 16) * (HD + 2) * sizeof(float);
-  static bool attr_set = false;
-  if (lds > 64 * 1024 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_decode_kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    ME_CHECK(e == hipSuccess, "attention: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    attr_set = true;
-  }
-  attn_decode_kernel<<<a.spread_heads ? dim3(Hkv * col_tiles, num_seqs, num_parts) : dim3(num_seqs, Hkv * col_tiles, num_parts),
-                       dim3(256), lds, stream>>>(a);
-  ME_LAUNCH_CHECK();
-  if (num_parts > 1) {
-    attn_reduce_kernel<<<dim3(num_seqs, Hq), dim3(128), 0, stream>>>(a);
-    ME_LAUNCH_CHECK();
-  }
-  return 0;
+  return launch_decode(a, num_seqs, part_size, num_parts, scratch, spread_heads, false, stream);
+}
+
+// A whole decode step's attention from the packed projection rows [num_seqs, (Hq + 2 Hkv) * HD] (row r belongs
+// to sequence r, its token stands at position context_lens[r] - 1): per-head norms of q and k (q_w, k_w
+// float32 [HD], or both null), rotation by `rope` [rope_rows, HD/2, 2] (or null), the new key and value into
+// their page (the one the block table names for that position), attention over the pages. The rows are left as
+// they were. max_context: no context_lens entry is larger (checked against rope_rows here, since the kernel
+// reads the table at context_lens[r] - 1).
+extern "C" int me_attn_decode_fused(const void* qkv, int64_t row_stride, void* out, int64_t out_stride,
+                                    const float* q_w, const float* k_w, float eps, const float* rope, int rope_rows,
+                                    void* k_cache, void* v_cache, const int32_t* block_tables, int bt_stride,
+                                    const int32_t* context_lens, int max_context, int num_seqs, int Hq, int Hkv,
+                                    int page, float scale, int window, int part_size, int num_parts,
+                                    float* scratch, int spread_heads, hipStream_t stream) {
+  if (num_seqs == 0) return 0;
+  AttnArgs a;
+  if (fill_common(a, qkv, row_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
+                  num_seqs, Hq, Hkv, page, scale, window)) return -1;
+  ME_CHECK((q_w == nullptr) == (k_w == nullptr), "attention: give both norm weights or neither");
+  ME_CHECK(rope == nullptr || (max_context >= 0 && max_context <= rope_rows),
+           "attention: a context of %d tokens is beyond the rotation table's %d positions", max_context, rope_rows);
+  ME_CHECK(rope == nullptr || reinterpret_cast<uintptr_t>(rope) % 8 == 0, "attention: the rotation table must be 8-byte aligned");
+  ME_CHECK(row_stride >= (int64_t)(Hq + 2 * Hkv) * HD, "attention: packed rows must hold q, k and v");
+  a.raw_k = (const bf16_t*)qkv + (int64_t)Hq * HD;
+  a.raw_v = a.raw_k + (int64_t)Hkv * HD;
+  a.q_w = q_w; a.k_w = k_w; a.eps = eps; a.rope = rope;
+  a.k_cache_w = (bf16_t*)k_cache; a.v_cache_w = (bf16_t*)v_cache;
+  return launch_decode(a, num_seqs, part_size, num_parts, scratch, spread_heads, true, stream);
 }

@@ -70,6 +70,7 @@ _CORE_PROTOS = {
 _ATTN_PROTOS = {
     "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, P, P, I, P],
     "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, I, P],
+    "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, I, P],
 }
 
 _core: _Lib | None = None
@@ -351,6 +352,45 @@ class HipBackend:
                      _ptr(pf), seq_of_token.data_ptr() + num_decodes * 4, num_decodes, _stream())
         return out
 
+    def decode_step_attention(self, qkv, q_weight, k_weight, eps, table, k_cache, v_cache, page: int, block_tables,
+                              context_lens, max_context: int, scale: float, window: int | None, Hq: int, Hkv: int,
+                              D: int, even_contexts: bool = False):
+        """A pure decode step's `qk_norm_rope_store` and `paged_attention` as one launch: rows [B, (Hq+2Hkv)*D]
+        as the packed product left them (row r is request r's one new token, at position context_lens[r] - 1).
+        The kernel norms and rotates q and the new key in float32, rounds them to bfloat16 as the separate
+        kernel leaves them in the rows, writes the new key and value to the page the block table names for
+        that position and attends over the pages. The rows stay as they were. Takes what `decode_step_fuses`
+        admits. Returns [B, Hq*D]. (reference models/qwen3.py:34-38, layers/attention.py:63-70: the same
+        four calls one after the other.)"""
+        B = qkv.shape[0]
+        _check(decode_step_fuses(qkv.dtype, D, page), "decode_step_attention: bfloat16 rows, head sizes in steps of 16 "
+               "up to 512 and pages of a power of two from 8 on")
+        _check(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (Hq + 2 * Hkv) * D,
+               f"decode_step_attention: rows must be [B, {(Hq + 2 * Hkv) * D}] with unit inner stride")
+        for w in (q_weight, k_weight):
+            _check(w is None or (w.dtype == torch.float32 and w.shape == (D,) and w.is_contiguous()),
+                   "decode_step_attention: norm weights must be float32 [D]")
+        _check((q_weight is None) == (k_weight is None), "decode_step_attention: give both norm weights or neither")
+        if table is not None:
+            _check(table.dtype == torch.float32 and table.is_contiguous() and table.shape[1:] == (D // 2, 2),
+                   "decode_step_attention: rotary table must be float32 [P, D/2, 2]")
+        _check(k_cache.shape[1:] == (Hkv, page, D) and v_cache.shape[1:] == (Hkv, D, page) and k_cache.is_contiguous()
+               and v_cache.is_contiguous() and k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype,
+               "decode_step_attention: caches must be K [pages, Hkv, page, D] and V [pages, Hkv, D, page] of the rows' dtype")
+        _check(block_tables.dim() == 2 and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
+               and block_tables.shape[0] >= B and _is_i32(context_lens) and context_lens.numel() >= B,
+               "decode_step_attention: block tables int32 [B, MB], context lengths int32 [B]")
+        _check(block_tables.shape[1] * page >= max_context, "decode_step_attention: block tables shorter than the longest context")
+        out = torch.empty((B, Hq * D), dtype=qkv.dtype, device=qkv.device)
+        part_size, num_parts = decode_partitions(B, Hq, Hkv, max_context)
+        scratch = _scratch(B * Hq * num_parts * (D + 2), qkv.device) if num_parts > 1 else None
+        attn_lib(D).call("me_attn_decode_fused", qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0),
+                         _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0],
+                         k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
+                         context_lens.data_ptr(), int(max_context), B, Hq, Hkv, page, float(scale), int(window or 0),
+                         part_size, num_parts, _ptr(scratch), 0 if even_contexts else 1, _stream())
+        return out
+
     # -- matrix products -----------------------------------------------------------------
     def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
                allow_partials: bool = False, out: torch.Tensor | None = None):
@@ -489,6 +529,7 @@ PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forc
 PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS wherever it fits (0: never)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
+FUSE_DECODE_STEP = True        # False: pure decode steps run norm/rotation/cache write and attention as two launches
 # The fused form evaluates the gate in every workgroup (N/16 of them), which is free while the
 # product waits for its weights but not over a long K: at 4096x12288, one row, fused 63 us against
 # 27 us for the plain product after a separate gating kernel (3 us).
@@ -658,6 +699,12 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int) -> tup
     return part, parts
 
 
+def decode_step_fuses(dtype: torch.dtype, D: int, page: int) -> bool:
+    """Whether `decode_step_attention` takes these rows: what the matrix-core attention kernels take."""
+    return bool(FUSE_DECODE_STEP and dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page >= 8
+                and page & (page - 1) == 0)
+
+
 def decode_contexts_even(num_seqs: int, min_context: int, max_context: int) -> bool:
     """Whether the decode kernel may keep each request's work on one XCD (8 requests or more whose
     contexts differ by 5 % at most), or has to spread every request over the XCDs. With all of a request
@@ -693,6 +740,7 @@ def silu_and_mul(*a, **k): return backend().silu_and_mul(*a, **k)
 def qk_norm_rope_store(*a, **k): return backend().qk_norm_rope_store(*a, **k)
 def store_kv(*a, **k): return backend().store_kv(*a, **k)
 def paged_attention(*a, **k): return backend().paged_attention(*a, **k)
+def decode_step_attention(*a, **k): return backend().decode_step_attention(*a, **k)
 def linear(*a, **k): return backend().linear(*a, **k)
 def silu_mul_linear(*a, **k): return backend().silu_mul_linear(*a, **k)
 def sample(*a, **k): return backend().sample(*a, **k)

@@ -62,6 +62,13 @@ class Attention(Mixer):
         kw = self.k_norm_weight if (self.qk_norm_eps is not None and self.own_kv) else qw
         table = self.position.rotary_table() if self.position is not None else None
         eps = self.qk_norm_eps or 0.0
+        if (store and step.num_decodes == step.num_tokens and (self.position is None or table is not None)
+                and ops.decode_step_fuses(qkv.dtype, D, cache.page_size)):
+            # only single tokens: norm, rotary, cache write and attention in one launch
+            o = ops.decode_step_attention(qkv, qw, kw, eps, table, cache.k, cache.v, cache.page_size, grp.block_tables,
+                                          step.context_lens, step.max_decode_context, self.scale, self.window,
+                                          Hq, Hkv, D, even_contexts=step.decode_contexts_even)
+            return self.o.forward(o, allow_partials=True)
         if self.position is None or table is not None:
             # norm + rotary + cache write in one pass
             if store:

@@ -102,6 +102,23 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
     return out
 
 
+def decode_step_attention(qkv, q_weight, k_weight, eps, table, k_cache, v_cache, page, block_tables, context_lens,
+                          max_context, scale, window, Hq, Hkv, D, even_contexts=False, compute_dtype=torch.float32):
+    """The two twins above, one after the other, on a copy of the rows: row r is request r's new token at
+    position context_lens[r] - 1, its slot is what the block table names for that position (a row with
+    context 0 is padding: nothing is written for it and it sees nothing)."""
+    B = qkv.shape[0]
+    ctx = context_lens[:B].long()
+    positions = (ctx - 1).clamp(min=0).to(torch.int32)
+    pages = block_tables[torch.arange(B, device=qkv.device), (positions // page).long()].long()
+    slots = torch.where((ctx > 0) & (pages >= 0), pages * page + positions.long() % page, torch.full_like(pages, -1)).to(torch.int32)
+    rows = qkv.clone()
+    qk_norm_rope_store(rows, q_weight, k_weight, eps, table, positions, slots, k_cache, v_cache, Hq, Hkv, D, page, store=True)
+    seq = torch.arange(B, dtype=torch.int32, device=qkv.device)
+    return paged_attention(rows[:, :Hq * D], k_cache, v_cache, page, block_tables, context_lens, seq, positions, None, B,
+                           max_context, scale, window, Hq, Hkv, D, compute_dtype=compute_dtype)
+
+
 def linear(x, w, out_dtype=None, allow_partials=False, out=None):
     y = (x.float() @ w.float().t()).to(out_dtype or x.dtype)
     if out is not None:
@@ -153,6 +170,7 @@ class PlainBackend:
     qk_norm_rope_store = staticmethod(qk_norm_rope_store)
     store_kv = staticmethod(store_kv)
     paged_attention = staticmethod(paged_attention)
+    decode_step_attention = staticmethod(decode_step_attention)
     linear = staticmethod(linear)
     silu_mul_linear = staticmethod(silu_mul_linear)
     sample = staticmethod(sample)

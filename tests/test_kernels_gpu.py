@@ -238,6 +238,55 @@ def test_attention_decode_batches(dtype, Hq, Hkv, D, page):
         close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,page", SHAPES + [(6, 3, 80, 8), (4, 4, 256, 16)])
+@pytest.mark.parametrize("window", [None, 50])
+def test_decode_step_in_one_launch(Hq, Hkv, D, page, window):
+    """Norms, rotation, cache write and attention of a pure decode step as one kernel, against the twins of
+    the separate kernels: outputs, what the pages hold afterwards (NaN wherever nothing was written), rows
+    untouched. Contexts: the new token alone, at a page's first and last place, first and last of a 32-key
+    block, in the last of many partitions; a padding row (context 0) writes nothing."""
+    torch.manual_seed(D + page)
+    P = 3200
+    ang = torch.outer(torch.arange(P, dtype=torch.float32), 1.0 / (1e4 ** (torch.arange(0, D, 2).float() / D)))
+    table = torch.stack((ang.cos(), ang.sin()), -1).contiguous().to(DEV)
+    qw, kw = torch.rand(D, device=DEV) + 0.5, torch.rand(D, device=DEV) + 0.5
+    for lens in ([1], [page, page + 1, 2 * page], [32, 33, 64, 65, 31], [1500, 7, 3000, 700], [130] * 9):
+        args = _attention_case(torch.bfloat16, Hq, Hkv, D, page, [(L, 1) for L in lens], window=window, seed=len(lens))
+        q, k_cache, v_cache, _, bt, ctx = args[:6]
+        rows = q._base
+        rows[:, Hq * D:] = torch.randn(len(lens), 2 * Hkv * D, device=DEV).to(torch.bfloat16)
+        B = len(lens)
+        # a padding row behind the others: context 0, a table without pages
+        rows = torch.cat((rows, torch.randn(1, rows.shape[1], device=DEV).to(torch.bfloat16)))
+        bt = torch.cat((bt, torch.full((1, bt.shape[1]), -1, dtype=torch.int32, device=DEV)))
+        ctx = torch.cat((ctx, torch.zeros(1, dtype=torch.int32, device=DEV)))
+        for b, L in enumerate(lens):                              # the new token's place holds nothing yet
+            pg = int(bt[b, (L - 1) // page])
+            k_cache[pg, :, (L - 1) % page, :] = float("nan")
+            v_cache[pg, :, :, (L - 1) % page] = float("nan")
+        for use_norm, use_rope in ((True, True), (False, True), (True, False)):
+            ka, va, kb, vb = k_cache.clone(), v_cache.clone(), k_cache.clone(), v_cache.clone()
+            before = rows.clone()
+            common = (qw if use_norm else None, kw if use_norm else None, 1e-6, table if use_rope else None)
+            tail = (page, bt, ctx, max(lens), D ** -0.5, window, Hq, Hkv, D)
+            got = hip().decode_step_attention(rows, *common, ka, va, *tail)
+            want = twin.decode_step_attention(rows, *common, kb, vb, *tail)
+            assert torch.equal(rows, before)
+            assert torch.equal(torch.isnan(ka), torch.isnan(kb)) and torch.equal(torch.isnan(va), torch.isnan(vb))
+            close(torch.nan_to_num(ka), torch.nan_to_num(kb), 4e-3)
+            assert torch.equal(torch.nan_to_num(va), torch.nan_to_num(vb))
+            close(got[:B], want[:B], 1.5e-2)
+            assert not got[B].isnan().any()
+            # and the same bits as the two launches it stands for (the q and k it forms are rounded alike)
+            k2, v2, r2 = k_cache.clone(), v_cache.clone(), rows[:B].clone()
+            pos = (ctx[:B] - 1)
+            slots = (bt[torch.arange(B, device=DEV), (pos // page).long()] * page + pos % page).to(torch.int32)
+            hip().qk_norm_rope_store(r2, *common, pos.to(torch.int32), slots, k2, v2, Hq, Hkv, D, page, True)
+            two = hip().paged_attention(r2[:, :Hq * D], k2, v2, page, bt[:B], ctx[:B], torch.arange(B, dtype=torch.int32, device=DEV),
+                                        pos.to(torch.int32), None, B, max(lens), D ** -0.5, window, Hq, Hkv, D)
+            close(got[:B], two, 4e-3)
+
+
 @pytest.mark.parametrize("window", [None, 100, 1000])
 def test_attention_decode_contexts_of_very_different_lengths(window):
     """One batch with contexts from 1 to 3,000 keys: the partitions are those of the longest, so most
