@@ -418,3 +418,189 @@ extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, in
   ME_LAUNCH_CHECK();
   return 0;
 }
+
+// ------------------------------------------------------------------ the skinny product behind an RMSNorm
+// y = (gamma * r / rms(r)) . w^T with r = the sum of the partial sums (+ the residual): what the norm kernel and
+// the skinny product do one after the other (reference layers/layernorm.py:11-24, then layers/linear.py:25-26),
+// as one launch, for a handful of rows. 1 / rms(r) is one number per row, so it is applied to the finished sums
+// in float32; the product itself runs on gamma * r rounded to bfloat16. Every workgroup forms that operand for
+// itself in LDS while its first weights are on their way (all M rows: M x K x (S + 1) floats out of L2) and adds
+// up r^2; the first workgroup also writes r, the new residual. K is not split. For one or two rows over a small
+// weight this saves about a microsecond of the six that the two launches take (1024 -> 4096: 5.4 against 6.4 us);
+// from three rows on, and over weights whose stream the prologue delays (4096 -> 24576: 44.8 against 41.4 us), the
+// two launches are faster, so the launcher takes at most NORM_MAX_ROWS rows.
+#define NORM_MAX_PARTIALS 8
+#define NORM_MAX_ROWS 2
+
+template <typename TX> struct Quad4;
+template <> struct Quad4<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+};
+template <> struct Quad4<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = static_cast<float>(t[i]);
+  }
+};
+
+template <typename TX, typename TO, bool EXACT_K>
+__global__ void __launch_bounds__(256)
+gemm_skinny_norm_kernel(const TX* __restrict__ xp, int S, int64_t part_stride, const float* __restrict__ res_in,
+                        float* __restrict__ res_out, const float* __restrict__ gamma, float eps,
+                        const bf16_t* __restrict__ w, int64_t ldw, TO* __restrict__ y, int64_t ldy, int M, int N,
+                        int K) {
+  extern __shared__ __align__(16) unsigned char norm_lds[];
+  const int ldx = K + 8;                                   // a row shifts by 16 bytes against the one before
+  bf16_t* xs = reinterpret_cast<bf16_t*>(norm_lds);        // [M][ldx] gamma * r
+  float* red = reinterpret_cast<float*>(norm_lds + (((size_t)M * ldx * sizeof(bf16_t) + 15) & ~(size_t)15));   // [4][256]
+  float* ssw = red + 4 * 256;                              // [4 waves][16 rows] sums of r^2
+  float* inv = ssw + 64;                                   // [16] 1 / rms
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int total_steps = (K + 127) / 128;
+  const bf16_t* wrow = w + (int64_t)(n0 + r < N ? n0 + r : 0) * ldw;
+  const bf16x8 z = gz8();
+
+  auto fetch = [&](int s, bool live, bf16x8 (&a)[4]) {
+    const int kb = 128 * s + 8 * g;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = kb + 32 * j;
+      a[j] = *reinterpret_cast<const bf16x8*>(live && (EXACT_K || k < K) ? wrow + k : w);
+    }
+  };
+  bf16x8 ring[2][4];
+  int s = wave;
+  fetch(s, s < total_steps, ring[0]);
+  pin_loads();
+
+  // ---- the rows: r = partial sums + residual, r^2 added up, gamma * r into LDS
+  constexpr int RA = NORM_MAX_ROWS;                        // rows whose loads go out together
+  const int quads = K >> 2;
+  for (int m0 = 0; m0 < M; m0 += RA) {
+    float ssr[RA];
+#pragma unroll
+    for (int a = 0; a < RA; ++a) ssr[a] = 0.f;
+    for (int q = threadIdx.x; q < quads; q += 256) {
+      float part[RA][NORM_MAX_PARTIALS][4], res[RA][4], gq[4];
+      Quad4<float>::load(gamma + 4 * q, gq);
+#pragma unroll
+      for (int a = 0; a < RA; ++a) {
+        const int m = m0 + a < M ? m0 + a : m0;
+#pragma unroll
+        for (int p = 0; p < NORM_MAX_PARTIALS; ++p)
+          if (p < S) Quad4<TX>::load(xp + p * part_stride + (int64_t)m * K + 4 * q, part[a][p]);
+        if (res_in) Quad4<float>::load(res_in + (int64_t)m * K + 4 * q, res[a]);
+      }
+#pragma unroll
+      for (int a = 0; a < RA; ++a) {
+        const int m = m0 + a;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = part[a][0][e];
+#pragma unroll
+        for (int p = 1; p < NORM_MAX_PARTIALS; ++p)
+          if (p < S) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += part[a][p][e];
+          }
+        if (res_in) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += res[a][e];
+        }
+        if (m < M) {
+          bf16x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            ssr[a] += v[e] * v[e];
+            o[e] = static_cast<bf16_t>(gq[e] * v[e]);
+          }
+          *reinterpret_cast<bf16x4*>(xs + m * ldx + 4 * q) = o;
+          if (blockIdx.x == 0 && res_out)
+            *reinterpret_cast<float4*>(res_out + (int64_t)m * K + 4 * q) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < RA; ++a) {
+      const float total = wave_sum(ssr[a]);
+      if (lane == 0 && m0 + a < M) ssw[wave * 16 + m0 + a] = total;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < M) {
+    const int m = threadIdx.x;
+    inv[m] = rsqrtf((ssw[m] + ssw[16 + m] + ssw[32 + m] + ssw[48 + m]) / (float)K + eps);
+  }
+
+  // ---- the product: weights from memory one step ahead, the rows from LDS
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  const bf16_t* xrow = xs + (r < M ? r : 0) * ldx;
+  auto product = [&](int step, const bf16x8 (&a)[4]) {
+    const int kb = 128 * step + 8 * g;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = kb + 32 * j;
+      const bool kok = EXACT_K || k < K;
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(xrow + (kok ? k : 0));
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kok ? a[j] : z, b, acc, 0, 0, 0);
+    }
+  };
+  while (s < total_steps) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      fetch(s + 4, s + 4 < total_steps, ring[u ^ 1]);
+      pin_loads();
+      if (s < total_steps) product(s, ring[u]);
+      s += 4;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[wave * 256 + r * 16 + 4 * g + i] = acc[i];
+  __syncthreads();
+  {
+    const int idx = threadIdx.x;
+    const int m = idx >> 4, n = n0 + (idx & 15);
+    if (m < M && n < N) {
+      const float v = red[idx] + red[256 + idx] + red[512 + idx] + red[768 + idx];
+      y[(int64_t)m * ldy + n] = from_f32<TO>(v * inv[m]);
+    }
+  }
+}
+
+// xp: bfloat16 or float32 [S, M, K] (S = 1: the rows themselves), contiguous; res_in float32 [M, K] or null;
+// res_out float32 [M, K] or null; gamma float32 [K]. y bfloat16 or float32 [M, N] with row stride ldy.
+extern "C" int me_gemm_skinny_norm_bf16(const void* xp, int x_dtype, int S, const float* res_in, float* res_out,
+                                        const float* gamma, float eps, const void* w, int64_t ldw, void* y,
+                                        int64_t ldy, int out_dtype, int M, int N, int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  ME_CHECK(M <= NORM_MAX_ROWS, "norm + skinny gemm: at most %d rows (%d)", NORM_MAX_ROWS, M);
+  ME_CHECK(S >= 1 && S <= NORM_MAX_PARTIALS, "norm + skinny gemm: %d partial sums outside 1..%d", S, NORM_MAX_PARTIALS);
+  ME_CHECK(K >= 8 && K % 8 == 0 && ldw % 8 == 0, "norm + skinny gemm: K=%d and the weight's row stride must be multiples of 8", K);
+  ME_CHECK(x_dtype == ME_F32 || (x_dtype == ME_BF16 && S == 1), "norm + skinny gemm: partial sums must be float32");
+  for (const void* p : {xp, (const void*)res_in, (const void*)res_out, (const void*)gamma, w})
+    ME_CHECK(reinterpret_cast<uintptr_t>(p) % 16 == 0, "norm + skinny gemm: operands must be 16-byte aligned");
+  ME_CHECK(xp && gamma && w && y && ldy >= N, "norm + skinny gemm: null operand or short output rows");
+  const size_t lds = ((size_t)M * (K + 8) * sizeof(bf16_t) + 15) / 16 * 16 + (4 * 256 + 64 + 16) * sizeof(float);
+  ME_CHECK(lds <= 64 * 1024, "norm + skinny gemm: %d rows of %d do not fit the workgroup's LDS", M, K);
+  dim3 grid((N + 15) / 16), block(256);
+  const bool exact = K % 128 == 0;
+  const int64_t part_stride = (int64_t)M * K;
+#define LAUNCH1(TX, TO, E)                                                                                   \
+  gemm_skinny_norm_kernel<TX, TO, E><<<grid, block, lds, stream>>>((const TX*)xp, S, part_stride, res_in,    \
+      res_out, gamma, eps, (const bf16_t*)w, ldw, (TO*)y, ldy, M, N, K)
+#define LAUNCH3(TX, TO) do { if (exact) LAUNCH1(TX, TO, true); else LAUNCH1(TX, TO, false); } while (0)
+  if (x_dtype == ME_F32 && out_dtype == ME_BF16) LAUNCH3(float, bf16_t);
+  else if (x_dtype == ME_BF16 && out_dtype == ME_BF16) LAUNCH3(bf16_t, bf16_t);
+  else if (x_dtype == ME_F32 && out_dtype == ME_F32) LAUNCH3(float, float);
+  else if (x_dtype == ME_BF16 && out_dtype == ME_F32) LAUNCH3(bf16_t, float);
+  else ME_CHECK(false, "norm + skinny gemm: bad dtype codes %d -> %d", x_dtype, out_dtype);
+#undef LAUNCH3
+#undef LAUNCH1
+  ME_LAUNCH_CHECK();
+  return 0;
+}

@@ -64,6 +64,7 @@ _CORE_PROTOS = {
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
+    "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, P],
     "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
@@ -455,6 +456,31 @@ class HipBackend:
         # float32 output form keeps the logits unrounded)
         return library_product(x, w, out_dtype, out=out)
 
+    def norm_linear(self, x: torch.Tensor, residual: torch.Tensor | None, norm_weight: torch.Tensor, eps: float,
+                    w: torch.Tensor, out_dtype: torch.dtype | None = None, want_residual: bool = True):
+        """`rms_norm` and `linear` behind it as one launch, for the few rows `norm_linear_fuses` admits:
+        r = x (+ residual), x being rows [M, K] or float32 partial sums [S, M, K]; y = (norm_weight * r
+        rounded to bfloat16) . w^T, scaled by 1 / rms(r) in float32 (the scale is one number per row, so
+        it is applied to the finished sums; the separate kernels round norm_weight * r / rms(r) instead:
+        the same relative rounding). Returns (y [M, N], r float32 [M, K] or None).
+        (reference layers/layernorm.py:11-24, layers/linear.py:25-26.)"""
+        _check(norm_linear_fuses(x, w), "norm_linear: bfloat16 weights, few rows, see norm_linear_fuses")
+        S = x.shape[0] if x.dim() == 3 else 1
+        M, K = x.shape[-2], x.shape[-1]
+        N = w.shape[0]
+        _check(norm_weight.dtype == torch.float32 and norm_weight.shape == (K,) and norm_weight.is_contiguous(),
+               "norm_linear: the norm's weight must be float32 [K]")
+        if residual is not None:
+            _check(residual.dtype == torch.float32 and residual.shape == (M, K) and residual.is_contiguous(),
+                   "norm_linear: residual must be contiguous float32 [M, K]")
+        out_dtype = out_dtype or w.dtype
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        res_out = torch.empty((M, K), dtype=torch.float32, device=x.device) if want_residual else None
+        core().call("me_gemm_skinny_norm_bf16", x.data_ptr(), _code(x.dtype), S, _ptr(residual), _ptr(res_out),
+                    norm_weight.data_ptr(), float(eps), w.data_ptr(), w.stride(0), y.data_ptr(), N, _code(out_dtype),
+                    M, N, K, _stream())
+        return y, res_out
+
     def silu_mul_linear(self, gu: torch.Tensor, w: torch.Tensor, allow_partials: bool = False):
         """(silu(gu[:, :I]) * gu[:, I:]) . w[N, I]^T: the gating fused into the product for few
         rows and a moderate width (bfloat16, M <= 16, I <= 4096, where the product is a weight stream
@@ -529,6 +555,9 @@ PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forc
 PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS wherever it fits (0: never)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
+FUSE_NORM_INTO_LINEAR = True   # False: the norm kernel and the product behind it always run as two launches
+NORM_FUSE_MAX_M = 2
+NORM_FUSE_MAX_WEIGHT = 8 << 20
 FUSE_DECODE_STEP = True        # False: pure decode steps run norm/rotation/cache write and attention as two launches
 # The fused form evaluates the gate in every workgroup (N/16 of them), which is free while the
 # product waits for its weights but not over a long K: at 4096x12288, one row, fused 63 us against
@@ -699,6 +728,29 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int) -> tup
     return part, parts
 
 
+def norm_linear_fuses(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether `norm_linear` takes rows x ([M, K], or float32 partial sums [S, M, K]) and weight w: a
+    bfloat16 weight that the unsplit skinny kernel would take, one or two rows, a weight of at most
+    NORM_FUSE_MAX_WEIGHT elements. Every workgroup forms the normed rows for itself, which costs each about
+    2 us; the norm kernel costs 3 us in a chain of decode kernels. Measured, us (two launches / one):
+    1024 -> 4096 with 4 partial sums: 1 row 6.4 / 5.4, 2 rows 6.3 / 5.7, 3 rows 6.4 / 7.5, 8 rows 6.6 / 11.2;
+    1024 -> 6144 with 6: 1 row 7.7 / 6.7, 2 rows 7.7 / 6.9, 4 rows 7.8 / 9.7; 4096 -> 6144: 1 row 16.5 / 15.7,
+    2 rows 16.2 / 16.2; 4096 -> 24576: 1 row 41.4 / 44.8 (the prologue delays the weight stream)."""
+    if not FUSE_NORM_INTO_LINEAR or w.dtype != torch.bfloat16 or w.dim() != 2 or x.dim() not in (2, 3):
+        return False
+    S = x.shape[0] if x.dim() == 3 else 1
+    M, K = x.shape[-2], x.shape[-1]
+    N = w.shape[0]
+    if x.dtype not in (torch.float32, torch.bfloat16) or (S > 1 and x.dtype != torch.float32) or S > 8:
+        return False
+    if not (1 <= M <= NORM_FUSE_MAX_M and K == w.shape[1] and K % 8 == 0 and x.is_contiguous() and w.stride(1) == 1
+            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        return False
+    if N * K > NORM_FUSE_MAX_WEIGHT or M * (K + 8) * 2 + 4416 > 64 * 1024:
+        return False
+    return skinny_takes(M, N, K)
+
+
 def decode_step_fuses(dtype: torch.dtype, D: int, page: int) -> bool:
     """Whether `decode_step_attention` takes these rows: what the matrix-core attention kernels take."""
     return bool(FUSE_DECODE_STEP and dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page >= 8
@@ -743,4 +795,5 @@ def paged_attention(*a, **k): return backend().paged_attention(*a, **k)
 def decode_step_attention(*a, **k): return backend().decode_step_attention(*a, **k)
 def linear(*a, **k): return backend().linear(*a, **k)
 def silu_mul_linear(*a, **k): return backend().silu_mul_linear(*a, **k)
+def norm_linear(*a, **k): return backend().norm_linear(*a, **k)
 def sample(*a, **k): return backend().sample(*a, **k)

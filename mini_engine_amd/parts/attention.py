@@ -19,6 +19,8 @@ class Attention(Mixer):
     another call has written.
     """
 
+    takes_pending_norm = True      # x goes to the packed product and nowhere else
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, qk_norm_eps: float | None = None, position: PositionEncoding | None = None,
                  window: int | None = None, own_kv: bool = True):

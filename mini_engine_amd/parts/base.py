@@ -154,6 +154,45 @@ class Norm(Part):
         """
         raise NotImplementedError
 
+    # Optional: linear_behind(x, residual, weight, out_dtype) -> (forward(x, residual)[0] . weight^T, new
+    # residual), norm and product as one kernel, or None where there is no such kernel for these shapes.
+
+
+class PendingNorm:
+    """A norm that has not run yet, in place of its output. A block hands one to a mixer or feed-forward
+    that declares `takes_pending_norm = True`; such a part passes it to its first `Linear`, which may run
+    norm and product as one kernel (`Norm.linear_behind`), or asks `value()` for the normed rows as a
+    tensor. Whichever happens first also yields the new residual, which the block reads afterwards."""
+
+    def __init__(self, norm: "Norm", x: torch.Tensor, residual: torch.Tensor | None):
+        self.norm, self.x, self.residual = norm, x, residual
+        self._y = None
+        self._new_residual = None
+
+    def value(self) -> torch.Tensor:
+        if self._y is None:
+            x = self.x
+            if x.dim() == 3 and not getattr(self.norm, "accepts_partials", False):
+                x = x.sum(0)
+            self._y, self._new_residual = self.norm.forward(x, self.residual)
+        return self._y
+
+    def into_linear(self, weight: torch.Tensor, out_dtype=None):
+        """The product of the normed rows with `weight` ([out, in]) if the norm can run inside it, else None."""
+        behind = getattr(self.norm, "linear_behind", None)
+        if self._y is not None or behind is None:
+            return None
+        got = behind(self.x, self.residual, weight, out_dtype)
+        if got is None:
+            return None
+        y, self._new_residual = got
+        return y
+
+    def new_residual(self) -> torch.Tensor:
+        if self._new_residual is None:
+            self.value()
+        return self._new_residual
+
 
 class PositionEncoding(Part):
     """Something applied to queries and keys as a function of token positions."""

@@ -1,7 +1,7 @@
 """How norm, mixer and feed-forward are arranged in a layer (reference models/qwen3.py:55-74)."""
 from __future__ import annotations
 
-from .base import FeedForward, Mixer, Norm, Part, register_part
+from .base import FeedForward, Mixer, Norm, Part, PendingNorm, register_part
 
 
 def norm_of(norm: Norm, x, residual):
@@ -36,7 +36,17 @@ class PreNormBlock(Part):
         return self.mixer.state_need()
 
     def forward(self, h, residual, step, cache, state):
-        x, residual = norm_of(self.norm1, h, residual)
-        a = self.mixer.forward(x, step, cache, state)
+        # a part that takes it gets the norm before it as a `PendingNorm` and may run it inside its first product
+        if getattr(self.mixer, "takes_pending_norm", False):
+            x = PendingNorm(self.norm1, h, residual)
+            a = self.mixer.forward(x, step, cache, state)
+            residual = x.new_residual()
+        else:
+            x, residual = norm_of(self.norm1, h, residual)
+            a = self.mixer.forward(x, step, cache, state)
+        if getattr(self.feed_forward, "takes_pending_norm", False):
+            x = PendingNorm(self.norm2, a, residual)
+            out = self.feed_forward.forward(x)
+            return out, x.new_residual()
         x, residual = norm_of(self.norm2, a, residual)
         return self.feed_forward.forward(x), residual

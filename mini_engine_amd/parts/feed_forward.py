@@ -11,6 +11,8 @@ class SwiGLU(FeedForward):
     """down(silu(gate(x)) * up(x)); gate and up are one packed product with gate's rows first
     (reference layers/linear.py:29-45, layers/activation.py:5-7)."""
 
+    takes_pending_norm = True      # x goes to the packed product and nowhere else
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         super().__init__()
         self.hidden_size = hidden_size

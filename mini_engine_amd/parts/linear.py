@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 from ..kernels import ops
-from .base import ParamSpec, Part
+from .base import ParamSpec, Part, PendingNorm
 
 
 class Linear(Part):
@@ -20,5 +20,11 @@ class Linear(Part):
 
     def forward(self, x, out_dtype=None, allow_partials: bool = False):
         """With allow_partials the result may be float32 partial sums [P, M, N] (a product whose K
-        range was split over workgroups); the consumer, a norm, adds them."""
+        range was split over workgroups); the consumer, a norm, adds them. x may be a `PendingNorm`:
+        the norm then runs inside the product where there is a kernel for that, else in front of it."""
+        if isinstance(x, PendingNorm):
+            y = x.into_linear(self.weight, out_dtype)
+            if y is not None:
+                return y
+            x = x.value()
         return ops.linear(x, self.weight, out_dtype, allow_partials)

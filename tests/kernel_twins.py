@@ -127,6 +127,16 @@ def linear(x, w, out_dtype=None, allow_partials=False, out=None):
     return y
 
 
+def norm_linear(x, residual, norm_weight, eps, w, out_dtype=None, want_residual=True, compute_dtype=torch.float32):
+    """The fused kernel's rounding points: gamma * r to the weight's dtype, product, then 1 / rms(r)."""
+    r = x.float().sum(0) if x.dim() == 3 else x.float()
+    if residual is not None:
+        r = r + residual
+    inv = torch.rsqrt(r.to(compute_dtype).pow(2).mean(-1, keepdim=True) + eps)
+    y = ((norm_weight * r).to(w.dtype).to(compute_dtype) @ w.to(compute_dtype).t()) * inv
+    return y.to(out_dtype or w.dtype), (r if want_residual else None)
+
+
 def silu_mul_linear(gu, w, allow_partials=False):
     return linear(silu_and_mul(gu), w)
 
@@ -173,4 +183,5 @@ class PlainBackend:
     decode_step_attention = staticmethod(decode_step_attention)
     linear = staticmethod(linear)
     silu_mul_linear = staticmethod(silu_mul_linear)
+    norm_linear = staticmethod(norm_linear)
     sample = staticmethod(sample)

@@ -420,6 +420,40 @@ def test_linear_skinny_bf16(M, N, K):
     close(parts.sum(0) if parts.dim() == 3 else parts, ref, 6e-3 if parts.dim() == 2 else 2e-5)
 
 
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("N,K", [(4096, 1024), (6144, 1024), (384, 80), (1000, 224), (100, 2048), (1536, 4096)])
+@pytest.mark.parametrize("S", [0, 1, 6])
+def test_norm_inside_the_skinny_product(M, N, K, S):
+    """RMSNorm (+ residual, + partial sums) and the product behind it as one kernel, against the twin with
+    the kernel's rounding points and against the two kernels it stands for. S = 0: bfloat16 rows without a
+    residual (a model's first layer); else float32 [S, M, K] with a residual."""
+    torch.manual_seed(M * 31 + S)
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    gamma = torch.rand(K, device=DEV) + 0.5
+    if S == 0:
+        x, res = (torch.randn(M, K, device=DEV) * 3).bfloat16(), None
+    else:
+        x, res = torch.randn(S, M, K, device=DEV), torch.randn(M, K, device=DEV) * 2
+        x[:, 0] *= 30                                     # rows of very different size: the scale is per row
+    assert ops.norm_linear_fuses(x, w)
+    assert not ops.norm_linear_fuses(x[..., :1, :].expand(*x.shape[:-2], 3, K).contiguous(), w)      # three rows: two launches
+    y, r = hip().norm_linear(x, res, gamma, 1e-6, w)
+    want_y, want_r = twin.norm_linear(x, res, gamma, 1e-6, w)
+    assert torch.equal(r, want_r) if S <= 1 else True
+    close(r, want_r, 1e-6)
+    close(y, want_y, 6e-3)                                 # bf16 output rounding, as for the product alone
+    normed, r2 = hip().rms_norm(x, gamma, 1e-6, res, torch.bfloat16)
+    assert torch.equal(r, r2)                              # the residual is summed in the same order
+    two = hip().linear(normed, w)
+    rows = two.float().abs().amax(dim=1, keepdim=True).clamp_min(1e-30)
+    assert float(((y.float() - two.float()).abs() / rows).max()) <= 1.5e-2      # row by row: bfloat16 rounding of the operand
+    y32, _ = hip().norm_linear(x, res, gamma, 1e-6, w, out_dtype=torch.float32, want_residual=False)
+    # float32 output, against the exact product of the operand that the kernel's own r rounds to (a last-bit
+    # difference in r can round gamma * r to the other bfloat16): accumulation error only
+    exact = twin.norm_linear(r, None, gamma, 1e-6, w, out_dtype=torch.float64, compute_dtype=torch.float64)[0]
+    close(y32, exact, 2e-5)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40])
 @pytest.mark.parametrize("N,I", [(1024, 3072), (80, 224), (72, 200)])
 def test_silu_mul_linear(M, N, I):

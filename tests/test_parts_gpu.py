@@ -59,6 +59,43 @@ def test_rotary_part_matches_plain_tables_and_unfused_apply():
     assert torch.allclose(q.double().cpu(), qr, atol=1e-5)
 
 
+@pytest.mark.parametrize("rows", [1, 2, 5])
+def test_norm_handed_to_the_next_part_unrun(rows):
+    """A part that `takes_pending_norm` gets the norm in front of it as a `PendingNorm`. Its first product runs
+    the norm inside itself where there is a kernel for that (bfloat16, one or two rows), otherwise the norm runs
+    in front of it: either way the part's output and the new residual are those of the plain formulas. A norm
+    without `linear_behind` (a toy one, defined here) is simply run."""
+    from mini_engine_amd.parts import PendingNorm
+    from mini_engine_amd.parts.base import Norm
+    dtype = torch.bfloat16
+    norm = make_part("norm", "rms", size=80, eps=3e-6); _bind(norm, dtype)
+    ff = make_part("feed_forward", "swiglu", hidden_size=80, intermediate_size=224); _bind(ff, dtype)
+    assert ff.takes_pending_norm
+    parts, r = torch.randn(3, rows, 80, device=DEV), torch.randn(rows, 80, device=DEV)
+    xr, rr = P.add_rms_norm(parts.double().sum(0), r.double(), norm.weight.double(), 3e-6)
+    w = ff.gate_up.weight.double()
+    ref = P.silu_and_mul(xr @ w[:224].T, xr @ w[224:].T) @ ff.down.weight.double().T
+
+    def check(pending):
+        y = ff.forward(pending)
+        y = y.sum(0) if y.dim() == 3 else y
+        assert float((y.double() - ref).abs().max() / ref.abs().max()) <= 2e-2
+        assert torch.allclose(pending.new_residual().double(), rr, atol=1e-5)
+
+    pending = PendingNorm(norm, parts, r)
+    check(pending)
+    assert (pending._y is None) == (rows <= 2)             # one or two rows: the norm never ran on its own
+
+    class PlainNorm(Norm):                                 # no partial sums, no fused form
+        def forward(self, x, residual):
+            return norm.forward(x, residual)
+
+    check(PendingNorm(PlainNorm(), parts, r))
+    late = PendingNorm(norm, parts, r)                     # asked for its value first: runs as a norm, once
+    first = late.value()
+    assert late.into_linear(ff.gate_up.weight) is None and late.value() is first
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
 @pytest.mark.parametrize("window", [None, 10])
 def test_attention_part_alone(dtype, tol, window):
