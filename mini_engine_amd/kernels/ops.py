@@ -334,7 +334,7 @@ class HipBackend:
             max_prefill_context = max(max_prefill_context, max_decode_context)
             num_decodes = 0
         if num_decodes > 0:
-            part_size, num_parts = decode_partitions(num_decodes, Hq, Hkv, max_decode_context)
+            part_size, num_parts = decode_partitions(num_decodes, Hq, Hkv, max_decode_context, even_contexts)
             scratch = _scratch(num_decodes * Hq * num_parts * (D + 2), q.device) if num_parts > 1 else None
             lib.call("me_attn_decode", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
@@ -383,7 +383,7 @@ class HipBackend:
                "decode_step_attention: block tables int32 [B, MB], context lengths int32 [B]")
         _check(block_tables.shape[1] * page >= max_context, "decode_step_attention: block tables shorter than the longest context")
         out = torch.empty((B, Hq * D), dtype=qkv.dtype, device=qkv.device)
-        part_size, num_parts = decode_partitions(B, Hq, Hkv, max_context)
+        part_size, num_parts = decode_partitions(B, Hq, Hkv, max_context, even_contexts)
         scratch = _scratch(B * Hq * num_parts * (D + 2), qkv.device) if num_parts > 1 else None
         attn_lib(D).call("me_attn_decode_fused", qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0),
                          _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0],
@@ -569,6 +569,8 @@ _COMPUTE_UNITS = 256
 _DECODE_WORKGROUPS = 4096
 _DECODE_WHOLE_WORKGROUPS = 2048
 _DECODE_WHOLE_MAX_KEYS = 4096
+_DECODE_EVEN_WHOLE_WORKGROUPS = 192
+_DECODE_EVEN_WHOLE_MAX_KEYS = 8192
 _DECODE_MAX_PARTITION = 2048
 _scratch_buf: dict = {}
 _scratch_retired: list = []      # outgrown buffers stay alive: a captured graph may still write to them
@@ -702,7 +704,7 @@ def choose_ksplit(M: int, N: int, K: int) -> int:
     return max(1, min(-(-_TARGET_WORKGROUPS // tiles), K // 512, 8))
 
 
-def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int) -> tuple:
+def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: bool = False) -> tuple:
     """(keys per partition, number of partitions) for the split decode kernel.
 
     A workgroup's 4 waves take 32 keys each per round, so a partition of 128 keys is one round
@@ -714,12 +716,20 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int) -> tup
     (128 sequences, four of 16 k keys among 100-2,048: 4096 x 4 311 us, 2048 x 8 283 us, 1024 x 16 280 us).
     From 2,048 workgroups on (256 sequences x 8 kv heads) a context up to 4,096 keys is one partition and
     needs no reduce kernel (256 x 4,096 keys: 719 us against 752 us in two; 256 x 100-600 keys: 74 against
-    83 us). (The reference's rule: layers/ops.py:44-51, split when sequences x kv heads cannot fill the
-    SMs, 256-key partitions.)"""
+    83 us). `even` (the contexts are equally long, `decode_contexts_even`): from 192 workgroups on (24
+    sequences x 8 kv heads) a context up to 8,192 keys is one partition: every workgroup then has the same
+    work, none waits for another's partial results and no reduce kernel follows (us, default split / one
+    partition: 24 x 2,048 keys 34.2 / 32.9, 32 x 2,048 44.1 / 39.6, 64 x 2,048 104.9 / 97.3, 64 x 512
+    25.9 / 21.7, 32 x 8,192 196.5 / 182.0, 128 x 2,048 201.8 / 187.7; 16 x 2,048 25.3 / 31.0, hence the
+    192; contexts of 100-2,048 keys gain nothing from it and long ones among short ones lose, hence only
+    for equal ones). (The reference's rule: layers/ops.py:44-51, split when sequences x kv heads cannot
+    fill the SMs, 256-key partitions.)"""
     col_tiles = (Hq // Hkv + 15) // 16
     base = max(1, num_seqs * Hkv * col_tiles)
     ctx = max(1, max_context)
     if base >= _DECODE_WHOLE_WORKGROUPS and ctx <= _DECODE_WHOLE_MAX_KEYS:
+        return -(-ctx // 128) * 128, 1
+    if even and base >= _DECODE_EVEN_WHOLE_WORKGROUPS and ctx <= _DECODE_EVEN_WHOLE_MAX_KEYS:
         return -(-ctx // 128) * 128, 1
     want = max(1, -(-_DECODE_WORKGROUPS // base), -(-ctx // _DECODE_MAX_PARTITION))
     want = min(64, want)

@@ -15,6 +15,10 @@ def test_decode_partitions_cover_the_context():
     # 2,048 workgroups without a split: contexts up to 4,096 keys stay whole
     assert ops.decode_partitions(256, 16, 8, 2048) == (2048, 1) and ops.decode_partitions(256, 16, 8, 4096) == (4096, 1)
     assert ops.decode_partitions(255, 16, 8, 2048)[1] > 1 and ops.decode_partitions(256, 16, 8, 4097)[1] > 1
+    # equally long contexts: whole from 192 workgroups on, up to 8,192 keys
+    assert ops.decode_partitions(24, 16, 8, 2048, even=True) == (2048, 1) and ops.decode_partitions(64, 32, 8, 8192, even=True) == (8192, 1)
+    assert ops.decode_partitions(23, 16, 8, 2048, even=True)[1] > 1 and ops.decode_partitions(64, 16, 8, 8193, even=True)[1] > 1
+    assert ops.decode_partitions(64, 16, 8, 2048, even=False)[1] > 1
 
 
 def test_prefill_segments_cover_the_span_and_hold_512_keys_or_more():

@@ -287,6 +287,18 @@ def test_decode_step_in_one_launch(Hq, Hkv, D, page, window):
             close(got[:B], two, 4e-3)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,page", [(16, 8, 128, 16), (6, 2, 32, 8), (64, 8, 128, 16)])
+def test_attention_decode_equal_contexts_in_one_partition(Hq, Hkv, D, page):
+    """Equally long contexts with 192 workgroups or more: one partition each, no reduce kernel."""
+    n = -(-192 // Hkv)
+    seqs = [(1500 + i % 20, 1) for i in range(n)]
+    assert ops.decode_partitions(n, Hq, Hkv, 1519, True)[1] == 1 and ops.decode_partitions(n, Hq, Hkv, 1519, False)[1] > 1
+    args = _attention_case(torch.bfloat16, Hq, Hkv, D, page, seqs, seed=3, peak=700)
+    want = twin.paged_attention(*args)
+    close(hip().paged_attention(*args, even_contexts=True), want, 1.5e-2)
+    close(hip().paged_attention(*args, even_contexts=False), want, 1.5e-2)
+
+
 @pytest.mark.parametrize("window", [None, 100, 1000])
 def test_attention_decode_contexts_of_very_different_lengths(window):
     """One batch with contexts from 1 to 3,000 keys: the partitions are those of the longest, so most
