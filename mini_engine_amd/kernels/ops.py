@@ -567,7 +567,7 @@ GATED_MAX_M = 16
 _TARGET_WORKGROUPS = 512
 _COMPUTE_UNITS = 256
 _DECODE_WORKGROUPS = 4096
-_DECODE_WHOLE_WORKGROUPS = 2048
+_DECODE_WHOLE_WORKGROUPS = 768
 _DECODE_WHOLE_MAX_KEYS = 4096
 _DECODE_EVEN_WHOLE_WORKGROUPS = 192
 _DECODE_EVEN_WHOLE_MAX_KEYS = 8192
@@ -714,9 +714,11 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
     partitions cover the context): a workgroup goes through its keys round by round, so in a batch with
     a few long contexts among short ones the long partitions are what is still running at the end
     (128 sequences, four of 16 k keys among 100-2,048: 4096 x 4 311 us, 2048 x 8 283 us, 1024 x 16 280 us).
-    From 2,048 workgroups on (256 sequences x 8 kv heads) a context up to 4,096 keys is one partition and
-    needs no reduce kernel (256 x 4,096 keys: 719 us against 752 us in two; 256 x 100-600 keys: 74 against
-    83 us). `even` (the contexts are equally long, `decode_contexts_even`): from 192 workgroups on (24
+    From 768 workgroups on (96 sequences x 8 kv heads) a context up to 2,048 keys (4,096 from 2,048 workgroups
+    on) is one partition and needs no reduce kernel (us, split / whole: 256 x 4,096 keys 752 / 719; 256 x 100-600 keys 83 / 74; contexts
+    of 100-2,048 keys: 192 sequences 159 / 145, 128 sequences 107 / 98, 100 of 600-2,048 keys 105 / 95; below, 40
+    sequences of 1,000-2,048 keys 41.6 / 44.2 and 64 of 100-2,048
+    56.1 / 55.8, hence the 768). `even` (the contexts are equally long, `decode_contexts_even`): from 192 workgroups on (24
     sequences x 8 kv heads) a context up to 8,192 keys is one partition: every workgroup then has the same
     work, none waits for another's partial results and no reduce kernel follows (us, default split / one
     partition: 24 x 2,048 keys 34.2 / 32.9, 32 x 2,048 44.1 / 39.6, 64 x 2,048 104.9 / 97.3, 64 x 512
@@ -727,7 +729,7 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
     col_tiles = (Hq // Hkv + 15) // 16
     base = max(1, num_seqs * Hkv * col_tiles)
     ctx = max(1, max_context)
-    if base >= _DECODE_WHOLE_WORKGROUPS and ctx <= _DECODE_WHOLE_MAX_KEYS:
+    if base >= _DECODE_WHOLE_WORKGROUPS and ctx <= (_DECODE_WHOLE_MAX_KEYS if base >= 2048 else _DECODE_WHOLE_MAX_KEYS // 2):
         return -(-ctx // 128) * 128, 1
     if even and base >= _DECODE_EVEN_WHOLE_WORKGROUPS and ctx <= _DECODE_EVEN_WHOLE_MAX_KEYS:
         return -(-ctx // 128) * 128, 1

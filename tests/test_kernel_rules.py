@@ -12,9 +12,9 @@ def test_decode_partitions_cover_the_context():
     # a partition holds at most 2,048 keys while 64 partitions cover the context
     assert ops.decode_partitions(128, 16, 8, 16384) == (2048, 8) and ops.decode_partitions(256, 16, 8, 8192) == (2048, 4)
     assert ops.decode_partitions(3, 6, 2, 130000) == (2048, 64) and ops.decode_partitions(4, 16, 8, 1 << 20) == (16384, 64)
-    # 2,048 workgroups without a split: contexts up to 4,096 keys stay whole
-    assert ops.decode_partitions(256, 16, 8, 2048) == (2048, 1) and ops.decode_partitions(256, 16, 8, 4096) == (4096, 1)
-    assert ops.decode_partitions(255, 16, 8, 2048)[1] > 1 and ops.decode_partitions(256, 16, 8, 4097)[1] > 1
+    # 768 workgroups without a split: contexts up to 4,096 keys stay whole
+    assert ops.decode_partitions(256, 16, 8, 2048) == (2048, 1) and ops.decode_partitions(96, 16, 8, 2048) == (2048, 1)
+    assert ops.decode_partitions(95, 16, 8, 2048)[1] > 1 and ops.decode_partitions(96, 16, 8, 2049)[1] > 1 and ops.decode_partitions(256, 16, 8, 4097)[1] > 1
     # equally long contexts: whole from 192 workgroups on, up to 8,192 keys
     assert ops.decode_partitions(24, 16, 8, 2048, even=True) == (2048, 1) and ops.decode_partitions(64, 32, 8, 8192, even=True) == (8192, 1)
     assert ops.decode_partitions(23, 16, 8, 2048, even=True)[1] > 1 and ops.decode_partitions(64, 16, 8, 8193, even=True)[1] > 1
