@@ -188,6 +188,46 @@ def folder_for(cfg, seed: int, root: str, on_device: bool) -> tuple:
     return root, None
 
 
+def box_rates() -> dict:
+    """What this GPU reaches on the plainest work of each kind, beside the published peaks that the fractions are
+    taken of: a device copy of 1 GiB (bytes read + written), one-row products over four weights of 201 MB in turn
+    (bytes read; the engine's own streaming kernel at the 8B sizes' largest product), and a library product of
+    8192^3 in bfloat16."""
+    import torch
+    from mini_engine_amd.kernels import ops
+    dev = torch.device("cuda")
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    a = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
+    b = torch.empty_like(a)
+    copy = timed(lambda: b.copy_(a), 10)
+    del b
+    size = 24576 * 4096
+    weights, row = [a[i * size:(i + 1) * size].view(24576, 4096) for i in range(4)], a[4 * size:4 * size + 4096].view(1, 4096)
+
+    def stream():
+        for weight in weights:
+            ops.linear(row, weight)
+
+    read = timed(stream, 5)
+    del a, weights, row
+    x = torch.randn(8192, 8192, device=dev).bfloat16()
+    w = torch.randn(8192, 8192, device=dev).bfloat16()
+    mm = timed(lambda: ops.library_product(x, w, torch.bfloat16), 10)
+    del x, w
+    torch.cuda.empty_cache()
+    return {"hbm_copy_GBs": round(2 * (1 << 30) / copy / 1e9, 1), "hbm_read_GBs": round(4 * size * 2 / read / 1e9, 1),
+            "library_product_bf16_TFLOPs": round(2 * 8192 ** 3 / mm / 1e12, 1)}
+
+
 def measure(args, size: str, layers, tmp: str, points: list, steps: int, warmup: int, serve: bool) -> dict:
     """Prefill, decode at the default batch and at `points`, and the served workloads, at one model size."""
     cfg, full_layers = model_config(size, layers)
@@ -308,6 +348,9 @@ def main(argv=None) -> int:
     for name in ("offline", "mixed_lengths"):
         if name in main_run:
             line[name] = main_run[name]
+    if args.dtype == "bfloat16":
+        line["box"] = box_rates()
+        log(f"this GPU: {line['box']}")
     print(json.dumps(line), flush=True)
     return 0
 
