@@ -330,6 +330,17 @@ def test_attention_far_key_stands_out(prefill_form, dtype):
         close(hip().paged_attention(*args), twin.paged_attention(*args), 1e-5 if dtype == torch.float32 else 1.5e-2)
 
 
+@pytest.mark.parametrize("window", [None, 1000])
+def test_attention_over_very_long_contexts(prefill_form, window):
+    """One request of 70,000 keys decoding (61 partitions of 1,152 keys, the most the reduce kernel merges is 64)
+    and a portion of 48 tokens behind 40,000 cached ones (cut into segments): the one key that matters lies far
+    back, near the start of the context when all keys are visible, near the window's far edge otherwise."""
+    for seqs, peak in (([(70000, 1)], 37 if window is None else 69100), ([(40048, 48)], 40000 - 900 if window else 11)):
+        args = _attention_case(torch.bfloat16, 16, 8, 128, 16, seqs, window=window, seed=5, peak=peak)
+        close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
+    assert ops.decode_partitions(1, 16, 8, 70000)[1] == 61
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(40, 8), (64, 8)])
 @pytest.mark.parametrize("window", [None, 100])
 def test_attention_wide_groups_at_head_size_128(prefill_form, monkeypatch, Hq, Hkv, window):
