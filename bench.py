@@ -235,7 +235,7 @@ def measure(args, size: str, layers, tmp: str, points: list, steps: int, warmup:
     on_device = args.weights == "device" or (args.weights == "auto" and params > 2e9)
     folder, random_weights = folder_for(cfg, args.seed, os.path.join(tmp, size), on_device)
     gen = max(args.gen, steps + warmup + 2)
-    max_len = max(args.context + gen + 128, 4096, 8192 if (serve and args.mixed_lengths) else 0)
+    max_len = max(args.context + gen + 128, args.prefill_tokens + 128, 4096, 8192 if (serve and args.mixed_lengths) else 0)
     batches = [args.batch] + points
     max_seqs = max(batches + ([256] if serve and (args.offline or args.mixed_lengths) else []))
     budget = max(args.prefill_tokens, 2048 if (serve and args.mixed_lengths) else 16384, max_seqs)
