@@ -128,7 +128,11 @@ struct SkinnyOperands {
 // EXACT_K: K is a multiple of 128, so no k-slot of any step lies beyond K and nothing is zeroed.
 // Rows beyond N or M are read from row 0 and not zeroed either: an output element depends on its
 // own weight row and token row only, and the elements of such rows are never written.
-template <int MT, typename TO, bool GATED, bool EXACT_K>
+// ACT (one tile of tokens, K not split): w is a packed gate/up weight [N = 2 I, K], gate rows first (reference
+// layers/linear.py:29-45), and y is silu(gate) * up, [M, I] (layers/activation.py:5-7): a workgroup takes 8 gate
+// features and the 8 up features that go with them as the 16 rows of its matrix operand and pairs them when it
+// merges its waves, so every gate is formed once, from the unrounded sums.
+template <int MT, typename TO, bool GATED, bool EXACT_K, bool ACT = false>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                    TO* __restrict__ y, int64_t ldy, float* __restrict__ partials, int M, int N, int K,
@@ -136,13 +140,17 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
   __shared__ float red[4][MT][256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16 * MT;
+  const int n0 = blockIdx.x * (ACT ? 8 : 16), m0 = blockIdx.y * 16 * MT;
   const int split = blockIdx.z;
   const int s_begin = split * steps_per_split;
   const int total_steps = (K + 127) / 128;
   const int s_end = min(total_steps, s_begin + steps_per_split);
 
-  const bf16_t* wrow = w + (int64_t)(n0 + r < N ? n0 + r : 0) * ldw;
+  const int half = N >> 1;                 // ACT: gate features 0..half-1, their up features behind them
+  int feature;
+  if (ACT) feature = n0 + (r & 7) < half ? (r < 8 ? n0 + r : half + n0 + r - 8) : 0;
+  else feature = n0 + r < N ? n0 + r : 0;
+  const bf16_t* wrow = w + (int64_t)feature * ldw;
   const bf16_t* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -222,6 +230,16 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[wave][mt][r * 16 + 4 * g + i] = acc[mt][i];
   __syncthreads();
+  if (ACT) {
+    const int idx = threadIdx.x, m = idx >> 3, f = idx & 7;
+    if (idx < 128 && m0 + m < M && n0 + f < half) {
+      const int ig = m * 16 + f, iu = ig + 8;
+      const float gate = red[0][0][ig] + red[1][0][ig] + red[2][0][ig] + red[3][0][ig];
+      const float up = red[0][0][iu] + red[1][0][iu] + red[2][0][iu] + red[3][0][iu];
+      y[(int64_t)(m0 + m) * ldy + n0 + f] = from_f32<TO>(gate / (1.f + expf(-gate)) * up);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < MT * 256; e += 256) {
     const int mt = e >> 8, idx = e & 255;
     const int m = m0 + 16 * mt + (idx >> 4), n = n0 + (idx & 15);
@@ -376,10 +394,31 @@ extern "C" int me_gemm_rows_bf16(const void* x, int64_t ldx, const void* w, int6
 }
 
 // y: bf16 or float32 [M, N]; or, when ksplit > 1, `partials` float32 [ksplit, M, N] (y unused).
+// gated: x is [M, 2K] and silu(x[:, :K]) * x[:, K:] is what is multiplied. act: w is a packed gate/up weight and y
+// is silu(gate) * up, [M, N / 2] (at most 16 rows, K not split, not together with gated).
 extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y,
                                    int64_t ldy, int out_dtype, float* partials, int ksplit, int M, int N,
-                                   int K, int gated, hipStream_t stream) {
+                                   int K, int gated, int act, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
+  if (act) {
+    ME_CHECK(!gated && ksplit == 1 && partials == nullptr && M <= 16 && N % 2 == 0,
+             "skinny gemm: the gating epilogue takes at most 16 rows, an unsplit K and an even number of weight rows");
+    ME_CHECK(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldy >= N / 2,
+             "skinny gemm: K=%d and the row strides must be multiples of 8", K);
+    ME_CHECK((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0),
+             "skinny gemm: operands must be 16-byte aligned");
+    const int steps = (K + 127) / 128;
+    dim3 grid((N / 2 + 7) / 8, 1, 1), block(256);
+#define LAUNCH_ACT(TO, E)                                                                                    \
+  gemm_skinny_kernel<1, TO, false, E, true><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, \
+                                                                        (TO*)y, ldy, nullptr, M, N, K, steps)
+    if (out_dtype == ME_BF16) { if (K % 128 == 0) LAUNCH_ACT(bf16_t, true); else LAUNCH_ACT(bf16_t, false); }
+    else if (out_dtype == ME_F32) { if (K % 128 == 0) LAUNCH_ACT(float, true); else LAUNCH_ACT(float, false); }
+    else ME_CHECK(false, "skinny gemm: bad output dtype code %d", out_dtype);
+#undef LAUNCH_ACT
+    ME_LAUNCH_CHECK();
+    return 0;
+  }
   ME_CHECK(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
            "skinny gemm: K=%d and the row strides must be multiples of 8", K);
   ME_CHECK((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0),
@@ -446,7 +485,7 @@ template <> struct Quad4<bf16_t> {
   }
 };
 
-template <typename TX, typename TO, bool EXACT_K>
+template <typename TX, typename TO, bool EXACT_K, bool ACT>
 __global__ void __launch_bounds__(256)
 gemm_skinny_norm_kernel(const TX* __restrict__ xp, int S, int64_t part_stride, const float* __restrict__ res_in,
                         float* __restrict__ res_out, const float* __restrict__ gamma, float eps,
@@ -460,9 +499,13 @@ gemm_skinny_norm_kernel(const TX* __restrict__ xp, int S, int64_t part_stride, c
   float* inv = ssw + 64;                                   // [16] 1 / rms
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * (ACT ? 8 : 16);
   const int total_steps = (K + 127) / 128;
-  const bf16_t* wrow = w + (int64_t)(n0 + r < N ? n0 + r : 0) * ldw;
+  const int half = N >> 1;                                 // ACT: as in gemm_skinny_kernel
+  int feature;
+  if (ACT) feature = n0 + (r & 7) < half ? (r < 8 ? n0 + r : half + n0 + r - 8) : 0;
+  else feature = n0 + r < N ? n0 + r : 0;
+  const bf16_t* wrow = w + (int64_t)feature * ldw;
   const bf16x8 z = gz8();
 
   auto fetch = [&](int s, bool live, bf16x8 (&a)[4]) {
@@ -562,8 +605,16 @@ gemm_skinny_norm_kernel(const TX* __restrict__ xp, int S, int64_t part_stride, c
 #pragma unroll
   for (int i = 0; i < 4; ++i) red[wave * 256 + r * 16 + 4 * g + i] = acc[i];
   __syncthreads();
-  {
-    const int idx = threadIdx.x;
+  const int idx = threadIdx.x;
+  if (ACT) {
+    const int m = idx >> 3, f = idx & 7;
+    if (idx < 128 && m < M && n0 + f < half) {
+      const int ig = m * 16 + f, iu = ig + 8;
+      const float gate = (red[ig] + red[256 + ig] + red[512 + ig] + red[768 + ig]) * inv[m];
+      const float up = (red[iu] + red[256 + iu] + red[512 + iu] + red[768 + iu]) * inv[m];
+      y[(int64_t)m * ldy + n0 + f] = from_f32<TO>(gate / (1.f + expf(-gate)) * up);
+    }
+  } else {
     const int m = idx >> 4, n = n0 + (idx & 15);
     if (m < M && n < N) {
       const float v = red[idx] + red[256 + idx] + red[512 + idx] + red[768 + idx];
@@ -573,10 +624,12 @@ gemm_skinny_norm_kernel(const TX* __restrict__ xp, int S, int64_t part_stride, c
 }
 
 // xp: bfloat16 or float32 [S, M, K] (S = 1: the rows themselves), contiguous; res_in float32 [M, K] or null;
-// res_out float32 [M, K] or null; gamma float32 [K]. y bfloat16 or float32 [M, N] with row stride ldy.
+// res_out float32 [M, K] or null; gamma float32 [K]. y bfloat16 or float32 with row stride ldy: [M, N], or with
+// act (w a packed gate/up weight, as in me_gemm_skinny_bf16) silu(gate) * up, [M, N / 2].
 extern "C" int me_gemm_skinny_norm_bf16(const void* xp, int x_dtype, int S, const float* res_in, float* res_out,
                                         const float* gamma, float eps, const void* w, int64_t ldw, void* y,
-                                        int64_t ldy, int out_dtype, int M, int N, int K, hipStream_t stream) {
+                                        int64_t ldy, int out_dtype, int M, int N, int K, int act,
+                                        hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   ME_CHECK(M <= NORM_MAX_ROWS, "norm + skinny gemm: at most %d rows (%d)", NORM_MAX_ROWS, M);
   ME_CHECK(S >= 1 && S <= NORM_MAX_PARTIALS, "norm + skinny gemm: %d partial sums outside 1..%d", S, NORM_MAX_PARTIALS);
@@ -584,22 +637,25 @@ extern "C" int me_gemm_skinny_norm_bf16(const void* xp, int x_dtype, int S, cons
   ME_CHECK(x_dtype == ME_F32 || (x_dtype == ME_BF16 && S == 1), "norm + skinny gemm: partial sums must be float32");
   for (const void* p : {xp, (const void*)res_in, (const void*)res_out, (const void*)gamma, w})
     ME_CHECK(reinterpret_cast<uintptr_t>(p) % 16 == 0, "norm + skinny gemm: operands must be 16-byte aligned");
-  ME_CHECK(xp && gamma && w && y && ldy >= N, "norm + skinny gemm: null operand or short output rows");
+  ME_CHECK(!act || N % 2 == 0, "norm + skinny gemm: a packed gate/up weight has an even number of rows (%d)", N);
+  ME_CHECK(xp && gamma && w && y && ldy >= (act ? N / 2 : N), "norm + skinny gemm: null operand or short output rows");
   const size_t lds = ((size_t)M * (K + 8) * sizeof(bf16_t) + 15) / 16 * 16 + (4 * 256 + 64 + 16) * sizeof(float);
   ME_CHECK(lds <= 64 * 1024, "norm + skinny gemm: %d rows of %d do not fit the workgroup's LDS", M, K);
-  dim3 grid((N + 15) / 16), block(256);
+  dim3 grid(act ? (N / 2 + 7) / 8 : (N + 15) / 16), block(256);
   const bool exact = K % 128 == 0;
   const int64_t part_stride = (int64_t)M * K;
-#define LAUNCH1(TX, TO, E)                                                                                   \
-  gemm_skinny_norm_kernel<TX, TO, E><<<grid, block, lds, stream>>>((const TX*)xp, S, part_stride, res_in,    \
+#define LAUNCH1(TX, TO, E, A)                                                                                \
+  gemm_skinny_norm_kernel<TX, TO, E, A><<<grid, block, lds, stream>>>((const TX*)xp, S, part_stride, res_in, \
       res_out, gamma, eps, (const bf16_t*)w, ldw, (TO*)y, ldy, M, N, K)
-#define LAUNCH3(TX, TO) do { if (exact) LAUNCH1(TX, TO, true); else LAUNCH1(TX, TO, false); } while (0)
+#define LAUNCH2(TX, TO, E) do { if (act) LAUNCH1(TX, TO, E, true); else LAUNCH1(TX, TO, E, false); } while (0)
+#define LAUNCH3(TX, TO) do { if (exact) LAUNCH2(TX, TO, true); else LAUNCH2(TX, TO, false); } while (0)
   if (x_dtype == ME_F32 && out_dtype == ME_BF16) LAUNCH3(float, bf16_t);
   else if (x_dtype == ME_BF16 && out_dtype == ME_BF16) LAUNCH3(bf16_t, bf16_t);
   else if (x_dtype == ME_F32 && out_dtype == ME_F32) LAUNCH3(float, float);
   else if (x_dtype == ME_BF16 && out_dtype == ME_F32) LAUNCH3(bf16_t, float);
   else ME_CHECK(false, "norm + skinny gemm: bad dtype codes %d -> %d", x_dtype, out_dtype);
 #undef LAUNCH3
+#undef LAUNCH2
 #undef LAUNCH1
   ME_LAUNCH_CHECK();
   return 0;

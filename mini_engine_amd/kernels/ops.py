@@ -62,9 +62,9 @@ _CORE_PROTOS = {
     "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
-    "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
+    "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
-    "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, P],
+    "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
@@ -445,26 +445,42 @@ class HipBackend:
         if ksplit > 1:
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
-                        ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, _stream())
+                        ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, 0, _stream())
             return parts
         if skinny_takes(M, N, K):
             y = new()
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
-                        _code(out_dtype), None, 1, M, N, K, 0, _stream())
+                        _code(out_dtype), None, 1, M, N, K, 0, 0, _stream())
             return y
         # many rows, or the head over a large vocabulary: the library product (float32 accumulation; the
         # float32 output form keeps the logits unrounded)
         return library_product(x, w, out_dtype, out=out)
 
+    def gated_linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """silu(x . w[:I]^T) * (x . w[I:]^T) for a packed gate/up weight w [2 I, K] (gate rows first), as one
+        launch: the product's workgroups pair each gate feature with its up feature when they merge their waves,
+        from the unrounded sums (the separate kernels round the product to bfloat16 first). For the few rows
+        `gated_linear_fuses` admits. Returns [M, I]. (reference layers/linear.py:29-45, layers/activation.py:5-7.)"""
+        _check(gated_linear_fuses(x, w), "gated_linear: bfloat16, few rows, see gated_linear_fuses")
+        M, K = x.shape
+        N = w.shape[0]
+        y = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
+        core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N // 2,
+                    ME_BF16, None, 1, M, N, K, 0, 1, _stream())
+        return y
+
     def norm_linear(self, x: torch.Tensor, residual: torch.Tensor | None, norm_weight: torch.Tensor, eps: float,
-                    w: torch.Tensor, out_dtype: torch.dtype | None = None, want_residual: bool = True):
+                    w: torch.Tensor, out_dtype: torch.dtype | None = None, want_residual: bool = True,
+                    gated: bool = False):
         """`rms_norm` and `linear` behind it as one launch, for the few rows `norm_linear_fuses` admits:
         r = x (+ residual), x being rows [M, K] or float32 partial sums [S, M, K]; y = (norm_weight * r
         rounded to bfloat16) . w^T, scaled by 1 / rms(r) in float32 (the scale is one number per row, so
         it is applied to the finished sums; the separate kernels round norm_weight * r / rms(r) instead:
-        the same relative rounding). Returns (y [M, N], r float32 [M, K] or None).
+        the same relative rounding). `gated`: w is a packed gate/up weight and y is silu(gate) * up, [M, N/2],
+        as in `gated_linear`. Returns (y [M, N], r float32 [M, K] or None).
         (reference layers/layernorm.py:11-24, layers/linear.py:25-26.)"""
         _check(norm_linear_fuses(x, w), "norm_linear: bfloat16 weights, few rows, see norm_linear_fuses")
+        _check(not gated or w.shape[0] % 2 == 0, "norm_linear: a packed gate/up weight has an even number of rows")
         S = x.shape[0] if x.dim() == 3 else 1
         M, K = x.shape[-2], x.shape[-1]
         N = w.shape[0]
@@ -474,11 +490,12 @@ class HipBackend:
             _check(residual.dtype == torch.float32 and residual.shape == (M, K) and residual.is_contiguous(),
                    "norm_linear: residual must be contiguous float32 [M, K]")
         out_dtype = out_dtype or w.dtype
-        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        cols = N // 2 if gated else N
+        y = torch.empty((M, cols), dtype=out_dtype, device=x.device)
         res_out = torch.empty((M, K), dtype=torch.float32, device=x.device) if want_residual else None
         core().call("me_gemm_skinny_norm_bf16", x.data_ptr(), _code(x.dtype), S, _ptr(residual), _ptr(res_out),
-                    norm_weight.data_ptr(), float(eps), w.data_ptr(), w.stride(0), y.data_ptr(), N, _code(out_dtype),
-                    M, N, K, _stream())
+                    norm_weight.data_ptr(), float(eps), w.data_ptr(), w.stride(0), y.data_ptr(), cols, _code(out_dtype),
+                    M, N, K, int(gated), _stream())
         return y, res_out
 
     def silu_mul_linear(self, gu: torch.Tensor, w: torch.Tensor, allow_partials: bool = False):
@@ -500,11 +517,11 @@ class HipBackend:
         if ksplit > 1:
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=gu.device)
             core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), None, N,
-                        ME_F32, parts.data_ptr(), ksplit, M, N, inter, 1, _stream())
+                        ME_F32, parts.data_ptr(), ksplit, M, N, inter, 1, 0, _stream())
             return parts
         y = torch.empty((M, N), dtype=gu.dtype, device=gu.device)
         core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
-                    ME_BF16, None, 1, M, N, inter, 1, _stream())
+                    ME_BF16, None, 1, M, N, inter, 1, 0, _stream())
         return y
 
     # -- sampling ------------------------------------------------------------------------
@@ -555,6 +572,8 @@ PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forc
 PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS wherever it fits (0: never)
 PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
+FUSE_GATE_INTO_GATE_UP = True  # False: silu(gate) * up is formed in front of the down product, not behind gate_up
+GATED_EPILOGUE_MAX_M = 16
 FUSE_NORM_INTO_LINEAR = True   # False: the norm kernel and the product behind it always run as two launches
 NORM_FUSE_MAX_M = 2
 NORM_FUSE_MAX_WEIGHT = 8 << 20
@@ -740,6 +759,24 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
     return part, parts
 
 
+def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
+    """Whether `rows` rows against the packed gate/up weight w [2 I, K] are few enough, and w of a kind, for the
+    gating to happen in the product's epilogue: a bfloat16 product that the unsplit skinny kernel takes, up to
+    GATED_EPILOGUE_MAX_M rows. At the 0.6B widths the gating in front of the down product costs every one of that
+    product's workgroups about 2 us; behind gate/up every gate is formed once."""
+    if not FUSE_GATE_INTO_GATE_UP or w.dtype != torch.bfloat16 or w.dim() != 2:
+        return False
+    N, K = w.shape
+    return (1 <= rows <= GATED_EPILOGUE_MAX_M and N % 2 == 0 and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0
+            and w.data_ptr() % 16 == 0 and skinny_takes(rows, N, K))
+
+
+def gated_linear_fuses(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether `gated_linear` takes rows x [M, K] and the packed gate/up weight w [2 I, K]."""
+    return (x.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1] and x.stride(1) == 1
+            and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and gated_linear_rows(x.shape[0], w))
+
+
 def norm_linear_fuses(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether `norm_linear` takes rows x ([M, K], or float32 partial sums [S, M, K]) and weight w: a
     bfloat16 weight that the unsplit skinny kernel would take, one or two rows, a weight of at most
@@ -808,4 +845,5 @@ def decode_step_attention(*a, **k): return backend().decode_step_attention(*a, *
 def linear(*a, **k): return backend().linear(*a, **k)
 def silu_mul_linear(*a, **k): return backend().silu_mul_linear(*a, **k)
 def norm_linear(*a, **k): return backend().norm_linear(*a, **k)
+def gated_linear(*a, **k): return backend().gated_linear(*a, **k)
 def sample(*a, **k): return backend().sample(*a, **k)

@@ -154,8 +154,9 @@ class Norm(Part):
         """
         raise NotImplementedError
 
-    # Optional: linear_behind(x, residual, weight, out_dtype) -> (forward(x, residual)[0] . weight^T, new
-    # residual), norm and product as one kernel, or None where there is no such kernel for these shapes.
+    # Optional: linear_behind(x, residual, weight, out_dtype, gated=False) -> (forward(x, residual)[0] . weight^T,
+    # new residual), norm and product as one kernel, or None where there is no such kernel for these shapes
+    # (gated: weight is a packed gate/up weight and the product is silu(gate) * up).
 
 
 class PendingNorm:
@@ -177,12 +178,13 @@ class PendingNorm:
             self._y, self._new_residual = self.norm.forward(x, self.residual)
         return self._y
 
-    def into_linear(self, weight: torch.Tensor, out_dtype=None):
-        """The product of the normed rows with `weight` ([out, in]) if the norm can run inside it, else None."""
+    def into_linear(self, weight: torch.Tensor, out_dtype=None, gated: bool = False):
+        """The product of the normed rows with `weight` ([out, in]) if the norm can run inside it, else None.
+        gated: `weight` is a packed gate/up weight and the product is silu(gate) * up."""
         behind = getattr(self.norm, "linear_behind", None)
         if self._y is not None or behind is None:
             return None
-        got = behind(self.x, self.residual, weight, out_dtype)
+        got = behind(self.x, self.residual, weight, out_dtype, gated) if gated else behind(self.x, self.residual, weight, out_dtype)
         if got is None:
             return None
         y, self._new_residual = got

@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 from ..kernels import ops
-from .base import FeedForward, register_part
+from .base import FeedForward, PendingNorm, register_part
 from .linear import Linear
 
 
@@ -22,5 +22,9 @@ class SwiGLU(FeedForward):
         self.add_child("down", Linear(intermediate_size, hidden_size))
 
     def forward(self, x):
+        rows = x.x.shape[-2] if isinstance(x, PendingNorm) else x.shape[0]
+        if ops.gated_linear_rows(rows, self.gate_up.weight):
+            # few rows: the gating in the gate/up product's epilogue (every gate formed once), a plain down product
+            return self.down.forward(self.gate_up.forward(x, gated=True), allow_partials=True)
         gu = self.gate_up.forward(x)
         return ops.silu_mul_linear(gu, self.down.weight, allow_partials=True)

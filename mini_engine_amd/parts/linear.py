@@ -18,13 +18,20 @@ class Linear(Part):
             raise ValueError("row blocks do not add up to out_features")
         self.add_param("weight", ParamSpec((out_features, in_features), init="matrix", dtype="compute"))
 
-    def forward(self, x, out_dtype=None, allow_partials: bool = False):
+    def forward(self, x, out_dtype=None, allow_partials: bool = False, gated: bool = False):
         """With allow_partials the result may be float32 partial sums [P, M, N] (a product whose K
         range was split over workgroups); the consumer, a norm, adds them. x may be a `PendingNorm`:
-        the norm then runs inside the product where there is a kernel for that, else in front of it."""
+        the norm then runs inside the product where there is a kernel for that, else in front of it.
+        gated: this is a packed gate/up map (gate's rows first) and the result is silu(gate) * up,
+        [M, out_features / 2] (reference layers/activation.py:5-7), from the product's own epilogue where
+        there is a kernel for that, else from the activation kernel behind it."""
         if isinstance(x, PendingNorm):
-            y = x.into_linear(self.weight, out_dtype)
+            y = x.into_linear(self.weight, out_dtype, gated)
             if y is not None:
                 return y
             x = x.value()
-        return ops.linear(x, self.weight, out_dtype, allow_partials)
+        if not gated:
+            return ops.linear(x, self.weight, out_dtype, allow_partials)
+        if ops.gated_linear_fuses(x, self.weight):
+            return ops.gated_linear(x, self.weight)
+        return ops.silu_and_mul(ops.linear(x, self.weight))

@@ -30,7 +30,7 @@ class RMSNorm(Norm):
     def forward(self, x, residual, want_residual: bool = True):
         return ops.rms_norm(x, self.weight, self.eps, residual, self.out_dtype, want_residual)
 
-    def linear_behind(self, x, residual, weight, out_dtype=None):
+    def linear_behind(self, x, residual, weight, out_dtype=None, gated: bool = False):
         if weight.dtype != self.out_dtype or not ops.norm_linear_fuses(x, weight):
             return None
-        return ops.norm_linear(x, residual, self.weight, self.eps, weight, out_dtype)
+        return ops.norm_linear(x, residual, self.weight, self.eps, weight, out_dtype, gated=gated)

@@ -127,13 +127,25 @@ def linear(x, w, out_dtype=None, allow_partials=False, out=None):
     return y
 
 
-def norm_linear(x, residual, norm_weight, eps, w, out_dtype=None, want_residual=True, compute_dtype=torch.float32):
+def _gate(y):
+    """silu(first half of the columns) * second half, on unrounded sums."""
+    inter = y.shape[1] // 2
+    return y[:, :inter] * torch.sigmoid(y[:, :inter]) * y[:, inter:]
+
+
+def gated_linear(x, w, compute_dtype=torch.float32):
+    return _gate(x.to(compute_dtype) @ w.to(compute_dtype).t()).to(x.dtype)
+
+
+def norm_linear(x, residual, norm_weight, eps, w, out_dtype=None, want_residual=True, gated=False, compute_dtype=torch.float32):
     """The fused kernel's rounding points: gamma * r to the weight's dtype, product, then 1 / rms(r)."""
     r = x.float().sum(0) if x.dim() == 3 else x.float()
     if residual is not None:
         r = r + residual
     inv = torch.rsqrt(r.to(compute_dtype).pow(2).mean(-1, keepdim=True) + eps)
     y = ((norm_weight * r).to(w.dtype).to(compute_dtype) @ w.to(compute_dtype).t()) * inv
+    if gated:
+        y = _gate(y)
     return y.to(out_dtype or w.dtype), (r if want_residual else None)
 
 
@@ -184,4 +196,5 @@ class PlainBackend:
     linear = staticmethod(linear)
     silu_mul_linear = staticmethod(silu_mul_linear)
     norm_linear = staticmethod(norm_linear)
+    gated_linear = staticmethod(gated_linear)
     sample = staticmethod(sample)

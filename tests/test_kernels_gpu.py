@@ -477,6 +477,30 @@ def test_norm_inside_the_skinny_product(M, N, K, S):
     close(y32, exact, 2e-5)
 
 
+@pytest.mark.parametrize("M", [1, 2, 5, 16])
+@pytest.mark.parametrize("I,K", [(3072, 1024), (224, 80), (100, 72), (1536, 4096)])
+def test_gating_in_the_gate_up_products_epilogue(M, I, K):
+    """silu(gate) * up formed where the packed gate/up product merges its waves (8 gate and 8 up features to a
+    workgroup), against the product in float64 and against the two kernels it stands for; and the same behind
+    an RMSNorm inside the product, for the one or two rows that takes."""
+    torch.manual_seed(M + I)
+    w = (torch.randn(2 * I, K, device=DEV) * 0.05).bfloat16()
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    assert ops.gated_linear_fuses(x, w) and not ops.gated_linear_fuses(torch.randn(17, K, device=DEV).bfloat16(), w)
+    got = hip().gated_linear(x, w)
+    assert got.shape == (M, I)
+    close(got, twin.gated_linear(x, w, compute_dtype=torch.float64), 6e-3)
+    close(got, hip().silu_and_mul(hip().linear(x, w)), 1.5e-2)         # those round the product before the gating
+    parts, res = torch.randn(3, M, K, device=DEV), torch.randn(M, K, device=DEV)
+    assert ops.norm_linear_fuses(parts, w) == (M <= 2 and 2 * I * K <= ops.NORM_FUSE_MAX_WEIGHT)
+    if ops.norm_linear_fuses(parts, w):
+        gamma = torch.rand(K, device=DEV) + 0.5
+        y, r = hip().norm_linear(parts, res, gamma, 1e-6, w, gated=True)
+        assert y.shape == (M, I)
+        want = twin.norm_linear(r, None, gamma, 1e-6, w, gated=True, out_dtype=torch.float64, compute_dtype=torch.float64)[0]
+        close(y, want, 6e-3)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40])
 @pytest.mark.parametrize("N,I", [(1024, 3072), (80, 224), (72, 200)])
 def test_silu_mul_linear(M, N, I):
