@@ -343,13 +343,14 @@ class HipBackend:
         if T > num_decodes:
             _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
             Tp = T - num_decodes
-            seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq, D)
+            col_tiles = prefill_col_tiles(max_prefill_context, win, Tp, Hq, D)
+            seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq, D, col_tiles)
             pf = torch.empty((Tp * Hq * max_segs * (D + 2),), dtype=torch.float32, device=q.device) if max_segs > 1 else None
             lib.call("me_attn_prefill", q.data_ptr() + num_decodes * q.stride(0) * es, q.stride(0),
                      out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
                      block_tables.stride(0), context_lens.data_ptr() + num_decodes * 4, prefill_cu.data_ptr(),
-                     B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, PREFILL_COL_TILES, PREFILL_THROUGH_LDS, seg_keys, max_segs,
+                     B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, col_tiles, PREFILL_THROUGH_LDS, seg_keys, max_segs,
                      _ptr(pf), seq_of_token.data_ptr() + num_decodes * 4, num_decodes, _stream())
         return out
 
@@ -570,7 +571,7 @@ LIBRARY_MAX_K = 16384
 ROWS_MIN_WEIGHT = 16 * 1024 * 1024
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 PREFILL_THROUGH_LDS = 1        # prefill attention, keys and values shared by a workgroup's waves through LDS wherever it fits (0: never)
-PREFILL_COL_TILES = 0     # 0: chosen by the launcher; 1 or 2 force the column tiles per wave
+PREFILL_COL_TILES = 0     # 0: chosen by prefill_col_tiles(); 1 or 2 force the column tiles per wave
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
 FUSE_GATE_INTO_GATE_UP = True  # False: silu(gate) * up is formed in front of the down product, not behind gate_up
 GATED_EPILOGUE_MAX_M = 16
@@ -605,7 +606,24 @@ def _scratch(num_floats: int, device) -> torch.Tensor:
     return buf
 
 
-def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D: int = 128) -> tuple:
+def prefill_col_tiles(max_context: int, window: int, num_tokens: int, Hq: int, D: int = 128) -> int:
+    """Column tiles (of 16 (token, head) pairs) per wave of the prefill kernel: 2 halves the reads of keys and
+    values per product but needs twice the columns per workgroup, so it is for launches with many columns (32,768
+    or more: 2,048 tokens of 16 heads), and for portions of 256 tokens or more of a prompt over 4,096 keys or
+    more, where each tile walks a long range and `prefill_segments` cuts that range into enough workgroups
+    (us at 16x128 heads, one tile / two: 512 tokens over 8,192 keys 96 / 65, over 16,384 172 / 120; 1,024 over
+    8,192 142 / 116; 256 over 32,768 176 / 128; 512 over 2,048 and 400 over 3,000 level: left at one).
+    PREFILL_COL_TILES forces it."""
+    if PREFILL_COL_TILES in (1, 2):
+        return PREFILL_COL_TILES
+    if D > 128:
+        return 1
+    cols = num_tokens * Hq
+    span = min(max_context, window + 256) if window else max_context
+    return 2 if cols >= 32768 or (cols >= 4096 and span >= 4096) else 1
+
+
+def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D: int = 128, col_tiles: int | None = None) -> tuple:
     """(keys per segment, most segments per tile) for the prefill kernel; (0, 1): no cutting.
 
     A tile's key range grows with its position, and a step with few new tokens over a long context
@@ -617,12 +635,28 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D:
     prompt: twice the workgroups fill the slots evenly); as many as give 768 workgroups below that.
     Measured at 16x128 heads (us, whole / cut): 64 tokens over 32,768 keys 1406 / 99, 1,024 over 4,096
     116 / 86, 2,048 over 8,192 333 / 237, one prompt of 4,096 tokens 166 / 135, of 2,048 86 / 56, of
-    1,536 52 / 43, of 1,024 36 / 33, 512 over 2,048 62 / 37. PREFILL_SEGMENT_KEYS forces a size."""
+    1,536 52 / 43, of 1,024 36 / 33, 512 over 2,048 62 / 37. A portion of a prompt that runs with two column
+    tiles per wave before its launch has 32,768 columns (`prefill_col_tiles`) gets segments of 512 to 1,024
+    keys, as many as give about 512 workgroups (512 tokens over 8,192 keys: segments of 512 / 1,024 / 1,376
+    keys 80 / 65 / 74 us; 256 over 8,192: 49 / 61 / 61; 1,024 over 4,096: 77 / 63 / 87).
+    PREFILL_SEGMENT_KEYS forces a size."""
     span = min(max_context, window + 256) if window else max_context
     if PREFILL_SEGMENT_KEYS is not None:
         seg = PREFILL_SEGMENT_KEYS
         return (seg, -(-span // seg) + 1) if seg > 0 and span > seg else (0, 1)
-    workgroups = max(1, num_tokens * Hq // (128 if num_tokens * Hq >= 32768 else 64))
+    cols = num_tokens * Hq
+    if col_tiles is None:
+        col_tiles = prefill_col_tiles(max_context, window, num_tokens, Hq, D)
+    most_by_memory = (1 << 28) // (cols * (D + 2) * 4) - 1      # the partial results are float32 [tokens, heads, segments + 1, D + 2]: under 256 MB
+    if col_tiles == 2 and cols < 32768:
+        tiles = -(-cols // 128)
+        seg = min(1024, max(512, -(-(-(-span // -(-512 // tiles))) // 32) * 32))
+        segs = min(-(-span // seg), most_by_memory)
+        if segs <= 1:
+            return 0, 1
+        seg = -(-(-(-span // segs)) // 32) * 32
+        return seg, -(-span // seg) + 1
+    workgroups = max(1, cols // (128 if col_tiles == 2 else 64))
     if workgroups > 640:
         segs = 1
     elif workgroups > 256:
@@ -632,8 +666,7 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D:
     else:
         segs = -(-768 // workgroups)
     segs = min(segs, span // (512 if span <= 4096 else 1024))      # segments of 512 keys or more, 1,024 over long ranges
-    # the partial results are float32 [tokens, heads, segments + 1, D + 2]: keep them under 256 MB
-    segs = min(segs, (1 << 28) // (num_tokens * Hq * (D + 2) * 4) - 1)
+    segs = min(segs, most_by_memory)
     if segs <= 1:
         return 0, 1
     seg = -(-(-(-span // segs)) // 32) * 32

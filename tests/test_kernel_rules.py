@@ -29,10 +29,17 @@ def test_prefill_segments_cover_the_span_and_hold_512_keys_or_more():
                                        (4096, 0, 1024, 16), (2048, 0, 512, 16)):
         seg, most = ops.prefill_segments(ctx, window, tokens, heads)
         span = min(ctx, window + 256) if window else ctx
-        assert seg >= (512 if span <= 4096 else 1024) and seg % 32 == 0 and (most - 1) * seg >= span
+        wide_portion = ops.prefill_col_tiles(ctx, window, tokens, heads) == 2 and tokens * heads < 32768
+        assert seg >= (512 if span <= 4096 or wide_portion else 1024) and seg % 32 == 0 and (most - 1) * seg >= span
         assert tokens * heads * most * 130 * 4 <= 1 << 28
     assert ops.prefill_segments(2048, 0, 2048, 16)[0] == 704          # a prompt from its beginning: thirds
-    assert ops.prefill_segments(4096, 0, 1024, 16)[0] == 2048         # a later portion, all ranges long: halves
+    # a later portion over a long context runs with two column tiles per wave and segments of 512-1,024 keys that give
+    # about 512 workgroups; a short context, or few tokens, stays with one column tile
+    assert ops.prefill_col_tiles(4096, 0, 1024, 16) == 2 and ops.prefill_segments(4096, 0, 1024, 16)[0] == 1024
+    assert ops.prefill_col_tiles(8192, 0, 256, 16) == 2 and ops.prefill_segments(8192, 0, 256, 16)[0] == 512
+    assert ops.prefill_col_tiles(2048, 0, 512, 16) == 1 and ops.prefill_col_tiles(8192, 0, 128, 16) == 1
+    assert ops.prefill_col_tiles(8192, 0, 2048, 16) == 2 and ops.prefill_segments(8192, 0, 2048, 16)[0] == 4096
+    assert ops.prefill_col_tiles(8192, 0, 512, 2, D=256) == 1          # head sizes beyond 128: one column tile
     assert ops.prefill_segments(8192, 512, 64, 16) == (0, 1)          # a window bounds the span
     assert ops.prefill_segments(1 << 20, 0, 8192, 64)[1] <= 3         # the partial results stay under 256 MB
 
