@@ -800,8 +800,13 @@ def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     if not FUSE_GATE_INTO_GATE_UP or w.dtype != torch.bfloat16 or w.dim() != 2:
         return False
     N, K = w.shape
+    # over large weights the library takes products of 4 rows or more, and the gating is then a kernel of its own;
+    # up to 8 rows over a K of 4,096 the skinny kernel with the gating in its epilogue is still ahead of the two
+    # (4096 -> 24576, us: 4 rows 38.9 / 45.5, 6 rows 41.4 / 45.6, 8 rows 43.9 / 45.5, 12 rows 49.2 / 46.2; over a K of
+    # 5,120 the library is level or ahead from 4 rows on: 5120 -> 34816, 4 rows 75.0 / 76.4, 6 rows 81.2 / 76.5)
+    takes = skinny_takes(rows, N, K) or (rows <= 8 and K <= 4096 and N < LIBRARY_MIN_N and rows <= SKINNY_MAX_M)
     return (1 <= rows <= GATED_EPILOGUE_MAX_M and N % 2 == 0 and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0
-            and w.data_ptr() % 16 == 0 and skinny_takes(rows, N, K))
+            and w.data_ptr() % 16 == 0 and takes)
 
 
 def gated_linear_fuses(x: torch.Tensor, w: torch.Tensor) -> bool:
