@@ -584,7 +584,6 @@ FUSE_DECODE_STEP = True        # False: pure decode steps run norm/rotation/cach
 # 27 us for the plain product after a separate gating kernel (3 us).
 GATED_MAX_K = 4096
 GATED_MAX_M = 16
-_TARGET_WORKGROUPS = 512
 _COMPUTE_UNITS = 256
 _DECODE_WORKGROUPS = 4096
 _DECODE_WHOLE_WORKGROUPS = 768
@@ -741,19 +740,29 @@ def library_streams_better(M: int, N: int, K: int) -> bool:
 
 
 def choose_ksplit(M: int, N: int, K: int) -> int:
-    """Workgroups over K for a skinny product: 1 when the N/16 feature tiles already fill the
-    compute units, else enough to reach the target, each split keeping >= 512 of K."""
+    """Workgroups over K for a skinny product whose consumer adds float32 partial sums (1: K is not split).
+
+    A product's time goes with the rounds its workgroups make over the 256 compute units, each round as long as
+    a workgroup's share of K: rounds(tiles x splits) / splits, plus a little for every further set of partial sums
+    that the consumer reads. The split with the least of that is taken, each split keeping 512 of K or more (4
+    steps of 128, one per wave); with 256 feature tiles or more only over a K of 4,096 or more, where an uneven
+    count (320 tiles: one round and a quarter) costs a quarter of the stream, and only up to 32 rows (beyond, the
+    library is level or ahead). Measured, product + norm in us by splits 1 / 2 / 3 / 4 / 6 / 8, one row:
+      1024 x 2048 (64 tiles):    6.8 / 5.6 / 5.5 / 5.3 / 5.7 / 5.6      1024 x 3072:  8.1 / 6.4 / 5.9 / 5.9 / 6.1 / 6.0
+      2048 x 6144 (128 tiles):   11.7 / 9.0 / 10.9 / 10.2 / 9.2 / 9.5   2560 x 9728 (160): 16.1 / 17.9 / 14.4 / 15.7 / 15.8 / 15.2
+      4096 x 12288 (256 tiles):  23.9 / 24.6 / 25.6 / 24.9 / 24.9 / 28.4
+      5120 x 8192 (320 tiles):   29.1 / 24.0 / 22.7 / 22.2 / 24.1 / 23.8   5120 x 25600: 73.3 / 60.4 / 56.8 / 52.1 / 54.4 / 53.7"""
     tiles = -(-N // 16) * -(-M // 64)
-    if tiles >= _TARGET_WORKGROUPS // 2:
-        # enough workgroups; but a count that leaves the 256 compute units unevenly loaded (320 feature
-        # tiles: one each and a quarter of them a second) over a long K streams a quarter slower than
-        # four times as many workgroups that come out even (5120 x 8192: 25.6 -> 18.7 us, 5120 x 25600: 70.8 -> 52.2 us;
-        # up to 32 rows: beyond, the library is level or ahead)
-        if tiles % _COMPUTE_UNITS and tiles < 4 * _COMPUTE_UNITS and K >= 4096 and M <= SKINNY_MAX_M:
-            return 4
+    if tiles >= _COMPUTE_UNITS and (K < 4096 or M > SKINNY_MAX_M):
         return 1
-    # each split keeps 4 steps of 128 or more, one per wave (2048 in 4 splits: product + norm 5.9 us, in 8: 6.3 us)
-    return max(1, min(-(-_TARGET_WORKGROUPS // tiles), K // 512, 8))
+    best, least = 1, None
+    for splits in range(1, 9):
+        if splits > 1 and K // splits < 512:
+            break
+        cost = -(-tiles * splits // _COMPUTE_UNITS) / splits + 0.02 * splits
+        if least is None or cost < least - 1e-9:
+            best, least = splits, cost
+    return best
 
 
 def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: bool = False) -> tuple:
