@@ -358,21 +358,27 @@ __device__ __forceinline__ void block_softmax(const AttnArgs& a, const f32x4 (&s
       sv[i] = (j <= col_hi && j >= col_lo) ? sv[i] : NEG;
     }
   }
+  // The reference point m of a column is shared by its four lanes and moves only when some score of the block
+  // lies more than RESCALE_STEP above it. Every lane tests its own 8 scores; only when one of the wave finds such
+  // a score is the column's maximum formed across the lanes (the common block needs no exchange between lanes).
   float bm = NEG;
 #pragma unroll
   for (int i = 0; i < 8; ++i) bm = fmaxf(bm, sv[i]);
-  bm = max_over_groups(bm);
-  const float m_blk = bm > 0.5f * NEG ? bm * c : NEG;
-  const bool rose = m_blk > m + RESCALE_STEP;
-  if (__any(rose)) {
-    const float m_new = rose ? m_blk : m;
-    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-    l *= alpha;
+  if (__any(bm > 0.5f * NEG && bm * c > m + RESCALE_STEP)) {
+    bm = max_over_groups(bm);
+    const float m_blk = bm > 0.5f * NEG ? bm * c : NEG;
+    // A branch of the lanes, not of the wave: the lanes that stay out keep their values, so the accumulators are
+    // scaled in the registers they are in (written as a choice per wave, the rescaled values get registers of their
+    // own and every accumulator is copied in every block that does not rescale).
+    if (m_blk > m + RESCALE_STEP) {
+      const float alpha = __builtin_amdgcn_exp2f(m - m_blk);
+      l *= alpha;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      acc[dt][0] *= alpha; acc[dt][1] *= alpha; acc[dt][2] *= alpha; acc[dt][3] *= alpha;
+      for (int dt = 0; dt < DT; ++dt) {
+        acc[dt][0] *= alpha; acc[dt][1] *= alpha; acc[dt][2] *= alpha; acc[dt][3] *= alpha;
+      }
+      m = m_blk;
     }
-    m = m_new;
   }
   float psum = 0.f;
 #pragma unroll
@@ -856,6 +862,315 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 }
 
+#if ME_HEAD_DIM == 128
+// =====================================================================================
+// Prefill / chunk kernel, keys and values brought into LDS by the memory system itself
+// (global_load_lds_dwordx4: every lane names 16 bytes of memory, and the 64 pieces of a wave's
+// instruction land in 1 KB of consecutive LDS), head size 128, pages of 16 keys or more, no window.
+// Against the form above this takes the staged block out of the registers and the LDS writes out of
+// the instruction stream, and lets a block be asked for NB - 1 blocks before its use instead of one:
+// in the form above an iteration cannot be shorter than the latency of its loads, which at two
+// workgroups per compute unit is what bounds it (1.8 us a block measured, where its matrix and vector
+// instructions account for 0.6).
+//   keys    8 instructions of 4 key rows (4 x 256 B); instruction i = 4 tt + (n >> 2) holds the rows
+//           tt * 16 + n of the operand order (see the top of the file), i.e. the 4 consecutive keys
+//           8 (i & 3) + 4 (i >> 2) + 0..3 of the block, and starts at i * (1 KB + 64 B); inside a row
+//           the 16-byte piece c lies at position c ^ (row & 3). A read of 16 rows n at one piece then
+//           touches 16 different bank groups (the padding separates the instructions, the exchange
+//           the rows inside one), and the exchange leaves 4 ks + (g ^ (n & 3)): the pieces of the
+//           four ks steps stay 64 bytes apart.
+//   values  [2 halves of 16 keys][128 channels][32 B]: an instruction is 32 channel rows of one half,
+//           so with pages of 16 keys it reads one page; piece (g & 1) of a row lies at (g & 1) ^ (channel >> 3 & 1).
+// A block that reaches beyond the context (the last one of a sequence) is loaded into registers,
+// zeroed where it must not be used, and written to the same places.
+// =====================================================================================
+#define DMA_KINST 1088
+#define DMA_KBYTES (8 * DMA_KINST)
+#define DMA_VHALF 4096
+#define DMA_BUF (DMA_KBYTES + 2 * DMA_VHALF)
+#define DMA_NB 3                       // buffers: three workgroups of a compute unit hold 3 x 3 x 16.5 KB of its 160 KB
+
+// 64 x 16 bytes from gbase + voff (bytes, per lane) to LDS at lds_addr + 16 * lane. The write to m0 needs one wait
+// state before an instruction that reads it for an LDS address.
+__device__ __forceinline__ void dma16(const bf16_t* gbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+// Keeps the reads of a whole operand array where they are written: without it the compiler moves every read
+// down to the product that uses it and waits for each in turn.
+template <int N>
+__device__ __forceinline__ void pin_operands(bf16x8 (&x)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(x[i]));
+}
+template <int N, int M>
+__device__ __forceinline__ void pin_operands(bf16x8 (&x)[N][M]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i)
+#pragma unroll
+    for (int j = 0; j < M; ++j) asm volatile("" : "+v"(x[i][j]));
+}
+
+// Reads of 16 bytes at addr + 512 i that the compiler does not know to be reads: it neither moves them to their
+// use nor waits for them, so lds_reads_done() has to stand between them and the first use of what they return.
+template <int I>
+__device__ __forceinline__ void lds_read16_ahead(uint32_t addr, bf16x8 (&x)[DT]) {
+  if constexpr (I < DT) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(x[I]) : "v"(addr), "n"(512 * I));
+    lds_read16_ahead<I + 1>(addr, x);
+  }
+}
+__device__ __forceinline__ void lds_reads_done(bf16x8 (&x)[DT]) {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  pin_operands(x);
+}
+
+struct DmaPages { int k, v; };   // the page of this wave's two key instructions and of its two value instructions
+
+template <int CT, int W>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))) attn_prefill_dma_kernel(AttnArgs a) {
+  extern __shared__ __align__(16) unsigned char pf_lds[];   // [NB][DMA_BUF]
+  constexpr int NB = DMA_NB, PD = NB - 1;                   // PD: blocks asked for ahead of the one in use
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g = lane >> 4;
+  const int kvh = blockIdx.x % a.Hkv;
+  const int x = gridDim.x / a.Hkv - 1 - blockIdx.x / a.Hkv;
+  int lo_b = 0, hi_b = a.num_seqs - 1;
+  while (lo_b < hi_b) {
+    const int mid = (lo_b + hi_b + 1) >> 1;
+    if (a.cu_seqlens[mid] / a.tok_tile + mid <= x) lo_b = mid; else hi_b = mid - 1;
+  }
+  const int b = lo_b;
+  const int q0 = a.cu_seqlens[b], q_len = a.cu_seqlens[b + 1] - q0;
+  const int tok0 = (x - (q0 / a.tok_tile + b)) * a.tok_tile;
+  if (tok0 >= q_len) return;
+  const int L = a.context_lens[b];
+  const int start = L - q_len;
+  // The table is read through the constant address space: entries are the same for every lane, and only from
+  // there does the compiler fetch them with scalar loads, which count apart from the loads into LDS (a vector
+  // load would be waited for together with every block on its way).
+  typedef const __attribute__((address_space(4))) int32_t* table_ptr;
+  const table_ptr bt = (table_ptr)(uintptr_t)(a.block_tables + (int64_t)b * a.bt_stride);
+  const TileRange tr = tile_range(a, tok0, q_len, L);
+  const int ncols = tr.tile_tokens * a.G;
+  const int seg = blockIdx.z;
+  if (seg >= tr.nseg) return;
+  const int seg_lo = a.seg_keys > 0 ? tr.tile_base + seg * a.seg_keys : tr.tile_base;
+  const int seg_hi = (a.seg_keys > 0 && seg + 1 < tr.nseg) ? seg_lo + a.seg_keys : (1 << 30);
+  const int last = min(tr.pos_last, seg_hi - 1);   // the same key range for every wave of the workgroup
+  const int nblk = (last - seg_lo) / 32 + 1;
+
+  const uint32_t lds0 = (uint32_t)(uintptr_t)pf_lds;
+  // what a lane names in memory, relative to its instruction's first byte, and where it reads its operands
+  const uint32_t voff_k = (lane >> 4) * 256 + (((lane & 15) ^ (lane >> 4)) * 16);
+  const uint32_t voff_v = ((lane >> 1) * a.page + (((lane & 1) ^ ((lane >> 4) & 1)) * 8)) * 2;
+  const uint32_t rd_k = (n >> 2) * DMA_KINST + (n & 3) * 256 + ((g ^ (n & 3)) * 16);
+  const uint32_t rd_v = DMA_KBYTES + (g >> 1) * DMA_VHALF + n * 32 + (((g & 1) ^ (n >> 3)) * 16);
+  const int kg0 = 8 * ((2 * wave) & 3) + 4 * (wave >> 1);   // first key of this wave's first key instruction; the second: + 8
+  const int vh = wave >> 1, vrow0 = 64 * (wave & 1);        // this wave's value instructions: half vh, channel rows vrow0 + 32 j
+  const uint32_t page_elems = (uint32_t)(a.Hkv * a.page * HD);                 // elements of a page, keys and values alike
+  const bf16_t* k_head = a.k_cache + (int64_t)kvh * a.page * HD;
+  const bf16_t* v_head = a.v_cache + ((int64_t)kvh * HD + vrow0) * a.page;
+
+  // table entries of the block at t0, asked for one block before they are used
+  auto lookup = [&](int t0) -> DmaPages {
+    DmaPages pg;
+    pg.k = t0 + kg0 < L ? bt[(t0 + kg0) >> a.page_shift] : 0;
+    pg.v = t0 + 16 * vh < L ? bt[(t0 + 16 * vh) >> a.page_shift] : 0;
+    return pg;
+  };
+  auto stage = [&](int t0, const DmaPages& pg, int bi) {
+    const uint32_t buf = bi * DMA_BUF;
+    const int krow = t0 + kg0 < L ? ((t0 + kg0) & (a.page - 1)) : 0;
+    const int vkey = t0 + 16 * vh < L ? ((t0 + 16 * vh) & (a.page - 1)) : 0;
+    const bf16_t* gk = k_head + (uint64_t)(uint32_t)pg.k * page_elems + krow * HD;
+    const bf16_t* gv = v_head + (uint64_t)(uint32_t)pg.v * page_elems + vkey;
+    if (t0 + 32 <= L) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) dma16(gk + 8 * j * HD, voff_k, lds0 + buf + (2 * wave + j) * DMA_KINST);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        dma16(gv + (int64_t)32 * j * a.page, voff_v, lds0 + buf + DMA_KBYTES + vh * DMA_VHALF + (vrow0 / 32 + j) * 1024);
+    } else {
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      const bf16x8 z = zero8();
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int key = t0 + kg0 + 8 * j + (lane >> 4);
+        // rows of a page that is held may be read beyond the context; without a page, page 0 is read
+        const bool held = t0 + kg0 + 8 * j < L;
+        const bf16_t* src = held ? gk + 8 * j * HD : k_head;
+        const bf16x8 kk = ld8(reinterpret_cast<const bf16_t*>(reinterpret_cast<const unsigned char*>(src) + voff_k));
+        *reinterpret_cast<bf16x8*>(pf_lds + buf + (2 * wave + j) * DMA_KINST + 16 * lane) = key < L ? kk : z;
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int key0 = t0 + 16 * vh + 8 * ((lane & 1) ^ ((lane >> 4) & 1));
+        const int nv = L - key0;
+        const bf16x8 vv = ld8(reinterpret_cast<const bf16_t*>(reinterpret_cast<const unsigned char*>(gv + (int64_t)32 * j * a.page) + voff_v));
+        u32x4 w = __builtin_bit_cast(u32x4, vv);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] &= (2 * i < nv ? 0x0000ffffu : 0u) | (2 * i + 1 < nv ? 0xffff0000u : 0u);
+        *reinterpret_cast<u32x4*>(pf_lds + buf + DMA_KBYTES + vh * DMA_VHALF + (vrow0 / 32 + j) * 1024 + 16 * lane) = w;
+      }
+    }
+  };
+
+  // every wave runs every round (a wave without columns in a round masks everything and writes nothing)
+  for (int c_base = 0; c_base < ncols; c_base += 4 * 16 * CT) {
+    const bool active = c_base + wave * 16 * CT < ncols;
+    const int c0 = active ? c_base + wave * 16 * CT : 0;
+    bf16x8 qb[CT][KS];
+    int col_lo[CT], col_hi[CT];
+    int64_t tq[CT];
+    int head[CT];
+    bool valid[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int cc = c0 + 16 * ct + n;
+      valid[ct] = active && cc < ncols;
+      const int tl = valid[ct] ? cc / a.G : 0;
+      const int hh = valid[ct] ? cc - tl * a.G : 0;
+      tq[ct] = q0 + tok0 + tl;
+      head[ct] = kvh * a.G + hh;
+      const int pos = start + tok0 + tl;
+      col_hi[ct] = valid[ct] ? pos : -1;
+      col_lo[ct] = 0;
+      load_q(a.q + tq[ct] * a.q_stride + (int64_t)head[ct] * HD, valid[ct], g, qb[ct]);
+    }
+    const int pos_first = start + tok0 + c0 / a.G;
+    const int full_hi = active ? pos_first - 31 : -(1 << 30);
+    float m[CT], l[CT];
+    f32x4 acc[CT][DT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      m[ct] = NEG; l[ct] = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    pf_barrier();                                    // the round before has finished with every buffer
+    DmaPages pg = lookup(seg_lo);
+#pragma unroll
+    for (int k = 0; k < PD; ++k) {
+      if (k < nblk) {
+        const DmaPages now = pg;
+        pg = lookup(seg_lo + 32 * (k + 1));
+        stage(seg_lo + 32 * k, now, k);
+      }
+    }
+    int cur = 0;
+    // One block: the wait for it, the request for the block PD further on, scores, softmax, values. FULL: every key
+    // of the block is visible to every column of this wave. Blocks are walked in ascending order, so a wave's FULL
+    // blocks come first and form a loop of their own (with both forms of the softmax in one loop body the compiler
+    // copies all accumulators in every iteration); every wave passes the same barriers in either loop.
+    auto block_step = [&](auto full_tag, int k) {
+      constexpr bool FULL = decltype(full_tag)::value;
+      const int t0 = seg_lo + 32 * k;
+      // block k has landed: at most the PD - 1 blocks asked for after it are still on their way
+      if (k + PD <= nblk) dma_wait<4 * (PD - 1)>(); else dma_wait<0>();
+      pf_barrier();                                  // ... for every wave, and buffer cur - 1 is free
+      if (k + PD < nblk) {
+        const DmaPages now = pg;
+        pg = lookup(t0 + 32 * (PD + 1));
+        stage(t0 + 32 * PD, now, cur == 0 ? NB - 1 : cur - 1);
+      }
+      const unsigned char* kb = pf_lds + cur * DMA_BUF + rd_k;
+      f32x4 st[CT][2];
+      bf16x8 pb[CT];
+      if constexpr (W == 2) {
+        // With 256 registers to a wave all of a block's key operands are asked for before the first score product,
+        // and its value operands before the softmax, which takes longer than they do: one LDS latency for each,
+        // not one for every pair of reads.
+        bf16x8 ka[2][KS];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            ka[tt][ks] = *reinterpret_cast<const bf16x8*>(kb + tt * 4 * DMA_KINST + 64 * ks);
+        pin_operands(ka);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+              st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[tt][ks], qb[ct][ks], st[ct][tt], 0, 0, 0);
+        }
+        bf16x8 va[DT];
+        lds_read16_ahead<0>(lds0 + cur * DMA_BUF + rd_v, va);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          block_softmax<FULL>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+        lds_reads_done(va);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt], pb[ct], acc[ct][dt], 0, 0, 0);
+      } else {
+        // With 168 registers the operands are read where they are used, and the third wave fills the waits.
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kb + tt * 4 * DMA_KINST + 64 * ks);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+              st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[ct][ks], st[ct][tt], 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          block_softmax<FULL>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+        const unsigned char* vb = pf_lds + cur * DMA_BUF + rd_v;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const bf16x8 va = *reinterpret_cast<const bf16x8*>(vb + 512 * dt);
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[ct], acc[ct][dt], 0, 0, 0);
+        }
+      }
+      cur = cur == NB - 1 ? 0 : cur + 1;
+    };
+    const int nfull = full_hi >= seg_lo ? min(nblk, (full_hi - seg_lo) / 32 + 1) : 0;
+    int k = 0;
+    for (; k < nfull; ++k) block_step(std::true_type{}, k);
+    for (; k < nblk; ++k) block_step(std::false_type{}, k);
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const float ls = column_sum(l[ct]);
+      if (valid[ct] && tr.nseg > 1) {
+        float* p = a.pf_scratch + (((int64_t)tq[ct] * a.Hq + head[ct]) * a.max_segs + seg) * (HD + 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          *reinterpret_cast<f32x4*>(p + 16 * dt + 4 * g) = acc[ct][dt];
+        if (g == 0) { p[HD] = m[ct]; p[HD + 1] = ls; }
+      } else if (valid[ct]) {
+        const float inv = ls > 0.f ? 1.f / ls : 0.f;
+        bf16_t* o = a.out + tq[ct] * a.out_stride + (int64_t)head[ct] * HD + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          bf16x4 r;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) r[i] = static_cast<bf16_t>(acc[ct][dt][i] * inv);
+          *reinterpret_cast<bf16x4*>(o + 16 * dt) = r;
+        }
+      }
+    }
+  }
+}
+#endif  // ME_HEAD_DIM == 128
+
 // Merge of the segments of cut tiles: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s.
 // Sixteen lanes per (token, head), each with HD/16 consecutive values; 16 rows to a workgroup. Rows of
 // tiles that were not cut already hold their result and return.
@@ -1234,6 +1549,18 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   // per CU its waves have no others to fill their waits at the barriers).
   // shared: 0 never, otherwise wherever it fits.
   const bool through_lds = 2 * PF_BUF <= 65536 && shared != 0;
+#if ME_HEAD_DIM == 128
+  // shared: 1 the memory system fills LDS where the kernel for that applies, 2 always through registers.
+  // Three waves to a SIMD where there are workgroups enough for three to a compute unit (8,192 tokens of one prompt:
+  // 321 against 356 us; 32,768: 3.83 against 4.20 ms), two with more registers each below that (512 tokens over
+  // 8,192 keys: 56 against 64 us).
+  if (through_lds && shared == 1 && window == 0 && page >= 16) {
+    const bool three = ct == 2 && tiles * Hkv >= 1024;
+    if (three) attn_prefill_dma_kernel<2, 3><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
+    else if (ct == 2) attn_prefill_dma_kernel<2, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
+    else attn_prefill_dma_kernel<1, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
+  } else
+#endif
   if (through_lds) {
     if (ct == 2) attn_prefill_shared_kernel<2><<<grid, dim3(256), 2 * PF_BUF, stream>>>(a);
     else attn_prefill_shared_kernel<1><<<grid, dim3(256), 2 * PF_BUF, stream>>>(a);

@@ -395,6 +395,33 @@ def test_attention_prefill_cut_into_segments(prefill_form, monkeypatch, seg_keys
         close(hip().paged_attention(*args, max_prefill_context=bound), twin.paged_attention(*args), 1.5e-2)
 
 
+@pytest.mark.parametrize("Hq,Hkv,page", [(16, 8, 16), (64, 8, 16), (2, 2, 64), (40, 8, 256)])
+def test_attention_prefill_lds_filled_by_the_loads_themselves(monkeypatch, Hq, Hkv, page):
+    """Head size 128, pages of 16 keys or more, no window: the loads write LDS directly, three buffers deep. Same
+    products in the same order as the form that stages through registers, so the results are equal bit for bit;
+    against the twin as everywhere. Contexts that end inside a block and inside a page (the cache holds NaN
+    wherever no key was written), one block, fewer blocks than buffers, segments, and a launch large enough for three waves
+    to a SIMD."""
+    seqs = [(5, 5), (31, 31), (32, 32), (33, 33), (64, 2), (65, 33), (97, 96), (129, 17), (page + 1, 2), (700, 700), (1000, 64)]
+    for seg_keys, peak in ((None, None), (96, 450), (256, 3)):
+        monkeypatch.setattr(ops, "PREFILL_SEGMENT_KEYS", seg_keys)
+        args = _attention_case(torch.bfloat16, Hq, Hkv, 128, page, seqs, seed=page + Hq, peak=peak)
+        monkeypatch.setattr(ops, "PREFILL_THROUGH_LDS", 1)
+        direct = hip().paged_attention(*args, max_prefill_context=1000)
+        monkeypatch.setattr(ops, "PREFILL_THROUGH_LDS", 2)
+        staged = hip().paged_attention(*args, max_prefill_context=1000)
+        assert not torch.isnan(direct).any() and torch.equal(direct, staged)
+        close(direct, twin.paged_attention(*args), 1.5e-2)
+    if Hq == 64:      # 16 tokens to a tile: 2,100 tokens are 132 tiles x 8 kv heads, beyond the 1,024 workgroups
+        monkeypatch.setattr(ops, "PREFILL_SEGMENT_KEYS", None)
+        args = _attention_case(torch.bfloat16, Hq, Hkv, 128, page, [(2100, 2100)], seed=7, peak=1500)
+        monkeypatch.setattr(ops, "PREFILL_THROUGH_LDS", 1)
+        direct = hip().paged_attention(*args, max_prefill_context=2100)
+        monkeypatch.setattr(ops, "PREFILL_THROUGH_LDS", 2)
+        assert torch.equal(direct, hip().paged_attention(*args, max_prefill_context=2100))
+        close(direct, twin.paged_attention(*args), 1.5e-2)
+
+
 def test_attention_prefill_segments_chosen_automatically():
     """A short chunk at the end of a long context is cut by the engine's own rule."""
     seqs = [(2500, 33), (1100, 2)]
