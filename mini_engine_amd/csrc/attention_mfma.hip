@@ -892,8 +892,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 // 64 x 16 bytes from gbase + voff (bytes, per lane) to LDS at lds_addr + 16 * lane. The write to m0 needs one wait
 // state before an instruction that reads it for an LDS address.
+// gbase and lds_addr are the same in every lane; the first lane's values are taken so that they lie in scalar
+// registers whatever the compiler has concluded about them.
 __device__ __forceinline__ void dma16(const bf16_t* gbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "memory");
+  const uint64_t g = reinterpret_cast<uint64_t>(gbase);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32)), lo = __builtin_amdgcn_readfirstlane((uint32_t)g);
+  const uint64_t base = (uint64_t)hi << 32 | lo;      // (the builtin returns int: widened as it is, a low half with its top bit set would fill the high half)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(base) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -1554,8 +1559,10 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   // Three waves to a SIMD where there are workgroups enough for three to a compute unit (8,192 tokens of one prompt:
   // 321 against 356 us; 32,768: 3.83 against 4.20 ms), two with more registers each below that (512 tokens over
   // 8,192 keys: 56 against 64 us).
-  if (through_lds && shared == 1 && window == 0 && page >= 16) {
-    const bool three = ct == 2 && tiles * Hkv >= 1024;
+  // (4 and 5: as 1 with two or three waves whatever the size, for measurements.)
+  if (through_lds && (shared == 1 || shared == 4 || shared == 5) && window == 0 && page >= 16 &&
+      (int64_t)Hkv * page * HD < (1ll << 31)) {
+    const bool three = ct == 2 && (shared == 5 || (shared == 1 && tiles * Hkv >= 1024));
     if (three) attn_prefill_dma_kernel<2, 3><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else if (ct == 2) attn_prefill_dma_kernel<2, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else attn_prefill_dma_kernel<1, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
