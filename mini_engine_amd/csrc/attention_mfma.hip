@@ -1556,13 +1556,15 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   const bool through_lds = 2 * PF_BUF <= 65536 && shared != 0;
 #if ME_HEAD_DIM == 128
   // shared: 1 the memory system fills LDS where the kernel for that applies, 2 always through registers.
-  // Three waves to a SIMD where there are workgroups enough for three to a compute unit (8,192 tokens of one prompt:
-  // 321 against 356 us; 32,768: 3.83 against 4.20 ms), two with more registers each below that (512 tokens over
-  // 8,192 keys: 56 against 64 us).
+  // Three waves to a SIMD where there are workgroups enough for three to a compute unit and the tiles are left
+  // whole, i.e. large launches that start at a prompt's beginning (8,192 tokens of one prompt, 16 query heads: 321
+  // against 356 us, 32 heads 524 against 597, 64 heads 998 against 1,069; 32,768 tokens: 3.83 against 4.20 ms), two
+  // with more registers each otherwise (512 tokens over 8,192 keys: 56 against 64 us; 2,048 tokens over 8,192 keys
+  // at 64 query heads, cut in segments: 475 against 533 us).
   // (4 and 5: as 1 with two or three waves whatever the size, for measurements.)
   if (through_lds && (shared == 1 || shared == 4 || shared == 5) && window == 0 && page >= 16 &&
       (int64_t)Hkv * page * HD < (1ll << 31)) {
-    const bool three = ct == 2 && (shared == 5 || (shared == 1 && tiles * Hkv >= 1024));
+    const bool three = ct == 2 && (shared == 5 || (shared == 1 && tiles * Hkv >= 1024 && a.max_segs == 1));
     if (three) attn_prefill_dma_kernel<2, 3><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else if (ct == 2) attn_prefill_dma_kernel<2, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else attn_prefill_dma_kernel<1, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
