@@ -1561,10 +1561,8 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   // against 356 us, 32 heads 524 against 597, 64 heads 998 against 1,069; 32,768 tokens: 3.83 against 4.20 ms), two
   // with more registers each otherwise (512 tokens over 8,192 keys: 56 against 64 us; 2,048 tokens over 8,192 keys
   // at 64 query heads, cut in segments: 475 against 533 us).
-  // (4 and 5: as 1 with two or three waves whatever the size, for measurements.)
-  if (through_lds && (shared == 1 || shared == 4 || shared == 5) && window == 0 && page >= 16 &&
-      (int64_t)Hkv * page * HD < (1ll << 31)) {
-    const bool three = ct == 2 && (shared == 5 || (shared == 1 && tiles * Hkv >= 1024 && a.max_segs == 1));
+  if (through_lds && shared == 1 && window == 0 && page >= 16 && (int64_t)Hkv * page * HD < (1ll << 31)) {
+    const bool three = ct == 2 && tiles * Hkv >= 1024 && a.max_segs == 1;
     if (three) attn_prefill_dma_kernel<2, 3><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else if (ct == 2) attn_prefill_dma_kernel<2, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else attn_prefill_dma_kernel<1, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
