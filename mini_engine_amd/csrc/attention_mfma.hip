@@ -932,6 +932,13 @@ __device__ __forceinline__ void lds_reads_done(bf16x8 (&x)[DT]) {
   pin_operands(x);
 }
 
+// A wave in its softmax goes first when the SIMD chooses whose instruction to issue: its vector instructions are
+// what the next products wait for, while a wave that is issuing products needs a slot only every 16 cycles
+// (2,048 tokens over 8,192 keys 156 -> 141 us, a prompt of 8,192 tokens 331 -> 318 us, of 32,768 3.85 -> 3.77 ms).
+__device__ __forceinline__ void softmax_priority(bool on) {
+  if (on) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
+}
+
 struct DmaPages { int k, v; };   // the page of this wave's two key instructions and of its two value instructions
 
 template <int CT, int W>
@@ -1109,9 +1116,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
         }
         bf16x8 va[DT];
         lds_read16_ahead<0>(lds0 + cur * DMA_BUF + rd_v, va);
+        softmax_priority(true);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
           block_softmax<FULL>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+        softmax_priority(false);
         lds_reads_done(va);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -1132,9 +1141,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
               st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[ct][ks], st[ct][tt], 0, 0, 0);
           }
         }
+        softmax_priority(true);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
           block_softmax<FULL>(a, st[ct], t0, col_lo[ct], col_hi[ct], m[ct], l[ct], acc[ct], g, pb[ct]);
+        softmax_priority(false);
         const unsigned char* vb = pf_lds + cur * DMA_BUF + rd_v;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -1528,7 +1539,7 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                                const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                int bt_stride, const int32_t* context_lens, const int32_t* cu_seqlens,
                                int num_seqs, int64_t num_tokens, int Hq, int Hkv, int page, float scale,
-                               int window, int col_tiles_per_wave, int shared, int seg_keys, int max_segs, float* pf_scratch,
+                               int window, int col_tiles_per_wave, int shared, int waves, int seg_keys, int max_segs, float* pf_scratch,
                                const int32_t* seq_of_token, int seq_base, hipStream_t stream) {
   if (num_seqs == 0 || num_tokens == 0) return 0;
   AttnArgs a;
@@ -1556,13 +1567,10 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   const bool through_lds = 2 * PF_BUF <= 65536 && shared != 0;
 #if ME_HEAD_DIM == 128
   // shared: 1 the memory system fills LDS where the kernel for that applies, 2 always through registers.
-  // Three waves to a SIMD where there are workgroups enough for three to a compute unit and the tiles are left
-  // whole, i.e. large launches that start at a prompt's beginning (8,192 tokens of one prompt, 16 query heads: 321
-  // against 356 us, 32 heads 524 against 597, 64 heads 998 against 1,069; 32,768 tokens: 3.83 against 4.20 ms), two
-  // with more registers each otherwise (512 tokens over 8,192 keys: 56 against 64 us; 2,048 tokens over 8,192 keys
-  // at 64 query heads, cut in segments: 475 against 533 us).
+  // waves: 3 asks for three waves to a SIMD (168 registers each) instead of two, with two column tiles; the
+  // caller knows the launches for which that pays.
   if (through_lds && shared == 1 && window == 0 && page >= 16 && (int64_t)Hkv * page * HD < (1ll << 31)) {
-    const bool three = ct == 2 && tiles * Hkv >= 1024 && a.max_segs == 1;
+    const bool three = ct == 2 && waves == 3;
     if (three) attn_prefill_dma_kernel<2, 3><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else if (ct == 2) attn_prefill_dma_kernel<2, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
     else attn_prefill_dma_kernel<1, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);

@@ -69,7 +69,7 @@ _CORE_PROTOS = {
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
-    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, P, P, I, P],
+    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, I, P, P, I, P],
     "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, I, P],
     "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, I, P],
 }
@@ -345,12 +345,13 @@ class HipBackend:
             Tp = T - num_decodes
             col_tiles = prefill_col_tiles(max_prefill_context, win, Tp, Hq, D)
             seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq, D, col_tiles)
+            waves = prefill_waves(max_prefill_context, Tp, B - num_decodes, Hq, Hkv, col_tiles, max_segs)
             pf = torch.empty((Tp * Hq * max_segs * (D + 2),), dtype=torch.float32, device=q.device) if max_segs > 1 else None
             lib.call("me_attn_prefill", q.data_ptr() + num_decodes * q.stride(0) * es, q.stride(0),
                      out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
                      block_tables.stride(0), context_lens.data_ptr() + num_decodes * 4, prefill_cu.data_ptr(),
-                     B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, col_tiles, PREFILL_THROUGH_LDS, seg_keys, max_segs,
+                     B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, col_tiles, PREFILL_THROUGH_LDS, waves, seg_keys, max_segs,
                      _ptr(pf), seq_of_token.data_ptr() + num_decodes * 4, num_decodes, _stream())
         return out
 
@@ -765,6 +766,27 @@ def choose_ksplit(M: int, N: int, K: int) -> int:
         if least is None or cost < least - 1e-9:
             best, least = splits, cost
     return best
+
+
+def prefill_waves(max_context: int, num_tokens: int, num_seqs: int, Hq: int, Hkv: int, col_tiles: int, max_segs: int) -> int:
+    """Waves per SIMD (2 or 3) of the prefill attention kernel whose loads write LDS themselves (head size 128).
+
+    Three waves of 168 registers where two column tiles per wave are in use, the tiles are left whole, there are
+    1,024 workgroups or more (three to a compute unit), and the prompts start at their beginning (the longest
+    context at most twice the mean number of new tokens per sequence): tiles of all lengths are then under way
+    at once (us, two / three waves: 8,192 tokens of one prompt at 16 query heads 356 / 321, at 32 heads 597 / 524,
+    at 64 heads 1,069 / 998; 32,768 tokens 4,200 / 3,830; eight prompts of 2,048 tokens 186 / 176). Portions
+    over a long prefix, whose tiles are equally long and walk the same keys together, run better with two waves
+    and 205 registers (2,048 tokens over 8,192 keys at 64 heads 475 / 533, over 6,000 keys 333 / 377, at 32 heads
+    270 / 282), and so do launches of few workgroups (512 tokens over 8,192 keys 56 / 64)."""
+    if col_tiles != 2 or max_segs != 1 or num_seqs < 1 or max_context <= 0:
+        return 2
+    group = max(1, Hq // max(1, Hkv))
+    tok_tile = max(1, 128 // group)
+    tiles = num_tokens // tok_tile + num_seqs
+    if tiles * Hkv < 1024 or max_context * num_seqs > 2 * num_tokens:
+        return 2
+    return 3
 
 
 def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: bool = False) -> tuple:
