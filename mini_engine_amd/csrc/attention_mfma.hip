@@ -934,7 +934,8 @@ __device__ __forceinline__ void lds_reads_done(bf16x8 (&x)[DT]) {
 
 // A wave in its softmax goes first when the SIMD chooses whose instruction to issue: its vector instructions are
 // what the next products wait for, while a wave that is issuing products needs a slot only every 16 cycles
-// (2,048 tokens over 8,192 keys 156 -> 141 us, a prompt of 8,192 tokens 331 -> 318 us, of 32,768 3.85 -> 3.77 ms).
+// (with two waves per SIMD: 2,048 tokens over 8,192 keys 151 -> 142 us, 512 over 8,192 55.0 -> 53.7 us, a prompt of
+// 2,048 tokens 45.7 -> 44.1 us; with three it changes nothing).
 __device__ __forceinline__ void softmax_priority(bool on) {
   if (on) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
 }

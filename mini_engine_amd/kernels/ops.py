@@ -589,6 +589,7 @@ GATED_MAX_K = 4096
 GATED_MAX_M = 16
 _COMPUTE_UNITS = 256
 _DECODE_WORKGROUPS = 4096
+_PREFILL_THREE_WAVES_WORKGROUPS = 2048
 _DECODE_WHOLE_WORKGROUPS = 768
 _DECODE_WHOLE_MAX_KEYS = 4096
 _DECODE_EVEN_WHOLE_WORKGROUPS = 192
@@ -772,19 +773,21 @@ def prefill_waves(max_context: int, num_tokens: int, num_seqs: int, Hq: int, Hkv
     """Waves per SIMD (2 or 3) of the prefill attention kernel whose loads write LDS themselves (head size 128).
 
     Three waves of 168 registers where two column tiles per wave are in use, the tiles are left whole, there are
-    1,024 workgroups or more (three to a compute unit), and the prompts start at their beginning (the longest
-    context at most twice the mean number of new tokens per sequence): tiles of all lengths are then under way
-    at once (us, two / three waves: 8,192 tokens of one prompt at 16 query heads 356 / 321, at 32 heads 597 / 524,
-    at 64 heads 1,069 / 998; 32,768 tokens 4,200 / 3,830; eight prompts of 2,048 tokens 186 / 176). Portions
-    over a long prefix, whose tiles are equally long and walk the same keys together, run better with two waves
-    and 205 registers (2,048 tokens over 8,192 keys at 64 heads 475 / 533, over 6,000 keys 333 / 377, at 32 heads
-    270 / 282), and so do launches of few workgroups (512 tokens over 8,192 keys 56 / 64)."""
+    2,048 workgroups or more, and the prompts start at their beginning (the longest context at most twice the mean
+    number of new tokens per sequence): tiles of all lengths are then under way at once and the third wave fills
+    the others' waits. us, two / three waves, the best of four runs taken in turn: one prompt at 16 query heads of
+    8,192 tokens 277 / 300, of 16,384 1,014 / 986, of 32,768 3,977 / 3,760; at 32 heads 8,192 tokens 511 / 504,
+    16,384 1,995 / 1,890; at 64 heads 4,096 tokens 282 / 271, 8,192 1,028 / 967, 16,384 3,994 / 3,751 (the
+    crossing lies at about 2,000 workgroups in each case). Portions over a long prefix, whose tiles are equally
+    long and walk the same keys together, run better with two waves and 205 registers (2,048 tokens over 8,192
+    keys at 64 heads 475 / 533, over 6,000 keys 333 / 377), and so do launches of few workgroups (512 tokens over
+    8,192 keys 56 / 64)."""
     if col_tiles != 2 or max_segs != 1 or num_seqs < 1 or max_context <= 0:
         return 2
     group = max(1, Hq // max(1, Hkv))
     tok_tile = max(1, 128 // group)
     tiles = num_tokens // tok_tile + num_seqs
-    if tiles * Hkv < 1024 or max_context * num_seqs > 2 * num_tokens:
+    if tiles * Hkv < _PREFILL_THREE_WAVES_WORKGROUPS or max_context * num_seqs > 2 * num_tokens:
         return 2
     return 3
 

@@ -45,15 +45,15 @@ def test_prefill_segments_cover_the_span_and_hold_512_keys_or_more():
 
 
 def test_three_waves_per_simd_only_for_large_launches_from_a_prompts_beginning():
-    assert ops.prefill_waves(8192, 8192, 1, 16, 8, 2, 1) == 3           # one prompt of 8,192 tokens: 129 tiles x 8 kv heads
+    assert ops.prefill_waves(16384, 16384, 1, 16, 8, 2, 1) == 3         # one prompt of 16,384 tokens: 257 tiles x 8 kv heads
+    assert ops.prefill_waves(8192, 8192, 1, 16, 8, 2, 1) == 2           # ... of 8,192: 1,032 workgroups, better with two
     assert ops.prefill_waves(2048, 16384, 8, 16, 8, 2, 1) == 3          # eight prompts of 2,048 tokens
-    assert ops.prefill_waves(2100, 2100, 1, 64, 8, 2, 1) == 3           # 16 tokens to a tile at a group of 8
-    assert ops.prefill_waves(1024, 9000, 16, 16, 8, 2, 1) == 3          # ragged prompts: the longest under twice the mean
-    assert ops.prefill_waves(8192, 2048, 1, 64, 8, 2, 1) == 2           # a portion over a long prefix
-    assert ops.prefill_waves(8192, 8192, 1, 16, 8, 2, 3) == 2           # tiles cut into segments
-    assert ops.prefill_waves(4096, 4096, 1, 16, 8, 2, 1) == 2           # 65 tiles x 8: too few workgroups
-    assert ops.prefill_waves(8192, 8192, 1, 16, 8, 1, 1) == 2           # one column tile per wave
-    assert ops.prefill_waves(0, 8192, 1, 16, 8, 2, 1) == 2              # no bound on the contexts known
+    assert ops.prefill_waves(4200, 4200, 1, 64, 8, 2, 1) == 3           # 16 tokens to a tile at a group of 8
+    assert ops.prefill_waves(1024, 18000, 32, 16, 8, 2, 1) == 3         # ragged prompts: the longest under twice the mean
+    assert ops.prefill_waves(16384, 4096, 1, 64, 8, 2, 1) == 2          # a portion over a long prefix
+    assert ops.prefill_waves(16384, 16384, 1, 16, 8, 2, 3) == 2         # tiles cut into segments
+    assert ops.prefill_waves(16384, 16384, 1, 16, 8, 1, 1) == 2         # one column tile per wave
+    assert ops.prefill_waves(0, 16384, 1, 16, 8, 2, 1) == 2             # no bound on the contexts known
 
 
 def test_ksplit_keeps_512_of_k_per_split_and_fills_the_gpu():
