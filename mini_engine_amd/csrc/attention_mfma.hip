@@ -920,6 +920,9 @@ __device__ __forceinline__ void pin_operands(bf16x8 (&x)[N][M]) {
 
 // Reads of 16 bytes at addr + 512 i that the compiler does not know to be reads: it neither moves them to their
 // use nor waits for them, so lds_reads_done() has to stand between them and the first use of what they return.
+// Until then the values must stay in the registers they were read into (a copy or a spill made by the compiler in
+// between would move what the registers held before): only for a kernel with registers to spare, which the form
+// with two waves per SIMD is (205 of 256; its test compares it bit for bit with the form that reads as usual).
 template <int I>
 __device__ __forceinline__ void lds_read16_ahead(uint32_t addr, bf16x8 (&x)[DT]) {
   if constexpr (I < DT) {
