@@ -866,7 +866,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 // =====================================================================================
 // Prefill / chunk kernel, keys and values brought into LDS by the memory system itself
 // (global_load_lds_dwordx4: every lane names 16 bytes of memory, and the 64 pieces of a wave's
-// instruction land in 1 KB of consecutive LDS), head size 128, pages of 16 keys or more, no window.
+// instruction land in 1 KB of consecutive LDS), head size 128, pages of 16 keys or more.
 // Against the form above this takes the staged block out of the registers and the LDS writes out of
 // the instruction stream, and lets a block be asked for NB - 1 blocks before its use instead of one:
 // in the form above an iteration cannot be shorter than the latency of its loads, which at two
@@ -881,8 +881,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 //           four ks steps stay 64 bytes apart.
 //   values  [2 halves of 16 keys][128 channels][32 B]: an instruction is 32 channel rows of one half,
 //           so with pages of 16 keys it reads one page; piece (g & 1) of a row lies at (g & 1) ^ (channel >> 3 & 1).
-// A block that reaches beyond the context (the last one of a sequence) is loaded into registers,
-// zeroed where it must not be used, and written to the same places.
+// A block that reaches beyond the context (the last one of a sequence), or back into pages behind a window that
+// may have been given back (the first one of a tile, with pages of 16 keys), is loaded into registers, zeroed where
+// it must not be used, and written to the same places.
 // =====================================================================================
 #define DMA_KINST 1088
 #define DMA_KBYTES (8 * DMA_KINST)
@@ -945,7 +946,7 @@ __device__ __forceinline__ void softmax_priority(bool on) {
 
 struct DmaPages { int k, v; };   // the page of this wave's two key instructions and of its two value instructions
 
-template <int CT, int W>
+template <int CT, int W, bool WINDOW>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))) attn_prefill_dma_kernel(AttnArgs a) {
   extern __shared__ __align__(16) unsigned char pf_lds[];   // [NB][DMA_BUF]
   constexpr int NB = DMA_NB, PD = NB - 1;                   // PD: blocks asked for ahead of the one in use
@@ -978,6 +979,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
   const int seg_hi = (a.seg_keys > 0 && seg + 1 < tr.nseg) ? seg_lo + a.seg_keys : (1 << 30);
   const int last = min(tr.pos_last, seg_hi - 1);   // the same key range for every wave of the workgroup
   const int nblk = (last - seg_lo) / 32 + 1;
+  // With a window, pages wholly behind it may have been given back: from the page that holds the tile's first
+  // visible key on, every page is held (pages are 16 keys or more, so this is a multiple of 16).
+  // (Without a window all of this is known when the kernel is compiled: the tests below cost the common case 2-7 %.)
+  const int first_held = WINDOW ? (tr.tile_lo >> a.page_shift) << a.page_shift : 0;
+  auto held = [&](int key) { return !WINDOW || key >= first_held; };
 
   const uint32_t lds0 = (uint32_t)(uintptr_t)pf_lds;
   // what a lane names in memory, relative to its instruction's first byte, and where it reads its operands
@@ -994,17 +1000,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
   // table entries of the block at t0, asked for one block before they are used
   auto lookup = [&](int t0) -> DmaPages {
     DmaPages pg;
-    pg.k = t0 + kg0 < L ? bt[(t0 + kg0) >> a.page_shift] : 0;
-    pg.v = t0 + 16 * vh < L ? bt[(t0 + 16 * vh) >> a.page_shift] : 0;
+    pg.k = (t0 + kg0 < L && held(t0 + kg0)) ? bt[(t0 + kg0) >> a.page_shift] : 0;
+    pg.v = (t0 + 16 * vh < L && held(t0 + 16 * vh)) ? bt[(t0 + 16 * vh) >> a.page_shift] : 0;
     return pg;
   };
   auto stage = [&](int t0, const DmaPages& pg, int bi) {
     const uint32_t buf = bi * DMA_BUF;
-    const int krow = t0 + kg0 < L ? ((t0 + kg0) & (a.page - 1)) : 0;
-    const int vkey = t0 + 16 * vh < L ? ((t0 + 16 * vh) & (a.page - 1)) : 0;
+    const int krow = (t0 + kg0 < L && held(t0 + kg0)) ? ((t0 + kg0) & (a.page - 1)) : 0;
+    const int vkey = (t0 + 16 * vh < L && held(t0 + 16 * vh)) ? ((t0 + 16 * vh) & (a.page - 1)) : 0;
     const bf16_t* gk = k_head + (uint64_t)(uint32_t)pg.k * page_elems + krow * HD;
     const bf16_t* gv = v_head + (uint64_t)(uint32_t)pg.v * page_elems + vkey;
-    if (t0 + 32 <= L) {
+    if (t0 + 32 <= L && held(t0)) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) dma16(gk + 8 * j * HD, voff_k, lds0 + buf + (2 * wave + j) * DMA_KINST);
 #pragma unroll
@@ -1017,15 +1023,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
       for (int j = 0; j < 2; ++j) {
         const int key = t0 + kg0 + 8 * j + (lane >> 4);
         // rows of a page that is held may be read beyond the context; without a page, page 0 is read
-        const bool held = t0 + kg0 + 8 * j < L;
-        const bf16_t* src = held ? gk + 8 * j * HD : k_head;
+        const bool mapped = t0 + kg0 + 8 * j < L && held(t0 + kg0);
+        const bf16_t* src = mapped ? gk + 8 * j * HD : k_head;
         const bf16x8 kk = ld8(reinterpret_cast<const bf16_t*>(reinterpret_cast<const unsigned char*>(src) + voff_k));
-        *reinterpret_cast<bf16x8*>(pf_lds + buf + (2 * wave + j) * DMA_KINST + 16 * lane) = key < L ? kk : z;
+        *reinterpret_cast<bf16x8*>(pf_lds + buf + (2 * wave + j) * DMA_KINST + 16 * lane) = (key < L && held(key)) ? kk : z;
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int key0 = t0 + 16 * vh + 8 * ((lane & 1) ^ ((lane >> 4) & 1));
-        const int nv = L - key0;
+        const int nv = held(key0) ? L - key0 : 0;    // (a piece of 8 keys lies wholly before or behind first_held)
         const bf16x8 vv = ld8(reinterpret_cast<const bf16_t*>(reinterpret_cast<const unsigned char*>(gv + (int64_t)32 * j * a.page) + voff_v));
         u32x4 w = __builtin_bit_cast(u32x4, vv);
 #pragma unroll
@@ -1054,11 +1060,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
       head[ct] = kvh * a.G + hh;
       const int pos = start + tok0 + tl;
       col_hi[ct] = valid[ct] ? pos : -1;
-      col_lo[ct] = 0;
+      col_lo[ct] = WINDOW ? max(0, pos - a.window + 1) : 0;
       load_q(a.q + tq[ct] * a.q_stride + (int64_t)head[ct] * HD, valid[ct], g, qb[ct]);
     }
-    const int pos_first = start + tok0 + c0 / a.G;
+    const int c_last = min(ncols, c0 + 16 * CT) - 1;
+    const int pos_first = start + tok0 + c0 / a.G, pos_last = start + tok0 + c_last / a.G;
     const int full_hi = active ? pos_first - 31 : -(1 << 30);
+    const int full_lo = WINDOW ? max(0, pos_last - a.window + 1) : 0;
     float m[CT], l[CT];
     f32x4 acc[CT][DT];
 #pragma unroll
@@ -1161,9 +1169,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
       }
       cur = cur == NB - 1 ? 0 : cur + 1;
     };
-    const int nfull = full_hi >= seg_lo ? min(nblk, (full_hi - seg_lo) / 32 + 1) : 0;
+    // blocks [first_full, end_full) lie wholly inside every column's range of this wave: behind the window's lower
+    // edge (if there is a window) and before the diagonal
+    const int end_full = full_hi >= seg_lo ? min(nblk, (full_hi - seg_lo) / 32 + 1) : 0;
     int k = 0;
-    for (; k < nfull; ++k) block_step(std::true_type{}, k);
+    if constexpr (WINDOW) {
+      const int first_full = full_lo > seg_lo ? min(end_full, (full_lo - seg_lo + 31) / 32) : 0;
+      for (; k < first_full; ++k) block_step(std::false_type{}, k);
+    }
+    for (; k < end_full; ++k) block_step(std::true_type{}, k);
     for (; k < nblk; ++k) block_step(std::false_type{}, k);
 
 #pragma unroll
@@ -1573,11 +1587,15 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
   // shared: 1 the memory system fills LDS where the kernel for that applies, 2 always through registers.
   // waves: 3 asks for three waves to a SIMD (168 registers each) instead of two, with two column tiles; the
   // caller knows the launches for which that pays.
-  if (through_lds && shared == 1 && window == 0 && page >= 16 && (int64_t)Hkv * page * HD < (1ll << 31)) {
+  if (through_lds && shared == 1 && page >= 16 && (int64_t)Hkv * page * HD < (1ll << 31)) {
     const bool three = ct == 2 && waves == 3;
-    if (three) attn_prefill_dma_kernel<2, 3><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
-    else if (ct == 2) attn_prefill_dma_kernel<2, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
-    else attn_prefill_dma_kernel<1, 2><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);
+#define DMA_LAUNCH(CTV, WV)                                                                                    \
+  do {                                                                                                         \
+    if (window > 0) attn_prefill_dma_kernel<CTV, WV, true><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);  \
+    else attn_prefill_dma_kernel<CTV, WV, false><<<grid, dim3(256), DMA_NB * DMA_BUF, stream>>>(a);            \
+  } while (0)
+    if (three) DMA_LAUNCH(2, 3); else if (ct == 2) DMA_LAUNCH(2, 2); else DMA_LAUNCH(1, 2);
+#undef DMA_LAUNCH
   } else
 #endif
   if (through_lds) {

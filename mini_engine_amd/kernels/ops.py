@@ -572,7 +572,7 @@ LIBRARY_MAX_K = 16384
 ROWS_MIN_WEIGHT = 16 * 1024 * 1024
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 # prefill attention, keys and values shared by a workgroup's waves through LDS: 0 never, 1 wherever it fits (written there
-# by the loads themselves at head size 128, pages of 16 keys or more and no window), 2 as 1 but always staged through registers
+# by the loads themselves at head size 128 and pages of 16 keys or more), 2 as 1 but always staged through registers
 PREFILL_THROUGH_LDS = 1
 PREFILL_COL_TILES = 0     # 0: chosen by prefill_col_tiles(); 1 or 2 force the column tiles per wave
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)

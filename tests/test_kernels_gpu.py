@@ -397,15 +397,18 @@ def test_attention_prefill_cut_into_segments(prefill_form, monkeypatch, seg_keys
 
 @pytest.mark.parametrize("Hq,Hkv,page", [(16, 8, 16), (64, 8, 16), (2, 2, 64), (40, 8, 256), (80, 1, 32)])
 def test_attention_prefill_lds_filled_by_the_loads_themselves(monkeypatch, Hq, Hkv, page):
-    """Head size 128, pages of 16 keys or more, no window: the loads write LDS directly, three buffers deep. Same
+    """Head size 128, pages of 16 keys or more: the loads write LDS directly, three buffers deep. Same
     products in the same order as the form that stages through registers, so the results are equal bit for bit;
     against the twin as everywhere. Contexts that end inside a block and inside a page (the cache holds NaN
     wherever no key was written), one block, fewer blocks than buffers, segments, a group of 80 heads (a token's
     columns take two rounds of the workgroup), and a launch large enough for three waves to a SIMD."""
     seqs = [(5, 5), (31, 31), (32, 32), (33, 33), (64, 2), (65, 33), (97, 96), (129, 17), (page + 1, 2), (700, 700), (1000, 64)]
-    for seg_keys, peak in ((None, None), (96, 450), (256, 3)):
+    # (segment size, the key that stands out, window): windows whose lower edge lies inside a block, at a block's
+    # start and at a page's start, with the pages behind them given back
+    for seg_keys, peak, window in ((None, None, None), (96, 450, None), (256, 3, None), (None, None, 50), (96, 690, 200),
+                                   (None, 940, 64), (256, None, 17)):
         monkeypatch.setattr(ops, "PREFILL_SEGMENT_KEYS", seg_keys)
-        args = _attention_case(torch.bfloat16, Hq, Hkv, 128, page, seqs, seed=page + Hq, peak=peak)
+        args = _attention_case(torch.bfloat16, Hq, Hkv, 128, page, seqs, window=window, seed=page + Hq, peak=peak)
         monkeypatch.setattr(ops, "PREFILL_THROUGH_LDS", 1)
         direct = hip().paged_attention(*args, max_prefill_context=1000)
         monkeypatch.setattr(ops, "PREFILL_THROUGH_LDS", 2)
