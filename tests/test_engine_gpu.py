@@ -269,16 +269,20 @@ def test_decode_graphs_replay_like_eager_steps(folders, dtype, name):
         assert err <= tol, f"{name} {r}: {err:.3g}"
 
 
+@pytest.mark.parametrize("window", [None, 100], ids=["full", "window"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-def test_real_layer_sizes(tmp_path_factory, dtype):
+def test_real_layer_sizes(tmp_path_factory, dtype, window):
     """Qwen3-0.6B's layer sizes (hidden 1024, 16 query / 8 key heads of 128, intermediate 3072, page 16)
     with 2 layers and a vocabulary that is no power of two: a long prompt in portions, then decoding,
-    beside a second request, against the plain implementation."""
+    beside a second request, against the plain implementation. `window`: the second layer sees the last 100
+    keys only, and the pages behind its window are given back while the first layer keeps all of them."""
     from mini_engine_amd.config.model_config import Qwen3Config
     from mini_engine_amd.weights.random_init import write_random_model
     cfgd = dict(architectures=["Qwen3ForCausalLM"], vocab_size=20011, hidden_size=1024, intermediate_size=3072,
                 num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6,
                 rope_theta=1e6, tie_word_embeddings=True, max_position_embeddings=4096)
+    if window:
+        cfgd.update(use_sliding_window=True, sliding_window=window, layer_types=["full_attention", "sliding_attention"])
     folder = write_random_model(Qwen3Config.from_dict(cfgd), 3, str(tmp_path_factory.mktemp("real")))
     model = load_model(folder, "cuda", dtype, 1024)
     manager = CacheManager(64, 16, ModelRunner.windows_of(model), enable_prefix_caching=False)
