@@ -29,7 +29,7 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 CORE_SOURCES = ["elementwise.hip", "rope_kv.hip", "attention_simple.hip",
-                "gemm.hip", "gemm_library.hip", "sampling.hip"]
+                "gemm.hip", "gemm_mid.hip", "gemm_library.hip", "sampling.hip"]
 ATTN_SOURCE = "attention_mfma.hip"
 HEADERS = ["common.h", "errors.inc", "sampling.h"]
 # Head sizes built by build_all(): the sizes of the benchmark models and of the test configurations.

@@ -65,6 +65,7 @@ _CORE_PROTOS = {
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
     "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, I, P],
+    "me_gemm_mid_bf16": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
@@ -454,6 +455,17 @@ class HipBackend:
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), None, 1, M, N, K, 0, 0, _stream())
             return y
+        mid = mid_takes(M, N, K, allow_partials and out_dtype == x.dtype)
+        if mid > 1:
+            parts = torch.empty((mid, M, N), dtype=torch.float32, device=x.device)
+            core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), parts.data_ptr(), N,
+                        ME_F32, mid, M, N, K, _stream())
+            return parts
+        if mid == 1:
+            y = new()
+            core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
+                        _code(out_dtype), 1, M, N, K, _stream())
+            return y
         # many rows, or the head over a large vocabulary: the library product (float32 accumulation; the
         # float32 output form keeps the logits unrounded)
         return library_product(x, w, out_dtype, out=out)
@@ -576,6 +588,8 @@ PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forc
 PREFILL_THROUGH_LDS = 1
 PREFILL_COL_TILES = 0     # 0: chosen by prefill_col_tiles(); 1 or 2 force the column tiles per wave
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
+USE_MID_PRODUCT = True          # False: products of 33-512 rows over small weights go to the library like the larger ones
+MID_MAX_WEIGHT = 8 << 20
 FUSE_GATE_INTO_GATE_UP = True  # False: silu(gate) * up is formed in front of the down product, not behind gate_up
 GATED_EPILOGUE_MAX_M = 16
 FUSE_NORM_INTO_LINEAR = True   # False: the norm kernel and the product behind it always run as two launches
@@ -767,6 +781,25 @@ def choose_ksplit(M: int, N: int, K: int) -> int:
         if least is None or cost < least - 1e-9:
             best, least = splits, cost
     return best
+
+
+def mid_takes(M: int, N: int, K: int, partials: bool) -> int:
+    """Whether the product of M rows against a bfloat16 weight [N, K] goes to the own kernel for a few hundred rows
+    over small weights (csrc/gemm_mid.hip), and in how many slices of K: 0 no, 1 one result, 4 float32 partial
+    sums over four slices (only when the consumer adds them, `partials`).
+
+    Its time is 7 us whatever the row count up to 256 (tiles of 64 x 64, one workgroup to a compute unit), where
+    the library's grows with the rows. us, own / library, weights warm, replayed: 4096 x 1024 at 65 / 128 / 192 /
+    256 / 384 rows 7.2 / 7.2 / 7.4 / 7.5 / 9.1 against 6.9 / 8.7 / 10.2 / 8.1 / 9.2; 6144 x 1024 7.2 / 7.3 / 8.8 /
+    9.3 / 11.9 against 7.7 / 8.6 / 10.3 / 11.9 / 12.2; with few output features and a long K in four slices:
+    1024 x 2048 at 65 / 256 / 512 rows 5.1 / 5.5 / 7.2 against 6.4 / 7.2 / 9.0, 1024 x 3072 6.1 / 6.6 / 9.3 against
+    6.7 / 8.7 / 11.5. Beyond 8 M weight elements (4096 x 2048 and up) and beyond these row counts the library's
+    larger tiles win (6144 x 1024 at 512 rows 14.6 against 12.7, 12288 x 2048 at 256 rows 23.5 against 23.0)."""
+    if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 256 or N * K > MID_MAX_WEIGHT or M <= 32:
+        return 0
+    if partials and N <= 2048 and K >= 2048 and M <= 512:
+        return 4
+    return 1 if M <= 256 else 0
 
 
 def prefill_waves(max_context: int, num_tokens: int, num_seqs: int, Hq: int, Hkv: int, col_tiles: int, max_segs: int) -> int:

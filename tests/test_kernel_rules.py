@@ -44,6 +44,17 @@ def test_prefill_segments_cover_the_span_and_hold_512_keys_or_more():
     assert ops.prefill_segments(1 << 20, 0, 8192, 64)[1] <= 3         # the partial results stay under 256 MB
 
 
+def test_a_few_hundred_rows_over_small_weights_go_to_the_own_product():
+    assert ops.mid_takes(128, 4096, 1024, False) == 1 and ops.mid_takes(256, 6144, 1024, False) == 1
+    assert ops.mid_takes(257, 6144, 1024, False) == 0                   # more rows: the library's larger tiles
+    assert ops.mid_takes(32, 4096, 1024, False) == 0                    # few rows: the skinny kernels
+    assert ops.mid_takes(128, 1024, 2048, True) == 4 and ops.mid_takes(512, 1024, 3072, True) == 4
+    assert ops.mid_takes(513, 1024, 3072, True) == 0 and ops.mid_takes(128, 1024, 2048, False) == 1
+    assert ops.mid_takes(128, 4096, 1024, True) == 1                    # many features: no slices of K
+    assert ops.mid_takes(128, 12288, 2048, False) == 0                  # beyond 8 M weight elements
+    assert ops.mid_takes(128, 4096, 1000, False) == 0                   # K no multiple of 64
+
+
 def test_three_waves_per_simd_only_for_large_launches_from_a_prompts_beginning():
     assert ops.prefill_waves(16384, 16384, 1, 16, 8, 2, 1) == 3         # one prompt of 16,384 tokens: 257 tiles x 8 kv heads
     assert ops.prefill_waves(8192, 8192, 1, 16, 8, 2, 1) == 2           # ... of 8,192: 1,032 workgroups, better with two

@@ -576,6 +576,32 @@ def test_linear_rows_kernel(M, N, K):
     close(hip().linear(xs, w, None, allow_partials=True).sum(0), xs.double() @ w.double().t(), 2e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 4096, 1024), (256, 6144, 1024), (130, 1024, 2048), (200, 1024, 3072), (512, 1024, 2048),
+                                   (100, 1000, 320), (40, 6144, 1024), (70, 68, 256), (77, 1028, 2112)])
+def test_linear_a_few_hundred_rows_over_small_weights(M, N, K):
+    """33-512 rows over weights of up to 8 M elements: the own kernel with tiles of 64 x 64 whose loads write LDS
+    themselves; row and feature counts that are no multiples of 64 (the last tiles read the matrix's last row again
+    and store nothing for it), K a multiple of 64 only, a row stride that is not K, bfloat16 and float32 results,
+    and four slices of K as float32 partial sums where the features are few and the consumer adds them."""
+    from mini_engine_amd.kernels import ops
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    ref = x.double() @ w.double().t()
+    assert ops.mid_takes(M, N, K, False) == (1 if M <= 256 else 0) and not ops.skinny_takes(M, N, K)
+    if M <= 256:
+        close(hip().linear(x, w), ref, 6e-3)
+        close(hip().linear(x, w, torch.float32), ref, 2e-5)
+        xs = torch.randn(M, K + 8, device=DEV).bfloat16()[:, :K]
+        close(hip().linear(xs, w), xs.double() @ w.double().t(), 6e-3)
+    parts = hip().linear(x, w, None, allow_partials=True)
+    if N <= 2048 and K >= 2048:
+        assert ops.mid_takes(M, N, K, True) == 4 and parts.shape == (4, M, N) and parts.dtype == torch.float32
+        close(parts.sum(0), ref, 2e-5)
+    else:
+        assert parts.dim() == 2
+        close(parts, ref, 6e-3)
+
+
 @pytest.mark.parametrize("M,N,K", [(200, 384, 80), (2048, 1024, 1024), (65, 100, 200), (70, 96, 44)])
 def test_linear_large_and_odd_bf16(M, N, K):
     """Above the skinny range the library product runs; K not a multiple of 8 takes the FMA kernel."""
