@@ -36,7 +36,10 @@ template <int N>
 __device__ __forceinline__ void mid_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 __device__ __forceinline__ void mid_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <typename TO, bool PARTIAL>
+// ACT: w is a packed gate/up weight [2 I, K] (gate rows first, N = 2 I); the tile's 64 weight rows are 32 gate rows and
+// the 32 up rows that go with them, a wave's two feature tiles are 16 gate features and their up features, and what
+// is written is silu(gate) * up [M, I], formed from the unrounded sums (reference layers/activation.py:5-7).
+template <typename TO, bool PARTIAL, bool ACT>
 __global__ void __launch_bounds__(256)
 gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                 TO* __restrict__ y, int64_t ldy, int M, int N, int K, int steps_per_split, int m_tiles, int n_tiles) {
@@ -52,7 +55,8 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
   const int mt = rest % m_tiles;
   const int nt = (rest / m_tiles) * 8 + (id & 7);
   if (nt >= n_tiles) return;
-  const int m0 = mt * MID_TM, n0 = nt * MID_TN;
+  const int I = N / 2;                              // ACT only
+  const int m0 = mt * MID_TM, n0 = nt * (ACT ? MID_TN / 2 : MID_TN);
   const int steps = K / MID_BK;
   const int s_lo = blockIdx.z * steps_per_split;
   const int s_hi = min(steps, s_lo + steps_per_split);
@@ -68,7 +72,10 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
     const int R = 8 * inst + (lane >> 3);
     const int c = (lane & 7) ^ ((R >> 1) & 7);
     is_x[q] = inst < MID_TM / 8;
-    const int64_t row = is_x[q] ? min(m0 + R, M - 1) : min(n0 + R - MID_TM, N - 1);
+    const int wr = R - MID_TM;                      // weight row of the tile
+    const int64_t row = is_x[q] ? min(m0 + R, M - 1)
+                        : ACT ? (wr < 32 ? min(n0 + wr, I - 1) : I + min(n0 + wr - 32, I - 1))
+                              : min(n0 + wr, N - 1);
     voff[q] = (uint32_t)(row * (is_x[q] ? ldx : ldw) * 2 + 16 * c);
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)mid_lds;
@@ -86,7 +93,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     rd_b[s] = (wm * 32 + n) * 128 + (((4 * s + g) ^ swz) * 16);
-    rd_a[s] = (MID_TM + wn * 32 + n) * 128 + (((4 * s + g) ^ swz) * 16);
+    rd_a[s] = (MID_TM + wn * (ACT ? 16 : 32) + n) * 128 + (((4 * s + g) ^ swz) * 16);
   }
   f32x4 acc[2][2];
 #pragma unroll
@@ -108,7 +115,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
     for (int s = 0; s < 2; ++s) {
       bf16x8 a[2], b[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const bf16x8*>(buf + rd_a[s] + 2048 * i);
+      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const bf16x8*>(buf + rd_a[s] + (ACT ? 4096 : 2048) * i);
 #pragma unroll
       for (int j = 0; j < 2; ++j) b[j] = *reinterpret_cast<const bf16x8*>(buf + rd_b[s] + 2048 * j);
 #pragma unroll
@@ -119,31 +126,47 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
     cur = cur == MID_NB - 1 ? 0 : cur + 1;
   }
   // lane (n, g) of tile (i, j): features n0 + 32 wn + 16 i + 4 g .. + 3 of token m0 + 32 wm + 16 j + n
+  // (ACT: tile 0 holds the gates and tile 1 the up values of features n0 + 16 wn + 4 g .. + 3)
   TO* out = PARTIAL ? y + (int64_t)blockIdx.z * M * ldy : y;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int t = m0 + wm * 32 + 16 * j + n;
+    if constexpr (ACT) {
+      const int f = n0 + wn * 16 + 4 * g;
+      if (t < M && f < I) {
+        typedef TO out4 __attribute__((ext_vector_type(4)));
+        out4 r;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int f = n0 + wn * 32 + 16 * i + 4 * g;
-      if (t < M && f < N) {
-        if constexpr (PARTIAL) {
-          *reinterpret_cast<f32x4*>(out + (int64_t)t * ldy + f) = acc[i][j];
-        } else {
-          typedef TO out4 __attribute__((ext_vector_type(4)));
-          out4 r;
+        for (int e = 0; e < 4; ++e) {
+          const float gate = acc[0][j][e];
+          r[e] = from_f32<TO>(gate / (1.f + __expf(-gate)) * acc[1][j][e]);
+        }
+        *reinterpret_cast<out4*>(out + (int64_t)t * ldy + f) = r;
+      }
+    } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) r[e] = from_f32<TO>(acc[i][j][e]);
-          *reinterpret_cast<out4*>(out + (int64_t)t * ldy + f) = r;
+      for (int i = 0; i < 2; ++i) {
+        const int f = n0 + wn * 32 + 16 * i + 4 * g;
+        if (t < M && f < N) {
+          if constexpr (PARTIAL) {
+            *reinterpret_cast<f32x4*>(out + (int64_t)t * ldy + f) = acc[i][j];
+          } else {
+            typedef TO out4 __attribute__((ext_vector_type(4)));
+            out4 r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = from_f32<TO>(acc[i][j][e]);
+            *reinterpret_cast<out4*>(out + (int64_t)t * ldy + f) = r;
+          }
         }
       }
     }
   }
 }
 
-// y: [M, N] of out_dtype (ksplit 1), or float32 partial sums [ksplit, M, N] with ldy = N.
+// y: [M, N] of out_dtype (ksplit 1), or float32 partial sums [ksplit, M, N] with ldy = N; act: w is a packed
+// gate/up weight [N = 2 I, K] and y is silu(gate) * up [M, I] (bfloat16, ksplit 1).
 extern "C" int me_gemm_mid_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
-                                int out_dtype, int ksplit, int M, int N, int K, hipStream_t stream) {
+                                int out_dtype, int ksplit, int M, int N, int K, int act, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   ME_CHECK(K >= MID_BK && K % MID_BK == 0, "mid gemm: K=%d must be a multiple of %d", K, MID_BK);
   ME_CHECK(N % 4 == 0 && ldy % 4 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "mid gemm: N=%d and the row strides must keep 16-byte pieces whole", N);
@@ -155,17 +178,19 @@ extern "C" int me_gemm_mid_bf16(const void* x, int64_t ldx, const void* w, int64
   ME_CHECK(ksplit == 1 || out_dtype == ME_F32, "mid gemm: partial sums are float32");
   const int steps_per_split = (steps + ksplit - 1) / ksplit;
   ME_CHECK((int64_t)(ksplit - 1) * steps_per_split < steps, "mid gemm: ksplit %d leaves a slice without work", ksplit);
-  const int m_tiles = (M + MID_TM - 1) / MID_TM, n_tiles = (N + MID_TN - 1) / MID_TN;
+  ME_CHECK(!act || (ksplit == 1 && out_dtype == ME_BF16 && N % 8 == 0), "mid gemm: the gating wants one bfloat16 result and I a multiple of 4");
+  const int m_tiles = (M + MID_TM - 1) / MID_TM, n_tiles = act ? (N / 2 + MID_TN / 2 - 1) / (MID_TN / 2) : (N + MID_TN - 1) / MID_TN;
   const int64_t ids = (int64_t)((n_tiles + 7) / 8) * 8 * m_tiles;
   ME_CHECK(ids < (1ll << 31), "mid gemm: too many tiles");
   const dim3 grid((unsigned)ids, 1, ksplit), block(256);
   const size_t lds = (size_t)MID_NB * MID_STAGE;
-#define MID_LAUNCH(TO, P)                                                                                          \
-  gemm_mid_kernel<TO, P><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, ldy, M, N, \
-                                                      K, steps_per_split, m_tiles, n_tiles)
-  if (ksplit > 1) MID_LAUNCH(float, true);
-  else if (out_dtype == ME_F32) MID_LAUNCH(float, false);
-  else MID_LAUNCH(bf16_t, false);
+#define MID_LAUNCH(TO, P, A)                                                                                       \
+  gemm_mid_kernel<TO, P, A><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, ldy, M, \
+                                                         N, K, steps_per_split, m_tiles, n_tiles)
+  if (act) MID_LAUNCH(bf16_t, false, true);
+  else if (ksplit > 1) MID_LAUNCH(float, true, false);
+  else if (out_dtype == ME_F32) MID_LAUNCH(float, false, false);
+  else MID_LAUNCH(bf16_t, false, false);
 #undef MID_LAUNCH
   ME_LAUNCH_CHECK();
   return 0;

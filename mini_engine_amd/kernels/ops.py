@@ -65,7 +65,7 @@ _CORE_PROTOS = {
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
     "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, I, P],
-    "me_gemm_mid_bf16": [P, L, P, L, P, L, I, I, I, I, I, P],
+    "me_gemm_mid_bf16": [P, L, P, L, P, L, I, I, I, I, I, I, P],
     "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
 }
@@ -459,12 +459,12 @@ class HipBackend:
         if mid > 1:
             parts = torch.empty((mid, M, N), dtype=torch.float32, device=x.device)
             core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), parts.data_ptr(), N,
-                        ME_F32, mid, M, N, K, _stream())
+                        ME_F32, mid, M, N, K, 0, _stream())
             return parts
         if mid == 1:
             y = new()
             core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
-                        _code(out_dtype), 1, M, N, K, _stream())
+                        _code(out_dtype), 1, M, N, K, 0, _stream())
             return y
         # many rows, or the head over a large vocabulary: the library product (float32 accumulation; the
         # float32 output form keeps the logits unrounded)
@@ -473,12 +473,16 @@ class HipBackend:
     def gated_linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         """silu(x . w[:I]^T) * (x . w[I:]^T) for a packed gate/up weight w [2 I, K] (gate rows first), as one
         launch: the product's workgroups pair each gate feature with its up feature when they merge their waves,
-        from the unrounded sums (the separate kernels round the product to bfloat16 first). For the few rows
+        from the unrounded sums (the separate kernels round the product to bfloat16 first). For the row counts
         `gated_linear_fuses` admits. Returns [M, I]. (reference layers/linear.py:29-45, layers/activation.py:5-7.)"""
         _check(gated_linear_fuses(x, w), "gated_linear: bfloat16, few rows, see gated_linear_fuses")
         M, K = x.shape
         N = w.shape[0]
         y = torch.empty((M, N // 2), dtype=x.dtype, device=x.device)
+        if M > GATED_EPILOGUE_MAX_M:        # a few hundred rows over a small weight: the gating in that kernel's epilogue
+            core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N // 2,
+                        ME_BF16, 1, M, N, K, 1, _stream())
+            return y
         core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N // 2,
                     ME_BF16, None, 1, M, N, K, 0, 1, _stream())
         return y
@@ -864,8 +868,10 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
 def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     """Whether `rows` rows against the packed gate/up weight w [2 I, K] are few enough, and w of a kind, for the
     gating to happen in the product's epilogue: a bfloat16 product that the unsplit skinny kernel takes, up to
-    GATED_EPILOGUE_MAX_M rows. At the 0.6B widths the gating in front of the down product costs every one of that
-    product's workgroups about 2 us; behind gate/up every gate is formed once."""
+    GATED_EPILOGUE_MAX_M rows, or one of 33-256 rows that the tiled kernel for small weights takes (`mid_takes`). At
+    the 0.6B widths the gating in front of the down product costs every one of that product's workgroups about 2 us;
+    behind gate/up every gate is formed once. At 33-256 rows the gating was a kernel of its own: a layer's feed-forward,
+    us, apart / in the epilogue: 40 rows 17.5 / 14.8, 64 rows 18.8 / 15.9, 128 rows 20.6 / 17.5, 256 rows 24.6 / 20.4."""
     if not FUSE_GATE_INTO_GATE_UP or w.dtype != torch.bfloat16 or w.dim() != 2:
         return False
     N, K = w.shape
@@ -874,8 +880,12 @@ def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     # (4096 -> 24576, us: 4 rows 38.9 / 45.5, 6 rows 41.4 / 45.6, 8 rows 43.9 / 45.5, 12 rows 49.2 / 46.2; over a K of
     # 5,120 the library is level or ahead from 4 rows on: 5120 -> 34816, 4 rows 75.0 / 76.4, 6 rows 81.2 / 76.5)
     takes = skinny_takes(rows, N, K) or (rows <= 8 and K <= 4096 and N < LIBRARY_MIN_N and rows <= SKINNY_MAX_M)
-    return (1 <= rows <= GATED_EPILOGUE_MAX_M and N % 2 == 0 and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0
-            and w.data_ptr() % 16 == 0 and takes)
+    aligned = N % 2 == 0 and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
+    if rows > GATED_EPILOGUE_MAX_M:
+        # a few hundred rows over a small weight: the kernel that takes the product (mid_takes) gates in its epilogue too,
+        # in place of a kernel of its own behind it
+        return aligned and N % 8 == 0 and not skinny_takes(rows, N, K) and mid_takes(rows, N, K, False) == 1
+    return 1 <= rows and aligned and takes
 
 
 def gated_linear_fuses(x: torch.Tensor, w: torch.Tensor) -> bool:

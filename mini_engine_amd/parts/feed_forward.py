@@ -24,7 +24,8 @@ class SwiGLU(FeedForward):
     def forward(self, x):
         rows = x.x.shape[-2] if isinstance(x, PendingNorm) else x.shape[0]
         if ops.gated_linear_rows(rows, self.gate_up.weight):
-            # few rows: the gating in the gate/up product's epilogue (every gate formed once), a plain down product
+            # few rows (or a few hundred over a small weight): the gating in the gate/up product's epilogue (every gate formed
+            # once), a plain down product
             return self.down.forward(self.gate_up.forward(x, gated=True), allow_partials=True)
         gu = self.gate_up.forward(x)
         return ops.silu_mul_linear(gu, self.down.weight, allow_partials=True)

@@ -1,4 +1,6 @@
 """The host-side rules that pick a kernel form (pure functions of the sizes), on the CPU."""
+import torch
+
 from mini_engine_amd.kernels import ops
 
 
@@ -53,6 +55,14 @@ def test_a_few_hundred_rows_over_small_weights_go_to_the_own_product():
     assert ops.mid_takes(128, 4096, 1024, True) == 1                    # many features: no slices of K
     assert ops.mid_takes(128, 12288, 2048, False) == 0                  # beyond 8 M weight elements
     assert ops.mid_takes(128, 4096, 1000, False) == 0                   # K no multiple of 64
+
+
+def test_gate_up_gates_in_its_epilogue_for_few_rows_and_for_a_few_hundred_over_small_weights():
+    w = torch.empty(6144, 1024, dtype=torch.bfloat16)
+    assert all(ops.gated_linear_rows(m, w) for m in (1, 8, 16, 33, 64, 256))
+    assert not any(ops.gated_linear_rows(m, w) for m in (17, 32, 257, 2048))   # the down product gates, or a kernel of its own
+    assert not ops.gated_linear_rows(128, torch.empty(12288, 2048, dtype=torch.bfloat16))    # the library's product
+    assert not ops.gated_linear_rows(128, torch.empty(6144, 1024))                            # float32
 
 
 def test_three_waves_per_simd_only_for_large_launches_from_a_prompts_beginning():

@@ -532,6 +532,28 @@ def test_gating_in_the_gate_up_products_epilogue(M, I, K):
         close(y, want, 6e-3)
 
 
+@pytest.mark.parametrize("M", [33, 65, 130, 256])
+@pytest.mark.parametrize("I,K", [(3072, 1024), (100, 256), (36, 320), (1000, 2048)])
+def test_gating_in_the_epilogue_for_a_few_hundred_rows(M, I, K):
+    """The same for 33 to 256 rows over a small weight: the tiled kernel takes 32 gate features and their 32 up features
+    to a workgroup; a last tile that is partly beyond I, and an I that is no multiple of 16."""
+    torch.manual_seed(M + I)
+    w = (torch.randn(2 * I, K, device=DEV) * 0.05).bfloat16()
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    if ops.skinny_takes(M, 2 * I, K):       # up to 64 rows over the smaller weights the skinny kernel has the product
+        assert not ops.gated_linear_fuses(x, w)
+        return
+    assert ops.gated_linear_fuses(x, w) and ops.mid_takes(M, 2 * I, K, False) == 1
+    got = hip().gated_linear(x, w)
+    assert got.shape == (M, I)
+    close(got, twin.gated_linear(x, w, compute_dtype=torch.float64), 6e-3)
+    close(got, hip().silu_and_mul(hip().linear(x, w)), 1.5e-2)         # those round the product before the gating
+    # one gate feature far out, so that a gate paired with another feature's up value shows
+    w2 = w.clone()
+    w2[I // 2] *= 40
+    close(hip().gated_linear(x, w2), twin.gated_linear(x, w2, compute_dtype=torch.float64), 6e-3)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40])
 @pytest.mark.parametrize("N,I", [(1024, 3072), (80, 224), (72, 200)])
 def test_silu_mul_linear(M, N, I):
