@@ -109,6 +109,18 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 __device__ __forceinline__ bf16x8 ld8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+// The same for data that is read once (a decode step's keys and values): marked as not to be kept by the caches,
+// which this GPU's memory system answers with a higher rate (a plain read of 4 GB: 5.2-6.4 TB/s, marked 5.7-7.3).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <bool STREAM>
+__device__ __forceinline__ bf16x8 ld8s(const bf16_t* p) {
+  if constexpr (STREAM) {
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return __builtin_bit_cast(bf16x8, v);
+  } else {
+    return ld8(p);
+  }
+}
 
 // Max / sum over the four lanes n, n+16, n+32, n+48 that share a column, left in all four.
 // v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of
@@ -178,6 +190,7 @@ __device__ __forceinline__ void lookup_pages(const AttnArgs& a, const int32_t* _
   pg.voff = pg.vgrp_ok ? vgrp - vpi * a.page : 0;
 }
 
+template <bool STREAM = false>
 __device__ __forceinline__ void load_kv(const AttnArgs& a, const BlockPages& pg, int kvh, int t0, int L, int n,
                                         int g, KVBlock& blk) {
   // a table entry that holds no page (-1) is treated like a key past the context: page 0, zeros
@@ -193,7 +206,7 @@ __device__ __forceinline__ void load_kv(const AttnArgs& a, const BlockPages& pg,
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = 32 * ks + 8 * g;
-      blk.k[tt][ks] = ld8(kp + ((HD % 32 == 0 || d0 < HD) ? d0 : 0));
+      blk.k[tt][ks] = ld8s<STREAM>(kp + ((HD % 32 == 0 || d0 < HD) ? d0 : 0));
     }
   }
   const bool vgrp_ok = pg.vgrp_ok && pg.vpage >= 0;
@@ -212,11 +225,12 @@ __device__ __forceinline__ void settle_value_page(KVBlock& blk) {
 }
 
 // V^T rows: channel 16*dt + n, keys t0 + 8g .. t0 + 8g + 7
+template <bool STREAM = false>
 __device__ __forceinline__ void load_v(const AttnArgs& a, const KVBlock& blk, int kvh, int t0, int L, int n, int g,
                                        VBlock& vb) {
   const bf16_t* vp = a.v_cache + (((int64_t)blk.vpage * a.Hkv + kvh) * HD + n) * a.page + blk.voff;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) vb.v[dt] = ld8(vp + (int64_t)dt * 16 * a.page);
+  for (int dt = 0; dt < DT; ++dt) vb.v[dt] = ld8s<STREAM>(vp + (int64_t)dt * 16 * a.page);
   // keys at or past L hold foreign or unwritten data (possibly NaN): their bits are cleared
   const int nv = blk.vkeys;
 #pragma unroll
@@ -224,11 +238,12 @@ __device__ __forceinline__ void load_v(const AttnArgs& a, const KVBlock& blk, in
     vb.vmask[j] = (2 * j < nv ? 0x0000ffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
 }
 
+template <bool STREAM = false>
 __device__ __forceinline__ void load_block(const AttnArgs& a, const int32_t* __restrict__ bt, int kvh, int t0,
                                            int L, int lo_min, int n, int g, KVBlock& blk) {
   BlockPages pg;
   lookup_pages(a, bt, t0, L, lo_min, n, g, pg);
-  load_kv(a, pg, kvh, t0, L, n, g, blk);
+  load_kv<STREAM>(a, pg, kvh, t0, L, n, g, blk);
 }
 
 // Scores of the block against one 16-column tile, online-softmax update, and P.V.
@@ -1282,6 +1297,10 @@ __device__ __forceinline__ void decode_part_range(const AttnArgs& a, int L, int&
 // workgroups whose partition holds position L - 1 do the same for the new key and copy the new value: they
 // attend to both from LDS, in place of what the page holds there, and the first column tile's workgroup writes
 // them into the page. No workgroup reads what another one writes.
+#ifndef ME_DECODE_STREAMS
+#define ME_DECODE_STREAMS 1
+#endif
+constexpr bool DECODE_STREAMS = ME_DECODE_STREAMS != 0;
 template <bool PROLOGUE>
 __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
   extern __shared__ float lds[];  // [4 waves][cols][HD + 2]; PROLOGUE: then bfloat16 [cols + 2][HD]
@@ -1380,7 +1399,7 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     bf16_t new_v = static_cast<bf16_t>(0.f);
     const int vd = threadIdx.x < HD ? threadIdx.x : 0;
     if (holds_new) new_v = a.raw_v[t * a.q_stride + (int64_t)kvh * HD + vd];
-    if (has_keys) load_block(a, bt, kvh, t0, L, lo, n, g, A);
+    if (has_keys) load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
     if (wave < nheads) finish_head(wave, first);
     for (int h = wave + 4; h < nheads; h += 4) {
       RawHead r;
@@ -1398,7 +1417,7 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     }
     __syncthreads();
   } else if (has_keys) {
-    load_block(a, bt, kvh, t0, L, lo, n, g, A);
+    load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
   }
   if (has_keys) {
     bf16x8 qb[KS];
@@ -1407,7 +1426,7 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     const int col_hi = valid ? pos : -1;
     while (true) {
       VBlock vb;
-      load_v(a, A, kvh, t0, L, n, g, vb);
+      load_v<DECODE_STREAMS>(a, A, kvh, t0, L, n, g, vb);
       if (holds_new && pos >= t0 && pos < t0 + 32) {
         // the block with the new token: its key row and its value column come from LDS
         const int rel = pos - t0;
@@ -1435,7 +1454,7 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
       else attend_block<false>(a, A, vb, t0, qb, lo, col_hi, m, l, acc, g);
       t0 += 128;
       if (t0 >= p_hi) break;
-      load_block(a, bt, kvh, t0, L, lo, n, g, A);
+      load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
     }
   }
   l = column_sum(l);
