@@ -132,12 +132,21 @@ struct SkinnyOperands {
 // layers/linear.py:29-45), and y is silu(gate) * up, [M, I] (layers/activation.py:5-7): a workgroup takes 8 gate
 // features and the 8 up features that go with them as the 16 rows of its matrix operand and pairs them when it
 // merges its waves, so every gate is formed once, from the unrounded sums.
-template <int MT, typename TO, bool GATED, bool EXACT_K, bool ACT = false>
-__global__ void __launch_bounds__(256)
+// WIDE (one tile of tokens, EXACT_K, not GATED; for large weights): a load of a wave takes whole rows of the step,
+// 256 contiguous bytes of each of four weight rows, marked as not to be kept by the caches, instead of 64 bytes of
+// each of sixteen: only loads that take whole 128-byte lines gain by the mark (a kernel that only reads a 201-524 MB
+// weight: 5.3-6.1 TB/s in the plain pattern, 5.9-6.9 so), and the pieces then pass through a wave's own 4 KB of LDS to
+// reach the lanes that the matrix instruction wants them in.
+template <int MT, typename TO, bool GATED, bool EXACT_K, bool ACT = false, bool WIDE = false>
+__global__ void __launch_bounds__(256, WIDE ? 5 : 1)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                    TO* __restrict__ y, int64_t ldy, float* __restrict__ partials, int M, int N, int K,
                    int steps_per_split) {
+  static_assert(!WIDE || (MT == 1 && !GATED && EXACT_K), "the wide loads are built for one tile of tokens and whole steps");
   __shared__ float red[4][MT][256];
+  // WIDE: per wave 16 rows of 16 pieces of 16 bytes, a row 272 bytes from the next, so that the 16 rows a read takes
+  // at once are spread over all banks and every address is a lane's base plus a constant
+  __shared__ __align__(16) unsigned char wtile[WIDE ? 4 : 1][WIDE ? 16 * 272 : 16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * (ACT ? 8 : 16), m0 = blockIdx.y * 16 * MT;
@@ -151,6 +160,17 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
   if (ACT) feature = n0 + (r & 7) < half ? (r < 8 ? n0 + r : half + n0 + r - 8) : 0;
   else feature = n0 + r < N ? n0 + r : 0;
   const bf16_t* wrow = w + (int64_t)feature * ldw;
+  // WIDE: load j of lane (piece r, g) takes piece r of the step from row 4 j + g of the workgroup's sixteen, as a
+  // byte offset from w (the launcher admits weights under 2 GB) formed where it is used: four row addresses kept
+  // would not fit the registers of five waves to a SIMD
+  const uint32_t ldw_bytes = (uint32_t)ldw * 2u;
+  auto wide_offset = [&](int j, int s) -> uint32_t {
+    const int rr = 4 * j + g;
+    int f;
+    if (ACT) f = j < 2 ? min(n0 + rr, half - 1) : half + min(n0 + rr - 8, half - 1);
+    else f = min(n0 + rr, N - 1);
+    return (uint32_t)f * ldw_bytes + 16u * (uint32_t)r + 256u * (uint32_t)s;
+  };
   const bf16_t* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -170,7 +190,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
     for (int j = 0; j < 4; ++j) {
       const int k = kb + 32 * j;
       const int ks = (EXACT_K || k < K) ? k : 0;
-      op.a[j] = *reinterpret_cast<const bf16x8*>(live ? wrow + ks : w);
+      if (WIDE) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const uint32_t off = live ? wide_offset(j, s) : 0u;
+        op.a[j] = __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(w) + off)));
+      } else {
+        op.a[j] = *reinterpret_cast<const bf16x8*>(live ? wrow + ks : w);
+      }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         op.b[mt][j] = *reinterpret_cast<const bf16x8*>(live ? xrow[mt] + ks : x);
@@ -180,10 +206,21 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
   };
   auto product = [&](int s, const SkinnyOperands<MT, GATED>& op) {
     const int kb = 128 * s + 8 * g;
+    bf16x8 wide_a[4];
+    if (WIDE) {
+      // the wave's LDS operations run in the order they are issued: what its lanes write here, its lanes read below
+      unsigned char* tile = wtile[wave];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *reinterpret_cast<bf16x8*>(tile + (g * 272 + r * 16) + j * (4 * 272)) = op.a[j];
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wide_a[j] = *reinterpret_cast<const bf16x8*>(tile + (r * 272 + g * 16) + j * 64);
+      asm volatile("" ::: "memory");
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const bool kok = EXACT_K || kb + 32 * j < K;
-      const bf16x8 a = kok ? op.a[j] : z;
+      const bf16x8 a = WIDE ? wide_a[j] : (kok ? op.a[j] : z);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         bf16x8 b = op.b[mt][j];
@@ -398,8 +435,11 @@ extern "C" int me_gemm_rows_bf16(const void* x, int64_t ldx, const void* w, int6
 // is silu(gate) * up, [M, N / 2] (at most 16 rows, K not split, not together with gated).
 extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y,
                                    int64_t ldy, int out_dtype, float* partials, int ksplit, int M, int N,
-                                   int K, int gated, int act, hipStream_t stream) {
+                                   int K, int gated, int act, int wide, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
+  // wide: the caller asks for the wide loads (large weights); they apply to one tile of tokens, K in whole steps of
+  // 128, an ungated input and a weight under 2 GB, and are left out otherwise
+  const bool wide_ok = wide && M <= 16 && !gated && K % 128 == 0 && (int64_t)(N - 1) * ldw + K <= (int64_t)0x3fffffff;
   if (act) {
     ME_CHECK(!gated && ksplit == 1 && partials == nullptr && M <= 16 && N % 2 == 0,
              "skinny gemm: the gating epilogue takes at most 16 rows, an unsplit K and an even number of weight rows");
@@ -412,7 +452,10 @@ extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, in
 #define LAUNCH_ACT(TO, E)                                                                                    \
   gemm_skinny_kernel<1, TO, false, E, true><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, \
                                                                         (TO*)y, ldy, nullptr, M, N, K, steps)
-    if (out_dtype == ME_BF16) { if (K % 128 == 0) LAUNCH_ACT(bf16_t, true); else LAUNCH_ACT(bf16_t, false); }
+    if (out_dtype == ME_BF16 && wide_ok) {
+      gemm_skinny_kernel<1, bf16_t, false, true, true, true><<<grid, block, 0, stream>>>(
+          (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, nullptr, M, N, K, steps);
+    } else if (out_dtype == ME_BF16) { if (K % 128 == 0) LAUNCH_ACT(bf16_t, true); else LAUNCH_ACT(bf16_t, false); }
     else if (out_dtype == ME_F32) { if (K % 128 == 0) LAUNCH_ACT(float, true); else LAUNCH_ACT(float, false); }
     else ME_CHECK(false, "skinny gemm: bad output dtype code %d", out_dtype);
 #undef LAUNCH_ACT
@@ -444,7 +487,14 @@ extern "C" int me_gemm_skinny_bf16(const void* x, int64_t ldx, const void* w, in
     if (exact) LAUNCH1(1, TO, true, true); else LAUNCH1(1, TO, true, false);                                 \
   } while (0)
   ME_CHECK(!gated || mt == 1, "skinny gemm: the gated form takes at most 16 rows (%d)", M);
-  if (out_dtype == ME_F32 || partials) {
+  if (wide_ok && (out_dtype == ME_F32 || out_dtype == ME_BF16 || partials)) {
+    if (out_dtype == ME_F32 || partials)
+      gemm_skinny_kernel<1, float, false, true, false, true><<<grid, block, 0, stream>>>(
+          (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (float*)y, ldy, partials, M, N, K, steps_per_split);
+    else
+      gemm_skinny_kernel<1, bf16_t, false, true, false, true><<<grid, block, 0, stream>>>(
+          (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, partials, M, N, K, steps_per_split);
+  } else if (out_dtype == ME_F32 || partials) {
     if (gated) LAUNCH_GATED(float); else if (mt == 4) LAUNCH(4, float); else if (mt == 2) LAUNCH(2, float); else LAUNCH(1, float);
   } else if (out_dtype == ME_BF16) {
     if (gated) LAUNCH_GATED(bf16_t); else if (mt == 4) LAUNCH(4, bf16_t); else if (mt == 2) LAUNCH(2, bf16_t); else LAUNCH(1, bf16_t);

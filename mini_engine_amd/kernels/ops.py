@@ -62,7 +62,7 @@ _CORE_PROTOS = {
     "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
-    "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, P],
+    "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
     "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_mid_bf16": [P, L, P, L, P, L, I, I, I, I, I, I, P],
@@ -448,12 +448,12 @@ class HipBackend:
         if ksplit > 1:
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
-                        ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, 0, _stream())
+                        ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, 0, skinny_wide(N, K), _stream())
             return parts
         if skinny_takes(M, N, K):
             y = new()
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
-                        _code(out_dtype), None, 1, M, N, K, 0, 0, _stream())
+                        _code(out_dtype), None, 1, M, N, K, 0, 0, skinny_wide(N, K), _stream())
             return y
         mid = mid_takes(M, N, K, allow_partials and out_dtype == x.dtype)
         if mid > 1:
@@ -484,7 +484,7 @@ class HipBackend:
                         ME_BF16, 1, M, N, K, 1, _stream())
             return y
         core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N // 2,
-                    ME_BF16, None, 1, M, N, K, 0, 1, _stream())
+                    ME_BF16, None, 1, M, N, K, 0, 1, skinny_wide(N, K), _stream())
         return y
 
     def norm_linear(self, x: torch.Tensor, residual: torch.Tensor | None, norm_weight: torch.Tensor, eps: float,
@@ -535,11 +535,11 @@ class HipBackend:
         if ksplit > 1:
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=gu.device)
             core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), None, N,
-                        ME_F32, parts.data_ptr(), ksplit, M, N, inter, 1, 0, _stream())
+                        ME_F32, parts.data_ptr(), ksplit, M, N, inter, 1, 0, 0, _stream())
             return parts
         y = torch.empty((M, N), dtype=gu.dtype, device=gu.device)
         core().call("me_gemm_skinny_bf16", gu.data_ptr(), gu.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
-                    ME_BF16, None, 1, M, N, inter, 1, 0, _stream())
+                    ME_BF16, None, 1, M, N, inter, 1, 0, 0, _stream())
         return y
 
     # -- sampling ------------------------------------------------------------------------
@@ -569,20 +569,29 @@ SKINNY_WIDE_MAX_M = 64
 SKINNY_WIDE_MAX_WEIGHT = 5 * 1024 * 1024
 PARTIALS_MAX_M = 64      # rows up to which a product split over K (float32 partial sums) pays
 LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go to the library at any M
-# Large weights with LIBRARY_MIN_ROWS or more rows go to the library: every workgroup of the skinny
-# kernel reads all of x, which at 8 to 16 rows is as much traffic as the weights themselves.
-# Measured with weights streamed from HBM (us, skinny / library), Qwen3-8B sizes:
-#   rows   qkv 6144x4096   o 4096x4096   gate_up 24576x4096   down 4096x12288
-#     1    13.1 / 14.5      8.3 / 15.4      39.3 / 45.8          21.2 / 22.6
-#     4    14.9 / 14.4      9.2 / 15.6      42.4 / 45.7          21.8 / 22.6
-#     8    15.6 / 14.4      9.1 / 15.5      47.1 / 46.3          24.7 / 22.9
-#    16    18.3 / 14.5     10.5 / 15.6      55.1 / 46.3          31.7 / 23.2
-#    32    27.2 / 15.2     15.3 / 13.1         -                 43.9 / 28.8
-# (o is below the size threshold.) At Qwen3-32B sizes, 8 rows: qkv 10240x5120 31.5 / 24.8,
-# o 5120x8192 29.2 / 20.8 (22.1 with K split in four), gate_up 51200x5120 130 / 95.3, but down
-# 5120x25600 66.8 (K split in four) / 137: the library's choice for a very long K is poor, hence
-# LIBRARY_MAX_K. All Qwen3-0.6B products favour the skinny kernel (3.3-5.5 us against 7.4-12 us).
+# Large weights go to the library from a row count on: every workgroup of the skinny kernel reads all of x, which
+# at 8 to 16 rows is as much traffic as the weights themselves. With its wide loads (skinny_wide: K in whole steps
+# of 128, up to 16 rows) the skinny kernel streams a large weight at 5.3-6.0 TB/s where the library reaches 4-5, and
+# stays ahead up to 16 rows over a K of up to 4,096 and up to 10 rows over a longer K. Measured with weights streamed
+# from HBM (us, skinny / library; gate_up with the gating: in the epilogue / a kernel behind the library's product):
+#   rows   qkv 6144x4096   o 4096x4096 (slices)   gate_up 24576x4096   down 4096x12288 (slices)
+#     1    11.3 / 14.5        7.9 / 15.4             33.6 / 48.8          18.2 / 21.8
+#     4    11.6 / 14.6        8.0 / 15.5             33.6 / 47.1          18.2 / 21.7
+#     8    12.4 / 14.5        8.2 / 15.5             34.6 / 47.0          19.0 / 21.7
+#    12    13.3 / 14.5        8.5 / 15.6             38.0 / 47.4          20.3 / 21.9
+#    16    14.6 / 14.5        9.0 / 15.5             42.2 / 47.3          22.6 / 22.3
+#   rows   qkv 10240x5120  o 5120x8192 (slices)   gate_up 51200x5120   gate_up 34816x5120   down 5120x25600 (slices)
+#     4    20.2 / 23.3       17.0 / 19.7             85.7 / 98.1          60.8 / 86.5          43.7 / 137
+#     8    22.4 / 23.7       17.3 / 20.2             94.8 / 98.5          64.3 / 80.2          47.3 / 138
+#    12    25.2 / 24.1       18.2 / 20.6            104.1 / 95.0          73.4 / 79.7          52.5 / 139
+#    16    29.0 / 24.5       19.7 / 21.2            119.8 / 95.4          84.0 / 81.0          60.5 / 140
+# (the library's choice for a very long K is poor, hence LIBRARY_MAX_K). Without the wide loads (K no multiple of
+# 128, or 17 rows and more) the library is level from 4 rows on: 6144x4096 at 4 / 8 / 16 / 32 rows 14.9 / 14.4,
+# 15.6 / 14.4, 18.3 / 14.5, 27.2 / 15.2; 24576x4096 42.4 / 45.7, 47.1 / 46.3, 55.1 / 46.3. All Qwen3-0.6B products
+# favour the skinny kernel (3.3-5.5 us against 7.4-12 us).
 LIBRARY_MIN_ROWS = 4
+LIBRARY_MIN_ROWS_WIDE = 17          # with the wide loads, K up to 4,096: never within their 16 rows
+LIBRARY_MIN_ROWS_WIDE_LONG_K = 11   # ... over a longer K
 LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
 LIBRARY_MAX_K = 16384
 ROWS_MIN_WEIGHT = 16 * 1024 * 1024
@@ -694,6 +703,20 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D:
     return seg, -(-span // seg) + 1
 
 
+SKINNY_WIDE_MIN_WEIGHT = 1 << 22
+
+
+def skinny_wide(N: int, K: int) -> int:
+    """Whether the skinny product reads a weight [N, K] with its wide loads: a wave's load takes 256 contiguous bytes
+    of each of four rows, marked as not to be kept by the caches, and the pieces reach their lanes through LDS. For
+    weights of SKINNY_WIDE_MIN_WEIGHT elements or more (the kernel applies them to up to 16 rows and a K in whole
+    steps of 128). us, plain / wide, weights cold, the same bits: 24576 x 4096 with the gating at 1 / 3 / 8 rows
+    39.0 / 33.6, 41.1 / 33.9, 47.2 / 36.0; 4096 x 12288 in slices 21.8 / 18.8, 22.1 / 18.9; 5120 x 25600 53.0 / 44.5,
+    57.2 / 44.8; 6144 x 4096 13.1 / 11.2; 4096 x 4096 in slices 8.3 / 7.8; 6144 x 1024 at 1 / 8 rows 4.8 / 4.6, 5.4 /
+    5.0; 4096 x 1024 3.7 / 3.7 (small weights are over before the mark matters)."""
+    return 1 if N * K >= SKINNY_WIDE_MIN_WEIGHT else 0
+
+
 def skinny_takes(M: int, N: int, K: int) -> bool:
     """Whether the skinny kernel (without a split over K) takes an aligned bfloat16 product."""
     rows_ok = M <= SKINNY_MAX_M or (M <= SKINNY_WIDE_MAX_M and N * K <= SKINNY_WIDE_MAX_WEIGHT)
@@ -733,7 +756,9 @@ def rows_takes(M: int, N: int, K: int) -> bool:
     """Whether a product whose consumer adds float32 partial sums goes to the rows kernel (64 features per
     workgroup, the tokens staged once per workgroup in LDS, K split over up to 8 workgroups): large
     weights with 17 to 64 rows, where the skinny kernel reads the tokens again for every 16 features and
-    the library streams at 1.7-3.5 TB/s, and from 8 rows on over a K too long for the library.
+    the library streams at 1.7-3.5 TB/s, and from 8 rows on over a K too long for the library that is no multiple
+    of 128 (otherwise the skinny kernel's wide loads are ahead up to 16 rows: 5120 x 25600 at 8 / 16 rows 47.3 / 60.5
+    us against 63.2 here at 8).
     Measured, us (rows kernel / best of library and skinny), weights from HBM:
       4096 x 4096:   24 rows 10.6 / 13.2,  48 rows 13.5 / 13.6,  64 rows 14.6 / 15.0
       4096 x 12288:  24 rows 25.0 / 26.9,  48 rows 30.2 / 33.6,  64 rows 31.7 / 37.3
@@ -744,7 +769,7 @@ def rows_takes(M: int, N: int, K: int) -> bool:
         return False
     if M > 16:
         return M <= 32 or K >= 12288
-    return M >= 8 and K > LIBRARY_MAX_K
+    return M >= 8 and K > LIBRARY_MAX_K and not (K % 128 == 0 and skinny_wide(N, K))
 
 
 def rows_ksplit(K: int) -> int:
@@ -758,7 +783,11 @@ def rows_ksplit(K: int) -> int:
 
 def library_streams_better(M: int, N: int, K: int) -> bool:
     """Whether a product of few rows goes to the library rather than the skinny kernel."""
-    return M >= LIBRARY_MIN_ROWS and N * K >= LIBRARY_MIN_WEIGHT and K <= LIBRARY_MAX_K
+    if N * K < LIBRARY_MIN_WEIGHT or K > LIBRARY_MAX_K:
+        return False
+    if K % 128 == 0 and M <= 16 and skinny_wide(N, K):
+        return M >= (LIBRARY_MIN_ROWS_WIDE if K <= 4096 else LIBRARY_MIN_ROWS_WIDE_LONG_K)
+    return M >= LIBRARY_MIN_ROWS
 
 
 def choose_ksplit(M: int, N: int, K: int) -> int:
@@ -875,10 +904,10 @@ def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     if not FUSE_GATE_INTO_GATE_UP or w.dtype != torch.bfloat16 or w.dim() != 2:
         return False
     N, K = w.shape
-    # over large weights the library takes products of 4 rows or more, and the gating is then a kernel of its own;
-    # up to 8 rows over a K of 4,096 the skinny kernel with the gating in its epilogue is still ahead of the two
-    # (4096 -> 24576, us: 4 rows 38.9 / 45.5, 6 rows 41.4 / 45.6, 8 rows 43.9 / 45.5, 12 rows 49.2 / 46.2; over a K of
-    # 5,120 the library is level or ahead from 4 rows on: 5120 -> 34816, 4 rows 75.0 / 76.4, 6 rows 81.2 / 76.5)
+    # over large weights the library takes the product from a row count on (library_streams_better), and the gating is
+    # then a kernel of its own; without the skinny kernel's wide loads (K no multiple of 128) the skinny kernel with the
+    # gating in its epilogue is still ahead of the two up to 8 rows over a K of 4,096 (4096 -> 24576, us: 4 rows 38.9 /
+    # 45.5, 8 rows 43.9 / 45.5, 12 rows 49.2 / 46.2)
     takes = skinny_takes(rows, N, K) or (rows <= 8 and K <= 4096 and N < LIBRARY_MIN_N and rows <= SKINNY_MAX_M)
     aligned = N % 2 == 0 and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
     if rows > GATED_EPILOGUE_MAX_M:

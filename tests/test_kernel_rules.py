@@ -92,7 +92,10 @@ def test_ksplit_keeps_512_of_k_per_split_and_fills_the_gpu():
 def test_large_weights_with_several_rows_go_to_the_library():
     assert not ops.library_streams_better(1, 24576, 4096)              # one row: the skinny kernel
     assert not ops.library_streams_better(2, 24576, 4096)              # two rows: still level
-    assert ops.library_streams_better(8, 24576, 4096)
+    assert not ops.library_streams_better(16, 24576, 4096)             # up to 16 rows the skinny kernel's wide loads are ahead
+    assert ops.library_streams_better(17, 24576, 4096)
+    assert not ops.library_streams_better(10, 51200, 5120) and ops.library_streams_better(11, 51200, 5120)   # a longer K: up to 10
+    assert ops.library_streams_better(8, 24576, 4000)                  # K no multiple of 128: no wide loads, the library from 4 rows
     assert not ops.library_streams_better(8, 4096, 4096)               # below the size threshold
     assert not ops.library_streams_better(8, 5120, 25600)              # very long K: the library's choice is poor
     assert not ops.library_streams_better(16, 6144, 1024)
@@ -102,7 +105,7 @@ def test_skinny_kernel_takes_few_rows():
     assert ops.skinny_takes(32, 6144, 1024) and not ops.skinny_takes(33, 6144, 1024)
     assert ops.skinny_takes(64, 4096, 1024) and not ops.skinny_takes(65, 4096, 1024)
     assert not ops.skinny_takes(1, 151936, 1024)                       # the head goes to the library
-    assert not ops.skinny_takes(8, 24576, 4096)
+    assert ops.skinny_takes(16, 24576, 4096) and not ops.skinny_takes(17, 24576, 4096)   # large weights: as far as the wide loads go
 
 
 def test_rows_kernel_takes_many_rows_over_large_weights():
@@ -110,7 +113,8 @@ def test_rows_kernel_takes_many_rows_over_large_weights():
     assert ops.rows_takes(32, 4096, 12288) and ops.rows_takes(32, 5120, 8192) and not ops.rows_takes(64, 5120, 8192)
     assert not ops.rows_takes(64, 4096, 12288)       # from 33 rows the library's slices of K take these weights
     assert ops.rows_takes(64, 1400, 12296)           # ... unless K has no equal slices of a multiple of 8
-    assert ops.rows_takes(8, 5120, 25600) and not ops.rows_takes(4, 5120, 25600)     # few rows: only where the library is out
+    assert not ops.rows_takes(8, 5120, 25600) and not ops.rows_takes(4, 5120, 25600)   # few rows: the skinny kernel's wide loads
+    assert ops.rows_takes(8, 5120, 25608)                                              # ... unless K is no multiple of 128
     assert not ops.rows_takes(8, 4096, 12288) and not ops.rows_takes(64, 1024, 3072) and not ops.rows_takes(65, 5120, 25600)
     for K in (4096, 4104, 9728, 12288, 25600):
         ks, chunks = ops.rows_ksplit(K), -(-K // 512)

@@ -474,6 +474,33 @@ def test_linear_skinny_bf16(M, N, K):
     close(parts.sum(0) if parts.dim() == 3 else parts, ref, 6e-3 if parts.dim() == 2 else 2e-5)
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K", [(4100, 1024), (1024, 4096), (8200, 512), (2056, 2048)])
+def test_linear_skinny_wide_loads(monkeypatch, M, N, K):
+    """Weights of 4 M elements or more, up to 16 rows, K in whole steps of 128: a wave's load takes 256 contiguous bytes
+    of each of four rows and the pieces reach their lanes through LDS. The same bits as the plain loads give, for one
+    result, partial sums over slices of K and the gating epilogue; a last workgroup with fewer than 16 rows (or 8 gate
+    features); rows of x and w that are longer than K."""
+    assert ops.skinny_wide(N, K) and ops.skinny_takes(M, N, K)
+    torch.manual_seed(M + N)
+    x = torch.randn(M, K + 64, device=DEV).bfloat16()[:, :K]
+    w = (torch.randn(N, K + 128, device=DEV) * 0.05).bfloat16()[:, :K]
+    ref = x.double() @ w.double().t()
+    def all_forms():
+        parts = hip().linear(x, w, None, allow_partials=True)
+        return (hip().linear(x, w), hip().linear(x, w, torch.float32), parts, hip().gated_linear(x, w))
+    wide = all_forms()
+    monkeypatch.setattr(ops, "SKINNY_WIDE_MIN_WEIGHT", 1 << 40)
+    plain = all_forms()
+    for a, b in zip(wide, plain):
+        assert a.shape == b.shape and torch.equal(a, b)
+    close(wide[0], ref, 6e-3)
+    close(wide[1], ref, 2e-5)
+    close(wide[2].sum(0) if wide[2].dim() == 3 else wide[2], ref, 6e-3 if wide[2].dim() == 2 else 2e-5)
+    assert wide[2].dim() == (3 if ops.choose_ksplit(M, N, K) > 1 else 2)
+    close(wide[3], twin.gated_linear(x, w, compute_dtype=torch.float64), 6e-3)
+
+
 @pytest.mark.parametrize("M", [1, 2])
 @pytest.mark.parametrize("N,K", [(4096, 1024), (6144, 1024), (384, 80), (1000, 224), (100, 2048), (1536, 4096)])
 @pytest.mark.parametrize("S", [0, 1, 6])
@@ -583,7 +610,7 @@ def test_linear_partials_are_used_where_tiles_are_few():
         close(parts.sum(0), x.double() @ w.double().t(), 2e-5)
 
 
-@pytest.mark.parametrize("M,N,K", [(24, 4096, 4096), (17, 4100, 4104), (20, 4000, 4224), (64, 1400, 12296), (32, 1368, 12288), (9, 1000, 16896)])
+@pytest.mark.parametrize("M,N,K", [(24, 4096, 4096), (17, 4100, 4104), (20, 4000, 4224), (64, 1400, 12296), (32, 1368, 12288), (9, 1000, 16904)])
 def test_linear_rows_kernel(M, N, K):
     """17 to 64 rows over large weights (and fewer over a very long K), partial sums allowed: 64 features per
     workgroup, the tokens staged in LDS chunk by chunk; feature counts and K that are no multiples of 64, 128 or 512."""
