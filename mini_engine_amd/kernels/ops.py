@@ -568,7 +568,13 @@ SKINNY_MAX_M = 32
 SKINNY_WIDE_MAX_M = 64
 SKINNY_WIDE_MAX_WEIGHT = 5 * 1024 * 1024
 PARTIALS_MAX_M = 64      # rows up to which a product split over K (float32 partial sums) pays
-LIBRARY_MIN_N = 32768    # outputs this wide (the head over the vocabulary) go to the library at any M
+# Outputs this wide (the head over the vocabulary, gate/up of the largest sizes) go to the library, except up to
+# WIDE_OUTPUT_SKINNY_ROWS rows where the skinny kernel's wide loads apply (us, skinny to float32 / library: 151936 x 1024
+# at 1 / 8 / 12 / 16 rows 47.8 / 59.9, 51.0 / 62.3, 60.1 / 64.4, 67.9 / 66.3; 151936 x 2560 125 / 249, 141 / 246, 165 / 246,
+# 187 / 246; 151936 x 4096 182 / 252 (6.8 TB/s), 199 / 252, 224 / 257, 253 / 259; 151936 x 5120 231 / 308, 261 / 305, 306 /
+# 313, 355 / 318)
+LIBRARY_MIN_N = 32768
+WIDE_OUTPUT_SKINNY_ROWS = 12
 # Large weights go to the library from a row count on: every workgroup of the skinny kernel reads all of x, which
 # at 8 to 16 rows is as much traffic as the weights themselves. With its wide loads (skinny_wide: K in whole steps
 # of 128, up to 16 rows) the skinny kernel streams a large weight at 5.3-6.0 TB/s where the library reaches 4-5, and
@@ -720,7 +726,9 @@ def skinny_wide(N: int, K: int) -> int:
 def skinny_takes(M: int, N: int, K: int) -> bool:
     """Whether the skinny kernel (without a split over K) takes an aligned bfloat16 product."""
     rows_ok = M <= SKINNY_MAX_M or (M <= SKINNY_WIDE_MAX_M and N * K <= SKINNY_WIDE_MAX_WEIGHT)
-    return rows_ok and N < LIBRARY_MIN_N and not library_streams_better(M, N, K)
+    if N >= LIBRARY_MIN_N:
+        rows_ok = M <= WIDE_OUTPUT_SKINNY_ROWS and K % 128 == 0 and skinny_wide(N, K) == 1
+    return rows_ok and not library_streams_better(M, N, K)
 
 
 LIBRARY_SPLIT_MIN_ROWS = 33

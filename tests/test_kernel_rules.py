@@ -104,7 +104,9 @@ def test_large_weights_with_several_rows_go_to_the_library():
 def test_skinny_kernel_takes_few_rows():
     assert ops.skinny_takes(32, 6144, 1024) and not ops.skinny_takes(33, 6144, 1024)
     assert ops.skinny_takes(64, 4096, 1024) and not ops.skinny_takes(65, 4096, 1024)
-    assert not ops.skinny_takes(1, 151936, 1024)                       # the head goes to the library
+    assert ops.skinny_takes(1, 151936, 1024) and ops.skinny_takes(12, 151936, 4096)      # the head: up to 12 rows with the wide loads
+    assert not ops.skinny_takes(13, 151936, 1024) and not ops.skinny_takes(1, 151936, 1000)  # ... else the library
+    assert ops.skinny_takes(10, 151936, 5120) and not ops.skinny_takes(11, 151936, 5120)  # a longer K: up to 10
     assert ops.skinny_takes(16, 24576, 4096) and not ops.skinny_takes(17, 24576, 4096)   # large weights: as far as the wide loads go
 
 
