@@ -300,12 +300,17 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
 #define ROWS_GRANULES (ROWS_CHUNK / 8)
 
 // EXACT_K: K is a multiple of the chunk, so neither a step nor a staged granule lies beyond K.
-template <int MT, typename TO, bool EXACT_K>
+// WIDE (EXACT_K only): the weights are read as in the skinny kernel's wide form: a wave's load takes 256 contiguous
+// bytes of each of four of its rows, marked as not to be kept by the caches, and the pieces pass through the wave's
+// own 16 x 272 bytes of LDS to the lanes that the matrix instruction wants them in.
+template <int MT, typename TO, bool EXACT_K, bool WIDE = false>
 __global__ void __launch_bounds__(256)
 gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                  TO* __restrict__ y, int64_t ldy, float* __restrict__ partials, int M, int N, int K,
                  int chunks_per_split) {
+  static_assert(!WIDE || EXACT_K, "the wide loads are built for whole steps");
   extern __shared__ __align__(16) unsigned char rows_lds[];
+  __shared__ __align__(16) unsigned char wtile[WIDE ? 4 : 1][WIDE ? 16 * 272 : 16];
   bf16_t* xs = reinterpret_cast<bf16_t*>(rows_lds);     // [16 * MT][ROWS_CHUNK]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -318,12 +323,20 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __rest
   const bf16x8 z = gz8();
   const int rows = min(M, 16 * MT);
 
+  const uint32_t ldw_bytes = (uint32_t)ldw * 2u;        // WIDE: byte offsets from w (the launcher admits weights under 2 GB)
   auto fetch = [&](int s, bool live, bf16x8 (&a)[4]) {
     const int kb = 128 * s + 8 * g;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int k = kb + 32 * j;
-      a[j] = *reinterpret_cast<const bf16x8*>(live && (EXACT_K || k < K) ? wrow + k : w);
+      if (WIDE) {
+        // load j of lane (piece r, g): piece r of the step from row 4 j + g of the wave's sixteen
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const uint32_t off = live ? (uint32_t)min(n0 + 4 * j + g, N - 1) * ldw_bytes + 16u * (uint32_t)r + 256u * (uint32_t)s : 0u;
+        a[j] = __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(w) + off)));
+      } else {
+        const int k = kb + 32 * j;
+        a[j] = *reinterpret_cast<const bf16x8*>(live && (EXACT_K || k < K) ? wrow + k : w);
+      }
     }
   };
   f32x4 acc[MT];
@@ -364,10 +377,21 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __rest
       fetch(s + 1, s + 1 <= s_last, ring[(u + 1) & 1]);
       pin_loads();
       if (s <= s_last) {
+        bf16x8 wide_a[4];
+        if (WIDE) {
+          // the wave's LDS operations run in the order they are issued: what its lanes write here, its lanes read below
+          unsigned char* tile = wtile[wave];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) *reinterpret_cast<bf16x8*>(tile + (g * 272 + r * 16) + j * (4 * 272)) = ring[u & 1][j];
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int j = 0; j < 4; ++j) wide_a[j] = *reinterpret_cast<const bf16x8*>(tile + (r * 272 + g * 16) + j * 64);
+          asm volatile("" ::: "memory");
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const bool kok = EXACT_K || 128 * s + 32 * j + 8 * g < K;
-          const bf16x8 a = kok ? ring[u & 1][j] : z;
+          const bf16x8 a = WIDE ? wide_a[j] : (kok ? ring[u & 1][j] : z);
           const int q = 16 * u + 4 * j + g;           // granule of k = 128 s + 32 j + 8 g inside the chunk
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
@@ -395,8 +419,10 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __rest
   }
 }
 
+// wide: the caller asks for the wide loads; they apply to a K in whole chunks and a weight under 2 GB.
 extern "C" int me_gemm_rows_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
-                                 int out_dtype, float* partials, int ksplit, int M, int N, int K, hipStream_t stream) {
+                                 int out_dtype, float* partials, int ksplit, int M, int N, int K, int wide,
+                                 hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   ME_CHECK(M <= 64, "rows gemm: at most 64 rows (%d)", M);
   ME_CHECK(K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0,
@@ -414,7 +440,14 @@ extern "C" int me_gemm_rows_bf16(const void* x, int64_t ldx, const void* w, int6
 #define LAUNCH1(MTV, TO, E)                                                                                     \
   gemm_rows_kernel<MTV, TO, E><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, \
                                                              ldy, partials, M, N, K, chunks_per_split)
-#define LAUNCH2(MTV, TO) do { if (exact) LAUNCH1(MTV, TO, true); else LAUNCH1(MTV, TO, false); } while (0)
+#define LAUNCH_WIDE(MTV, TO)                                                                                          \
+  gemm_rows_kernel<MTV, TO, true, true><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,   \
+                                                                      (TO*)y, ldy, partials, M, N, K, chunks_per_split)
+  const bool wide_ok = wide && exact && (int64_t)(N - 1) * ldw + K <= (int64_t)0x3fffffff;
+#define LAUNCH2(MTV, TO)                                                                                       \
+  do {                                                                                                         \
+    if (wide_ok) LAUNCH_WIDE(MTV, TO); else if (exact) LAUNCH1(MTV, TO, true); else LAUNCH1(MTV, TO, false);   \
+  } while (0)
 #define LAUNCH(TO)                                                                             \
   do {                                                                                         \
     if (mt == 1) LAUNCH2(1, TO); else if (mt == 2) LAUNCH2(2, TO); else if (mt == 3) LAUNCH2(3, TO); \
@@ -425,6 +458,7 @@ extern "C" int me_gemm_rows_bf16(const void* x, int64_t ldx, const void* w, int6
   else ME_CHECK(false, "rows gemm: bad output dtype code %d", out_dtype);
 #undef LAUNCH
 #undef LAUNCH2
+#undef LAUNCH_WIDE
 #undef LAUNCH1
   ME_LAUNCH_CHECK();
   return 0;

@@ -63,7 +63,7 @@ _CORE_PROTOS = {
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, I, P],
-    "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, P],
+    "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
     "me_gemm_skinny_norm_bf16": [P, I, I, P, P, P, F, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_mid_bf16": [P, L, P, L, P, L, I, I, I, I, I, I, P],
     "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
@@ -441,7 +441,7 @@ class HipBackend:
             ksplit = rows_ksplit(K)
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
             core().call("me_gemm_rows_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
-                        ME_F32, parts.data_ptr(), ksplit, M, N, K, _stream())
+                        ME_F32, parts.data_ptr(), ksplit, M, N, K, rows_wide(M, N, ksplit), _stream())
             return parts
         ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype
                                             and not library_streams_better(M, N, K)) else 1
@@ -778,6 +778,17 @@ def rows_takes(M: int, N: int, K: int) -> bool:
     if M > 16:
         return M <= 32 or K >= 12288
     return M >= 8 and K > LIBRARY_MAX_K and not (K % 128 == 0 and skinny_wide(N, K))
+
+
+def rows_wide(M: int, N: int, ksplit: int) -> int:
+    """Whether the rows kernel reads its weights with the wide loads of the skinny kernel (`skinny_wide`): up to 32
+    rows and with two workgroups or more to a compute unit. The pass through LDS lengthens a wave's chain from load
+    to product, which other workgroups on the compute unit must fill, and the wave tiles' 17 KB beside 48-64 KB of
+    staged tokens leave room for one workgroup only. us, plain / wide, in 8 slices of K: 4096 x 4096 at 17 / 32 rows
+    10.4 / 9.8, 11.4 / 10.8; 4096 x 12288 24.2 / 22.3, 25.7 / 23.8; 5120 x 8192 22.4 / 19.3, 24.2 / 21.6; 5120 x 25600
+    67.5 / 53.8, 69.8 / 56.5; at 48 / 64 rows 4096 x 12288 30.0 / 29.4, 31.5 / 46.3; unsplit (96-384 workgroups):
+    6144 x 4096 at 17 rows 26.2 / 33.3, 24576 x 4096 52.2 / 49.0, at 64 rows 63.8 / 108."""
+    return 1 if M <= 32 and -(-N // 64) * ksplit >= 2 * _COMPUTE_UNITS else 0
 
 
 def rows_ksplit(K: int) -> int:

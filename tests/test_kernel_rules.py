@@ -110,6 +110,11 @@ def test_skinny_kernel_takes_few_rows():
     assert ops.skinny_takes(16, 24576, 4096) and not ops.skinny_takes(17, 24576, 4096)   # large weights: as far as the wide loads go
 
 
+def test_rows_kernel_reads_wide_with_few_rows_and_many_workgroups():
+    assert ops.rows_wide(24, 4096, 8) == 1 and ops.rows_wide(32, 5120, 8) == 1
+    assert ops.rows_wide(33, 4096, 8) == 0 and ops.rows_wide(24, 6144, 1) == 0 and ops.rows_wide(24, 4096, 4) == 0
+
+
 def test_rows_kernel_takes_many_rows_over_large_weights():
     assert ops.rows_takes(24, 4096, 4096) and not ops.rows_takes(64, 4096, 4096)     # above 32 rows only over a long K
     assert ops.rows_takes(32, 4096, 12288) and ops.rows_takes(32, 5120, 8192) and not ops.rows_takes(64, 5120, 8192)

@@ -625,6 +625,21 @@ def test_linear_rows_kernel(M, N, K):
     close(hip().linear(xs, w, None, allow_partials=True).sum(0), xs.double() @ w.double().t(), 2e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(24, 4096, 4096), (20, 4100, 4096), (32, 4160, 4096), (17, 5120, 8192)])
+def test_linear_rows_kernel_wide_loads(monkeypatch, M, N, K):
+    """The rows kernel with the weights read 256 contiguous bytes of four rows a load and passed through LDS (up to 32
+    rows, two workgroups or more to a compute unit, K in whole chunks): the same bits as with the plain loads; a last
+    workgroup whose waves have few rows or none; weight rows longer than K."""
+    assert ops.rows_takes(M, N, K) and ops.rows_wide(M, N, ops.rows_ksplit(K)) == 1
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K + 64, device=DEV) * 0.05).bfloat16()[:, :K]
+    wide = hip().linear(x, w, None, allow_partials=True)
+    monkeypatch.setattr(ops, "rows_wide", lambda *a: 0)
+    plain = hip().linear(x, w, None, allow_partials=True)
+    assert wide.shape == (ops.rows_ksplit(K), M, N) and torch.equal(wide, plain)
+    close(wide.sum(0), x.double() @ w.double().t(), 2e-5)
+
+
 @pytest.mark.parametrize("M,N,K", [(65, 4096, 1024), (256, 6144, 1024), (130, 1024, 2048), (200, 1024, 3072), (512, 1024, 2048),
                                    (100, 1000, 320), (40, 6144, 1024), (70, 68, 256), (77, 1028, 2112)])
 def test_linear_a_few_hundred_rows_over_small_weights(M, N, K):
