@@ -9,7 +9,8 @@
 //  * me_gemm_skinny_bf16: the decode product, up to 64 rows (the caller decides from which row
 //    count the library is faster). Pure weight streaming: each workgroup owns 16 output features, its 4 waves split
 //    K, a wave reads 256 contiguous bytes of each of its 16 weight rows per step (each load takes 64
-//    contiguous bytes per row), the fetches run one step ahead of the products, products on
+//    contiguous bytes per row; over large weights 256 contiguous bytes of each of four rows, see the wide loads
+//    below), the fetches run one step ahead of the products, products on
 //    v_mfma_f32_16x16x32_bf16 with the tokens as the 16-wide B operand, waves merged through
 //    LDS. Optional split of K over workgroups writes float32 partial sums [S, M, N] that the
 //    consumer (the fused residual + RMSNorm kernel) adds in a fixed order.
@@ -103,6 +104,30 @@ __device__ __forceinline__ bf16x8 silu_mul8(const bf16x8 g, const bf16x8 u) {
   return r;
 }
 
+// ---- wide loads of a weight that a launch reads once (skinny and rows kernels, large weights)
+// A load of a wave in the plain pattern takes 64 bytes of each of sixteen rows, so that a row's 128-byte line is
+// asked for by two loads; marked as not to be kept by the caches, the second asks the memory again, and the mark,
+// which this GPU's memory answers with a higher rate, gains nothing. In the wide pattern load j of lane (piece r, g)
+// takes piece r (16 bytes) of the step's 256 bytes from row 4 j + g of the wave's sixteen: whole lines, marked.
+// The pieces then pass through a tile of the wave's own in LDS, 16 rows 272 bytes apart (so that the 16 rows a read
+// takes at once are spread over all banks, and every address is a lane's base plus a constant), to the lanes that
+// the matrix instruction wants them in: lane (row r, g) gets the pieces 4 j + g of row r. A wave's LDS operations
+// run in the order they are issued, so what its lanes write, its lanes read behind it without a barrier.
+#define WIDE_TILE_BYTES (16 * 272)
+__device__ __forceinline__ bf16x8 wide_load(const bf16_t* w, uint32_t byte_offset) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  return __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                                        reinterpret_cast<const unsigned char*>(w) + byte_offset)));
+}
+__device__ __forceinline__ void wide_to_lanes(unsigned char* tile, int r, int g, const bf16x8 (&loaded)[4], bf16x8 (&a)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) *reinterpret_cast<bf16x8*>(tile + (g * 272 + r * 16) + j * (4 * 272)) = loaded[j];
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int j = 0; j < 4; ++j) a[j] = *reinterpret_cast<const bf16x8*>(tile + (r * 272 + g * 16) + j * 64);
+  asm volatile("" ::: "memory");
+}
+
 // One macro step's operands. Loads are unconditional (a row or a k beyond the matrix is read from
 // row 0 / k 0 instead and zeroed afterwards), so they all go out together and the next step's
 // loads are in flight while this step's products run.
@@ -132,11 +157,8 @@ struct SkinnyOperands {
 // layers/linear.py:29-45), and y is silu(gate) * up, [M, I] (layers/activation.py:5-7): a workgroup takes 8 gate
 // features and the 8 up features that go with them as the 16 rows of its matrix operand and pairs them when it
 // merges its waves, so every gate is formed once, from the unrounded sums.
-// WIDE (one tile of tokens, EXACT_K, not GATED; for large weights): a load of a wave takes whole rows of the step,
-// 256 contiguous bytes of each of four weight rows, marked as not to be kept by the caches, instead of 64 bytes of
-// each of sixteen: only loads that take whole 128-byte lines gain by the mark (a kernel that only reads a 201-524 MB
-// weight: 5.3-6.1 TB/s in the plain pattern, 5.9-6.9 so), and the pieces then pass through a wave's own 4 KB of LDS to
-// reach the lanes that the matrix instruction wants them in.
+// WIDE (one tile of tokens, EXACT_K, not GATED; for large weights): the weights come by the wide loads above (a
+// kernel that only reads a 201-524 MB weight: 5.3-6.1 TB/s in the plain pattern, 5.9-6.9 so).
 template <int MT, typename TO, bool GATED, bool EXACT_K, bool ACT = false, bool WIDE = false>
 __global__ void __launch_bounds__(256, WIDE ? 5 : 1)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
@@ -144,9 +166,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
                    int steps_per_split) {
   static_assert(!WIDE || (MT == 1 && !GATED && EXACT_K), "the wide loads are built for one tile of tokens and whole steps");
   __shared__ float red[4][MT][256];
-  // WIDE: per wave 16 rows of 16 pieces of 16 bytes, a row 272 bytes from the next, so that the 16 rows a read takes
-  // at once are spread over all banks and every address is a lane's base plus a constant
-  __shared__ __align__(16) unsigned char wtile[WIDE ? 4 : 1][WIDE ? 16 * 272 : 16];
+  __shared__ __align__(16) unsigned char wtile[WIDE ? 4 : 1][WIDE ? WIDE_TILE_BYTES : 16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * (ACT ? 8 : 16), m0 = blockIdx.y * 16 * MT;
@@ -191,9 +211,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
       const int k = kb + 32 * j;
       const int ks = (EXACT_K || k < K) ? k : 0;
       if (WIDE) {
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        const uint32_t off = live ? wide_offset(j, s) : 0u;
-        op.a[j] = __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(w) + off)));
+        op.a[j] = wide_load(w, live ? wide_offset(j, s) : 0u);
       } else {
         op.a[j] = *reinterpret_cast<const bf16x8*>(live ? wrow + ks : w);
       }
@@ -207,16 +225,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
   auto product = [&](int s, const SkinnyOperands<MT, GATED>& op) {
     const int kb = 128 * s + 8 * g;
     bf16x8 wide_a[4];
-    if (WIDE) {
-      // the wave's LDS operations run in the order they are issued: what its lanes write here, its lanes read below
-      unsigned char* tile = wtile[wave];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) *reinterpret_cast<bf16x8*>(tile + (g * 272 + r * 16) + j * (4 * 272)) = op.a[j];
-      asm volatile("" ::: "memory");
-#pragma unroll
-      for (int j = 0; j < 4; ++j) wide_a[j] = *reinterpret_cast<const bf16x8*>(tile + (r * 272 + g * 16) + j * 64);
-      asm volatile("" ::: "memory");
-    }
+    if (WIDE) wide_to_lanes(wtile[wave], r, g, op.a, wide_a);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const bool kok = EXACT_K || kb + 32 * j < K;
@@ -300,9 +309,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __re
 #define ROWS_GRANULES (ROWS_CHUNK / 8)
 
 // EXACT_K: K is a multiple of the chunk, so neither a step nor a staged granule lies beyond K.
-// WIDE (EXACT_K only): the weights are read as in the skinny kernel's wide form: a wave's load takes 256 contiguous
-// bytes of each of four of its rows, marked as not to be kept by the caches, and the pieces pass through the wave's
-// own 16 x 272 bytes of LDS to the lanes that the matrix instruction wants them in.
+// WIDE (EXACT_K only): the weights come by the wide loads, as in the skinny kernel.
 template <int MT, typename TO, bool EXACT_K, bool WIDE = false>
 __global__ void __launch_bounds__(256)
 gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
@@ -310,7 +317,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __rest
                  int chunks_per_split) {
   static_assert(!WIDE || EXACT_K, "the wide loads are built for whole steps");
   extern __shared__ __align__(16) unsigned char rows_lds[];
-  __shared__ __align__(16) unsigned char wtile[WIDE ? 4 : 1][WIDE ? 16 * 272 : 16];
+  __shared__ __align__(16) unsigned char wtile[WIDE ? 4 : 1][WIDE ? WIDE_TILE_BYTES : 16];
   bf16_t* xs = reinterpret_cast<bf16_t*>(rows_lds);     // [16 * MT][ROWS_CHUNK]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -329,10 +336,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __rest
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (WIDE) {
-        // load j of lane (piece r, g): piece r of the step from row 4 j + g of the wave's sixteen
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        const uint32_t off = live ? (uint32_t)min(n0 + 4 * j + g, N - 1) * ldw_bytes + 16u * (uint32_t)r + 256u * (uint32_t)s : 0u;
-        a[j] = __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(w) + off)));
+        a[j] = wide_load(w, live ? (uint32_t)min(n0 + 4 * j + g, N - 1) * ldw_bytes + 16u * (uint32_t)r + 256u * (uint32_t)s : 0u);
       } else {
         const int k = kb + 32 * j;
         a[j] = *reinterpret_cast<const bf16x8*>(live && (EXACT_K || k < K) ? wrow + k : w);
@@ -378,16 +382,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __rest
       pin_loads();
       if (s <= s_last) {
         bf16x8 wide_a[4];
-        if (WIDE) {
-          // the wave's LDS operations run in the order they are issued: what its lanes write here, its lanes read below
-          unsigned char* tile = wtile[wave];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) *reinterpret_cast<bf16x8*>(tile + (g * 272 + r * 16) + j * (4 * 272)) = ring[u & 1][j];
-          asm volatile("" ::: "memory");
-#pragma unroll
-          for (int j = 0; j < 4; ++j) wide_a[j] = *reinterpret_cast<const bf16x8*>(tile + (r * 272 + g * 16) + j * 64);
-          asm volatile("" ::: "memory");
-        }
+        if (WIDE) wide_to_lanes(wtile[wave], r, g, ring[u & 1], wide_a);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const bool kok = EXACT_K || 128 * s + 32 * j + 8 * g < K;
