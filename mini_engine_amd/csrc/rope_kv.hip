@@ -233,9 +233,9 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, int64_t row_stride, const flo
 // The same arithmetic for steps with many tokens (prefill). Grid (groups of 8 consecutive tokens,
 // q/k workgroups + one value workgroup). q and k heads: LPH = D/16 lanes share a head, a lane reads 8 values of each
 // half (16 bytes), their 8 (cos, sin), and writes both back. Value heads: a thread takes 8 channels
-// of a head, reads them for the 8 tokens, transposes the 8x8 block in registers and writes one
-// 16-byte piece per channel into the transposed page (when the 8 slots are consecutive places of
-// one page, starting at a multiple of 8; otherwise value by value).
+// of a head, reads them for 8 tokens, transposes the 8x8 block in registers and writes one
+// 16-byte piece per channel into the transposed page (for 8 tokens whose slots are consecutive places of
+// one page, starting at a multiple of 8, wherever in the batch their rows begin; otherwise value by value).
 typedef bf16_t bf16x8r __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4r __attribute__((ext_vector_type(4)));
 
@@ -309,40 +309,48 @@ qk_norm_rope_store_tile_kernel(bf16_t* __restrict__ qkv, int64_t row_stride, con
     return;
   }
   // ---- value heads: the last workgroup of the 8 tokens
-  const int s0 = slots[t0];
-  bool run = cnt == 8 && s0 >= 0 && (s0 & 7) == 0;
-  if (run) {
-#pragma unroll
-    for (int i = 1; i < 8; ++i) run = run && slots[t0 + i] == s0 + i;
-  }
+  // The values go into the transposed page [channel][place]. Eight tokens whose slots are the eight places of an
+  // aligned group (consecutive, the first a multiple of 8) are written as one 16-byte piece per channel. Which rows
+  // of the batch form such a group has nothing to do with where the workgroups' rows begin (decode rows stand in
+  // front of the prompts' rows, a prompt is cut where the token budget ends), so the groups are found from the
+  // slots: a row begins a group if its slot is a multiple of 8 or does not follow the slot of the row before it; the
+  // group is that row and the rows behind it whose slots follow on, up to the end of the aligned eight. Every row
+  // lies in exactly one group, and a group is written by the workgroup that holds its first row (which reads up to
+  // seven rows of the workgroup behind it). Whole groups take the 16-byte way, the others value by value.
   const int dvecs = D >> 3;
-  for (int unit = threadIdx.x; unit < Hkv * dvecs; unit += 256) {
-    const int kvh = unit / dvecs, dv = unit - kvh * dvecs;
-    const bf16_t* src = qkv + t0 * row_stride + (int64_t)(heads + kvh) * D + 8 * dv;
-    if (run) {
-      u32x4r tok[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) tok[i] = *reinterpret_cast<const u32x4r*>(src + i * row_stride);
-      const int64_t pg = s0 / page, off = s0 - pg * page;
+  for (int i = 0; i < cnt; ++i) {
+    const int64_t t = t0 + i;
+    const int s0 = slots[t];
+    if (s0 < 0) continue;
+    const int lead = s0 & 7;
+    if (lead != 0 && t > 0 && slots[t - 1] == s0 - 1) continue;       // belongs to the group of a row before it
+    int n = 1;
+    while (n < 8 - lead && t + n < num_tokens && slots[t + n] == s0 + n) ++n;
+    const int64_t pg = s0 / page, off = s0 - pg * page;               // page % 8 == 0: a group lies within one page
+    for (int unit = threadIdx.x; unit < Hkv * dvecs; unit += 256) {
+      const int kvh = unit / dvecs, dv = unit - kvh * dvecs;
+      const bf16_t* src = qkv + t * row_stride + (int64_t)(heads + kvh) * D + 8 * dv;
       bf16_t* dst = v_cache + ((pg * Hkv + kvh) * (int64_t)D + 8 * dv) * page + off;
+      if (n == 8) {
+        u32x4r tok[8];
 #pragma unroll
-      for (int d = 0; d < 8; ++d) {   // channel d of the 8 tokens: word d/2 of each token, low or high half
-        u32x4r o;
+        for (int j = 0; j < 8; ++j) tok[j] = *reinterpret_cast<const u32x4r*>(src + j * row_stride);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t lo = tok[2 * j][d >> 1], hi = tok[2 * j + 1][d >> 1];
-          o[j] = (d & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+        for (int d = 0; d < 8; ++d) {   // channel d of the 8 tokens: word d/2 of each token, low or high half
+          u32x4r o;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = tok[2 * j][d >> 1], hi = tok[2 * j + 1][d >> 1];
+            o[j] = (d & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+          }
+          *reinterpret_cast<u32x4r*>(dst + (int64_t)d * page) = o;
         }
-        *reinterpret_cast<u32x4r*>(dst + (int64_t)d * page) = o;
-      }
-    } else {
-      for (int i = 0; i < cnt; ++i) {
-        const int slot = slots[t0 + i];
-        if (slot < 0) continue;
-        const int64_t pg = slot / page, off = slot - pg * page;
-        bf16_t* dst = v_cache + ((pg * Hkv + kvh) * (int64_t)D + 8 * dv) * page + off;
+      } else {
+        for (int j = 0; j < n; ++j) {
+          const bf16x8r v = *reinterpret_cast<const bf16x8r*>(src + j * row_stride);
 #pragma unroll
-        for (int d = 0; d < 8; ++d) dst[(int64_t)d * page] = src[i * row_stride + d];
+          for (int d = 0; d < 8; ++d) dst[(int64_t)d * page + j] = v[d];
+        }
       }
     }
   }

@@ -138,6 +138,17 @@ def test_qk_norm_rope_store_many_tokens(dtype, Hq, Hkv, D, page):
     hip().qk_norm_rope_store(a, None, None, 1e-5, table, pos, None, None, None, Hq, Hkv, D, page, False)
     twin.qk_norm_rope_store(b, None, None, 1e-5, table, pos, None, None, None, Hq, Hkv, D, page, False)
     close(a, b, tol)
+    # a mixed step: 5 decode rows in front of two prompts that start at page starts, so that no group of 8 batch rows
+    # is a group of 8 aligned slots, and the last aligned group ends with the last row
+    slots = torch.cat((torch.tensor([9 * page + 3, 2 * page, 11 * page + 15, 3 * page + 8, 12 * page + 1]),
+                       torch.arange(128) + 14 * page, torch.arange(64) + 32 * page)).to(torch.int32).to(DEV)
+    T2 = slots.numel()
+    a, b = qkv[:T2].clone(), qkv[:T2].clone()
+    ka, va = _caches(pages, Hkv, page, D, dtype); kb, vb = _caches(pages, Hkv, page, D, dtype)
+    hip().qk_norm_rope_store(a, qw, kw, 1e-5, table, pos[:T2], slots, ka, va, Hq, Hkv, D, page, True)
+    twin.qk_norm_rope_store(b, qw, kw, 1e-5, table, pos[:T2], slots, kb, vb, Hq, Hkv, D, page, True)
+    assert torch.equal(torch.isnan(va), torch.isnan(vb)) and torch.equal(torch.nan_to_num(va), torch.nan_to_num(vb))
+    close(torch.nan_to_num(ka), torch.nan_to_num(kb), tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
