@@ -931,8 +931,14 @@ def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     aligned = N % 2 == 0 and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
     if rows > GATED_EPILOGUE_MAX_M:
         # a few hundred rows over a small weight: the kernel that takes the product (mid_takes) gates in its epilogue too,
-        # in place of a kernel of its own behind it
-        return aligned and N % 8 == 0 and not skinny_takes(rows, N, K) and mid_takes(rows, N, K, False) == 1
+        # in place of a kernel of its own behind it; and from 17 rows on, where the skinny kernel would have the product
+        # itself: a layer's feed-forward at the 0.6B sizes, us, skinny product + gating + down / tiled product with the
+        # gating + down: 17 rows 14.1 / 13.6, 24 rows 14.8 / 13.8, 32 rows 15.9 / 14.1
+        if not (aligned and N % 8 == 0):
+            return False
+        if rows <= 32:
+            return mid_takes(33, N, K, False) == 1
+        return not skinny_takes(rows, N, K) and mid_takes(rows, N, K, False) == 1
     return 1 <= rows and aligned and takes
 
 

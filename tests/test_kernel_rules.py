@@ -59,8 +59,9 @@ def test_a_few_hundred_rows_over_small_weights_go_to_the_own_product():
 
 def test_gate_up_gates_in_its_epilogue_for_few_rows_and_for_a_few_hundred_over_small_weights():
     w = torch.empty(6144, 1024, dtype=torch.bfloat16)
-    assert all(ops.gated_linear_rows(m, w) for m in (1, 8, 16, 33, 64, 256))
-    assert not any(ops.gated_linear_rows(m, w) for m in (17, 32, 257, 2048))   # the down product gates, or a kernel of its own
+    assert all(ops.gated_linear_rows(m, w) for m in (1, 8, 16, 17, 32, 33, 64, 256))
+    assert not any(ops.gated_linear_rows(m, w) for m in (257, 2048))           # a kernel of its own
+    assert not ops.gated_linear_rows(24, torch.empty(12288, 2048, dtype=torch.bfloat16))     # 17-32 rows: only over small weights
     assert not ops.gated_linear_rows(128, torch.empty(12288, 2048, dtype=torch.bfloat16))    # the library's product
     assert not ops.gated_linear_rows(128, torch.empty(6144, 1024))                            # float32
 

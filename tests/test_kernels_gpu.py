@@ -555,7 +555,8 @@ def test_gating_in_the_gate_up_products_epilogue(M, I, K):
     torch.manual_seed(M + I)
     w = (torch.randn(2 * I, K, device=DEV) * 0.05).bfloat16()
     x = torch.randn(M, K, device=DEV).bfloat16()
-    assert ops.gated_linear_fuses(x, w) and not ops.gated_linear_fuses(torch.randn(17, K, device=DEV).bfloat16(), w)
+    assert ops.gated_linear_fuses(x, w)
+    assert ops.gated_linear_fuses(torch.randn(17, K, device=DEV).bfloat16(), w) == (ops.mid_takes(33, 2 * I, K, False) == 1)
     got = hip().gated_linear(x, w)
     assert got.shape == (M, I)
     close(got, twin.gated_linear(x, w, compute_dtype=torch.float64), 6e-3)
@@ -570,7 +571,7 @@ def test_gating_in_the_gate_up_products_epilogue(M, I, K):
         close(y, want, 6e-3)
 
 
-@pytest.mark.parametrize("M", [33, 65, 130, 256])
+@pytest.mark.parametrize("M", [17, 32, 33, 65, 130, 256])
 @pytest.mark.parametrize("I,K", [(3072, 1024), (100, 256), (36, 320), (1000, 2048)])
 def test_gating_in_the_epilogue_for_a_few_hundred_rows(M, I, K):
     """The same for 33 to 256 rows over a small weight: the tiled kernel takes 32 gate features and their 32 up features
@@ -578,10 +579,10 @@ def test_gating_in_the_epilogue_for_a_few_hundred_rows(M, I, K):
     torch.manual_seed(M + I)
     w = (torch.randn(2 * I, K, device=DEV) * 0.05).bfloat16()
     x = torch.randn(M, K, device=DEV).bfloat16()
-    if ops.skinny_takes(M, 2 * I, K):       # up to 64 rows over the smaller weights the skinny kernel has the product
+    if M > 32 and ops.skinny_takes(M, 2 * I, K):       # 33-64 rows over the smaller weights: the skinny kernel has the product
         assert not ops.gated_linear_fuses(x, w)
         return
-    assert ops.gated_linear_fuses(x, w) and ops.mid_takes(M, 2 * I, K, False) == 1
+    assert ops.gated_linear_fuses(x, w) and ops.mid_takes(max(M, 33), 2 * I, K, False) == 1
     got = hip().gated_linear(x, w)
     assert got.shape == (M, I)
     close(got, twin.gated_linear(x, w, compute_dtype=torch.float64), 6e-3)
