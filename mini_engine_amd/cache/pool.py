@@ -59,12 +59,30 @@ class CachePool:
                                         write=plan.call_writes[i]))
         self.num_state_slots = max(0, num_state_slots)
         self.states = []
+        self.state_initial = []        # per call: None (zeros) or a tensor of one row's shape
         for need in plan.state_needs:
             if need is None:
                 self.states.append(None)
+                self.state_initial.append(None)
+                continue
+            dt = _DTYPES[need.dtype]
+            st = torch.zeros((self.num_state_slots + 1,) + tuple(need.shape), dtype=dt, device=device)
+            first = None
+            if need.initial is not None:
+                first = torch.as_tensor(need.initial, dtype=dt).to(device).expand(tuple(need.shape)).contiguous()
+                st[:] = first
+            self.states.append(st)
+            self.state_initial.append(first)
+
+    def reset_state(self, slots: torch.Tensor) -> None:
+        """Rows `slots` (int64, on the device) of every state tensor back to what a request starts from."""
+        for st, first in zip(self.states, self.state_initial):
+            if st is None:
+                continue
+            if first is None:
+                st.index_fill_(0, slots, 0)
             else:
-                self.states.append(torch.zeros((self.num_state_slots + 1,) + tuple(need.shape),
-                                               dtype=_DTYPES[need.dtype], device=device))
+                st.index_copy_(0, slots, first.unsqueeze(0).expand((slots.numel(),) + tuple(first.shape)))
 
     def spare_page(self, group: int) -> int:
         return self.num_pages[group]

@@ -358,7 +358,7 @@ qk_norm_rope_store_tile_kernel(bf16_t* __restrict__ qkv, int64_t row_stride, con
 
 extern "C" int me_qk_norm_rope_store(void* qkv, int dtype, int64_t num_tokens, int64_t row_stride,
                                      const float* q_w, const float* k_w, float eps,
-                                     const float* table, int64_t table_positions,
+                                     const float* table, int64_t table_positions, int64_t position_bound,
                                      const int32_t* positions, const int32_t* slots, void* k_cache,
                                      void* v_cache, int Hq, int Hkv, int D, int page, int store,
                                      hipStream_t stream) {
@@ -369,6 +369,10 @@ extern "C" int me_qk_norm_rope_store(void* qkv, int dtype, int64_t num_tokens, i
   ME_CHECK(!store || (Hkv >= 1 && k_cache && v_cache), "qk_norm_rope_store: storing needs kv heads and caches");
   ME_CHECK(row_stride >= (int64_t)(Hq + (store ? 2 * Hkv : Hkv)) * D, "qk_norm_rope_store: row stride too small");
   ME_CHECK(!table || table_positions > 0, "qk_norm_rope_store: empty rotary table");
+  // position_bound: every position of the step is below it (what the host knows of the step; 0: not told)
+  ME_CHECK(!table || position_bound <= table_positions,
+           "qk_norm_rope_store: positions up to %lld are beyond the rotation table's %lld", (long long)position_bound - 1,
+           (long long)table_positions);
   const int heads = Hq + (store ? 2 * Hkv : Hkv);
   ME_CHECK(dtype == ME_BF16 || dtype == ME_F32, "qk_norm_rope_store: bad dtype code %d", dtype);
   // vectorised form: D/8 lanes per head must be a power of two, rows and caches 16-byte aligned

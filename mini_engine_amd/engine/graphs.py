@@ -43,6 +43,9 @@ def _pad4(n: int) -> int:
 class _Captured:
     def __init__(self, runner, bucket: int, ctx_cap: int, even: bool = False):
         self.bucket, self.ctx_cap, self.even = bucket, ctx_cap, even
+        # the cap is rounded for the block tables' width; what the kernels are told (and check against the
+        # position encoding's table) is never more than the engine's longest context
+        self.max_context = min(ctx_cap, runner.max_positions)
         ps = runner.manager.page_size
         self.G = len(runner.plan.group_needs)
         self.MB = -(-ctx_cap // ps)
@@ -91,7 +94,7 @@ class _Captured:
         return StepContext(
             num_tokens=B, num_seqs=B, num_decodes=B, positions=self.view("positions"),
             seq_of_token=self.view("seq_of_token"), context_lens=self.view("context_lens"),
-            cu_seqlens=self.view("cu"), prefill_cu=None, max_decode_context=self.ctx_cap,
+            cu_seqlens=self.view("cu"), prefill_cu=None, max_decode_context=self.max_context,
             decode_contexts_even=self.even,
             groups=[GroupStep(self.view(f"bt{g}").view(B, self.MB), self.view(f"slots{g}")) for g in range(self.G)],
             state_slots=self.view("state_slots"), first_chunk=self.view("first_chunk"),
@@ -179,10 +182,7 @@ class DecodeGraphs:
             cap.put("state_slots", state)
             fresh = state[:B][pos[:B] == 0]
             if fresh.size:              # a request whose first token this is starts from empty state (outside the graph)
-                idx = torch.tensor(fresh.tolist(), dtype=torch.long, device=r.device)
-                for st in r.pool.states:
-                    if st is not None:
-                        st.index_fill_(0, idx, 0)
+                r.pool.reset_state(torch.tensor(fresh.tolist(), dtype=torch.long, device=r.device))
         continues = self._continues(cap, reqs, pos, B)
         cap.last_starts = None                       # stays so if what follows raises
         if continues:
@@ -422,8 +422,9 @@ class MixedGraphs:
         need = decode_rows + exact.prefill_tokens + 1
         total = max(32, _pow2_at_least(need)) if need <= 256 else _round_up(need, 64 if need <= 1024 else 128)
         pad = total - decode_rows - exact.prefill_tokens
-        most_ctx = -(-r.max_positions // 8) * 8
-        cap = min(max(1024, _pow2_at_least(max(exact.decode_ctx, exact.prefill_ctx, pad))), most_ctx)
+        if pad > r.max_positions:
+            return None       # the padding request would stand at positions the engine does not have: run as it is
+        cap = min(max(1024, _pow2_at_least(max(exact.decode_ctx, exact.prefill_ctx, pad))), r.max_positions)
         ps = r.manager.page_size
         return StepLayout(
             decode_rows=decode_rows, prefill_reqs=exact.prefill_reqs + 1, prefill_tokens=total - decode_rows,

@@ -146,7 +146,9 @@ def pack_step(layout: StepLayout, out: np.ndarray, token_lists: list, starts: li
             slot[Dn:layout.decode_rows] = spare * ps
         if pad_req:
             b = B - 1
-            bt[b, :min(mb, -(-pad_tokens // ps))] = spare    # every page of the padding request is the spare one
+            if -(-pad_tokens // ps) > mb:
+                raise ValueError(f"the padding request's {pad_tokens} tokens need more than the layout's {mb} block-table columns")
+            bt[b, :-(-pad_tokens // ps)] = spare             # every page of the padding request is the spare one
             slot[cu[b]:cu[b + 1]] = spare * ps + pos[cu[b]:cu[b + 1]] % ps
         put(f"slots{g}", slot)
         put(f"bt{g}", bt.reshape(-1))

@@ -33,6 +33,7 @@ class Request:
     in_cache: int = field(init=False, default=0)        # tokens whose keys and values the cache holds
     from_prefix: int = field(init=False, default=0)     # of those, how many another request had left there
     portion: int = field(init=False, default=0)         # tokens it runs in the step being planned
+    times_evicted: int = field(init=False, default=0)   # how often it gave everything back and returned to the queue
 
     def __post_init__(self):
         self.tokens = [int(t) for t in self.tokens]

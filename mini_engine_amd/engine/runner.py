@@ -211,15 +211,13 @@ class ModelRunner:
         return self.model.logits(h, residual, row_view[:len(rows)])
 
     def zero_fresh_state(self, slots_of: list, starts: list) -> None:
-        """A request whose tokens start at position 0 starts from empty state."""
+        """A request whose tokens start at position 0 starts from its mixers' initial state (zeros unless
+        a `StateNeed` names another)."""
         if not self.pool.has_state:
             return
         fresh = [s for s, st in zip(slots_of, starts) if st == 0 and s >= 0]
         if fresh:
-            idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
-            for st in self.pool.states:
-                if st is not None:
-                    st.index_fill_(0, idx, 0)
+            self.pool.reset_state(torch.tensor(fresh, dtype=torch.long, device=self.device))
 
     # -- what the captured graphs share ----------------------------------------------------
     def graph_pool(self):

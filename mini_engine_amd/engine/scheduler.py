@@ -89,6 +89,8 @@ class Scheduler:
         self.waiting: deque = deque()
         self.running: list = []
         self.num_preemptions = 0
+        self.num_prefix_hits = 0               # admissions that found pages of their tokens already cached
+        self.num_prefix_hits_after_eviction = 0    # of those, requests fed again after an eviction
 
     # -- requests in ---------------------------------------------------------------------------
     def add(self, req: Request) -> None:
@@ -157,6 +159,7 @@ class Scheduler:
         self._give_back(req)
         req.phase = Phase.QUEUED
         req.portion = 0
+        req.times_evicted += 1
         self.order.enqueue(self.waiting, req, returning=True)
         self.num_preemptions += 1
 
@@ -177,6 +180,9 @@ class Scheduler:
                 return
             self.waiting.popleft()
             req.in_cache = req.from_prefix = reused
+            if reused:
+                self.num_prefix_hits += 1
+                self.num_prefix_hits_after_eviction += bool(req.times_evicted)
             req.phase = Phase.LIVE
             self.running.append(req)
             plan.take(req, n)

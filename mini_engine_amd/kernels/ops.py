@@ -58,7 +58,7 @@ _CORE_PROTOS = {
     "me_gather_rows": [P, P, P, L, L, L, P],
     "me_rms_norm": [P, I, I, L, P, P, P, P, I, L, I, F, P],
     "me_silu_and_mul": [P, P, I, L, I, P],
-    "me_qk_norm_rope_store": [P, I, L, L, P, P, F, P, L, P, P, P, P, I, I, I, I, I, P],
+    "me_qk_norm_rope_store": [P, I, L, L, P, P, F, P, L, L, P, P, P, P, I, I, I, I, I, P],
     "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
@@ -245,9 +245,11 @@ class HipBackend:
 
     # -- q/k norm + rotary + cache write -------------------------------------------------
     def qk_norm_rope_store(self, qkv, q_weight, k_weight, eps, table, positions, slots, k_cache, v_cache,
-                           Hq: int, Hkv: int, D: int, page: int, store: bool = True) -> None:
+                           Hq: int, Hkv: int, D: int, page: int, store: bool = True, position_bound: int = 0) -> None:
         """In place on packed rows: per-head RMSNorm of q and k (weights float32 [D] or None), then
-        rotary by `table` [P, D/2, 2] float32 (or None), q written back.
+        rotary by `table` [P, D/2, 2] float32 (or None), q written back. `position_bound`: every position
+        of the step is below it (the longest context the step's layout allows; 0: not told); a bound beyond
+        the table's rows is refused.
 
         store=True: rows are [T, (Hq+2Hkv)*D]; k and v are scattered to the pages at `slots`
         (slots < 0 skipped). store=False: rows are [T, (Hq+Hkv)*D] (Hkv may be 0); k is written
@@ -272,7 +274,7 @@ class HipBackend:
             _check(k_cache.shape[1:] == (Hkv, page, D) and v_cache.shape[1:] == (Hkv, D, page),
                    "qk_norm_rope_store: caches must be K [pages, Hkv, page, D] and V [pages, Hkv, D, page]")
         core().call("me_qk_norm_rope_store", qkv.data_ptr(), _code(qkv.dtype), T, qkv.stride(0), _ptr(q_weight),
-                    _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0],
+                    _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0], int(position_bound),
                     positions.data_ptr(), _ptr(slots) if store else None, _ptr(k_cache) if store else None,
                     _ptr(v_cache) if store else None, Hq, Hkv, D, page, int(store), _stream())
 

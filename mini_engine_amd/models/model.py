@@ -10,6 +10,7 @@ from dataclasses import dataclass
 
 import torch
 
+from ..kernels import ops
 from ..parts.base import CacheNeed, LayerCall, Part, StateNeed
 from ..parts.block import norm_of
 
@@ -53,7 +54,6 @@ class DecoderModel(Part):
         self.optional_sources = set(optional_sources or ())
         self.device = None
         self.dtype = None
-        self._head_takes_out = None
         for i, call in enumerate(self.order):
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"run order entry {i} names layer {call.layer}, the model has {len(self.layers)}")
@@ -107,16 +107,7 @@ class DecoderModel(Part):
     def logits(self, h, residual, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """Final norm of (h + residual), then the rows that want logits, then the head: float32
         [len(rows), vocab] (reference models/qwen3.py:91,116-117; layers/embed_head.py:19-23).
-        `out`: where to put them, for a head whose forward takes `out`; any other head's result is copied there."""
-        import inspect
-        from ..kernels import ops
+        `out`: where the head puts them (`parts.Head.forward(x, out)`)."""
         x, _ = norm_of(self.final_norm, h, residual)
         x = ops.gather_rows(x, rows)
-        if out is None:
-            return self.head.forward(x)
-        if self._head_takes_out is None:
-            self._head_takes_out = "out" in inspect.signature(self.head.forward).parameters
-        if self._head_takes_out:
-            return self.head.forward(x, out=out)
-        out.copy_(self.head.forward(x))
-        return out
+        return self.head.forward(x, out=out)

@@ -73,13 +73,14 @@ class Attention(Mixer):
             return self.o.forward(o, allow_partials=True)
         if self.position is None or table is not None:
             # norm + rotary + cache write in one pass
+            bound = max(step.max_decode_context, step.max_prefill_context)
             if store:
                 ops.qk_norm_rope_store(qkv, qw, kw, eps, table, step.positions, grp.slot_mapping,
-                                       cache.k, cache.v, Hq, Hkv, D, cache.page_size, store=True)
+                                       cache.k, cache.v, Hq, Hkv, D, cache.page_size, store=True, position_bound=bound)
             else:
                 rows = qkv if not self.own_kv else qkv[:, : self.q_size]
                 ops.qk_norm_rope_store(rows, qw, kw, eps, table, step.positions, None, None, None,
-                                       Hq, 0, D, cache.page_size, store=False)
+                                       Hq, 0, D, cache.page_size, store=False, position_bound=bound)
         else:
             # another position encoding: norm in place, the encoding's own apply, then the cache write
             nk = Hkv if self.own_kv else 0

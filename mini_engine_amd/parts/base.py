@@ -19,7 +19,10 @@ class ParamSpec:
     """One parameter tensor of a part.
 
     ``init`` names the distribution used by the random-weights mode:
-    ``"matrix"`` ~ N(0, 0.02) (linears, embeddings), ``"norm"`` ~ 1 + U(-0.1, 0.1).
+    ``"matrix"`` ~ N(0, 0.02) (linears, embeddings), ``"norm"`` ~ 1 + U(-0.1, 0.1); or it is a
+    function ``(shape, generator, device) -> float32 tensor`` for a parameter that wants another start
+    (a decay rate in (0, 1), a table of integers, ...): it draws from `generator` only, so that the
+    values depend on the seed alone.
     ``dtype`` is ``"compute"`` (the engine's dtype: bfloat16 or float32),
     ``"float32"`` (always 32-bit: norm weights, exact for both stored forms),
     ``"int32"`` (integer tables) or ``"stored"`` (what the checkpoint holds: bfloat16
@@ -27,7 +30,7 @@ class ParamSpec:
     """
 
     shape: tuple
-    init: str = "matrix"
+    init: object = "matrix"       # "matrix", "norm" or a function (shape, generator, device) -> tensor
     dtype: str = "compute"
 
 
@@ -80,10 +83,14 @@ class CacheNeed:
 @dataclass(frozen=True)
 class StateNeed:
     """Fixed-size per-request state of a mixer: one tensor ``[num_slots + 1, *shape]``; the last row is
-    a spare that belongs to no request (padding rows of a step with a fixed layout name it)."""
+    a spare that belongs to no request (padding rows of a step with a fixed layout name it).
+    ``initial``: what the state of a request holds before its first token: None for zeros, a number, or
+    nested tuples of numbers of `shape` (a running maximum starts at -inf, a product at 1, ...). The step
+    function writes it into a request's row when the request's tokens start at position 0."""
 
     shape: tuple
     dtype: str = "float32"
+    initial: object = None
 
 
 class Part:
@@ -231,6 +238,23 @@ class Mixer(Part):
 class FeedForward(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
+
+
+class Head(Part):
+    """Hidden rows to float32 logits. `project` is what a head implements; `forward` is what the model calls."""
+
+    def project(self, x: torch.Tensor) -> torch.Tensor:
+        """x [rows, hidden] -> float32 [rows, vocabulary]."""
+        raise NotImplementedError
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """`out`: a float32 [rows, vocabulary] tensor the logits must end up in (a step with a fixed layout
+        keeps one). A head whose product can write there overrides this; by default the result is copied."""
+        y = self.project(x)
+        if out is None:
+            return y
+        out.copy_(y)
+        return out
 
 
 @dataclass

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import ParamSpec, Part
+from .base import Head, ParamSpec, Part
 
 
 class TokenEmbedding(Part):
@@ -18,7 +18,7 @@ class TokenEmbedding(Part):
         return ops.gather_rows(self.weight, token_ids)
 
 
-class LMHead(Part):
+class LMHead(Head):
     """logits = x . W^T in float32. When tied, W is the embedding matrix itself: the same
     tensor, not a copy (reference models/qwen3.py:107-109)."""
 

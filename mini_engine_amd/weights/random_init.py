@@ -1,7 +1,7 @@
 """Seeded random weights: fill a model directly, or write a model folder.
 
 Distributions: matrices (linears, embeddings) ~ N(0, 0.02); norm weights (the per-head
-q/k norms too) ~ 1 + U(-0.1, 0.1). Tensors are generated in float32 on the CPU, one
+q/k norms too) ~ 1 + U(-0.1, 0.1); a parameter may bring a function of its own (`ParamSpec.init`). Tensors are generated in float32 on the CPU, one
 generator seeded once, in sorted order of their checkpoint names, so the values depend
 only on (config, seed).
 """
@@ -27,7 +27,12 @@ def _checkpoint_tensor_specs(model) -> list:
     return sorted((n, s, k, d) for n, (s, k, d) in out.items())
 
 
-def _draw(shape, kind: str, gen, device) -> torch.Tensor:
+def _draw(shape, kind, gen, device) -> torch.Tensor:
+    if callable(kind):
+        t = kind(tuple(shape), gen, device)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"an init function returned shape {tuple(t.shape)} for a parameter of shape {tuple(shape)}")
+        return t.to(torch.float32)
     if kind == "matrix":
         return torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * 0.02
     if kind == "norm":

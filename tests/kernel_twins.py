@@ -54,8 +54,12 @@ def write_pages(k, v, slots, k_cache, v_cache, page):
 
 
 def qk_norm_rope_store(qkv, q_weight, k_weight, eps, table, positions, slots, k_cache, v_cache,
-                       Hq, Hkv, D, page, store=True):
+                       Hq, Hkv, D, page, store=True, position_bound=0):
     T = qkv.shape[0]
+    if table is not None:
+        # what the kernel's launcher refuses, and what it could not see: a position beyond the table
+        assert position_bound <= table.shape[0], f"position bound {position_bound} beyond the table's {table.shape[0]} rows"
+        assert T == 0 or int(positions[:T].max()) < table.shape[0], "a position beyond the rotation table"
     q = _norm_rope(qkv[:, :Hq * D].float().clone().view(T, Hq, D), q_weight, eps, table, positions)
     if Hkv:
         k = _norm_rope(qkv[:, Hq * D:(Hq + Hkv) * D].float().clone().view(T, Hkv, D), k_weight, eps, table, positions)
@@ -108,6 +112,7 @@ def decode_step_attention(qkv, q_weight, k_weight, eps, table, k_cache, v_cache,
     position context_lens[r] - 1, its slot is what the block table names for that position (a row with
     context 0 is padding: nothing is written for it and it sees nothing)."""
     B = qkv.shape[0]
+    assert table is None or max_context <= table.shape[0], f"a context of {max_context} beyond the table's {table.shape[0]} rows"
     ctx = context_lens[:B].long()
     positions = (ctx - 1).clamp(min=0).to(torch.int32)
     pages = block_tables[torch.arange(B, device=qkv.device), (positions // page).long()].long()
@@ -162,6 +167,27 @@ def _fmix32(h):
     h = (h * 0xC2B2AE35) & m
     h ^= h >> 16
     return h
+
+
+def row_key(seed, stream, index):
+    """The two 32-bit words that key the noise of output number `index` of the request with noise stream
+    `stream` under `seed`: three rounds of SplitMix64's output function (add the golden-ratio constant, two
+    xor-shift-multiplies, a last xor-shift), each taking the next of (seed, stream, index) xored into the state;
+    (low word, high word) of the result. Written with numpy's wrapping 64-bit integers."""
+    import numpy as np
+    u = np.uint64
+
+    def mix(x):
+        with np.errstate(over="ignore"):
+            x = x + u(0x9E3779B97F4A7C15)
+            x = (x ^ (x >> u(30))) * u(0xBF58476D1CE4E5B9)
+            x = (x ^ (x >> u(27))) * u(0x94D049BB133111EB)
+        return x ^ (x >> u(31))
+
+    x = mix(u(seed % (1 << 64)))
+    x = mix(x ^ u(stream % (1 << 64)))
+    x = mix(x ^ u(index % (1 << 64)))
+    return int(x & u(0xFFFFFFFF)), int(x >> u(32))
 
 
 def exp_noise(keys, V, device):

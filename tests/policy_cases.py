@@ -104,4 +104,66 @@ def windowed_model(make, folders, exact):
         assert all(llm.manager.num_free_pages(g) == options["num_kvcache_blocks"] for g in range(2))
 
 
-ALL = [priority_policy, priority_order, long_prefill_threshold, prefill_first, many_live_requests, windowed_model]
+def eviction_with_prefix_cache(make, folders, exact):
+    """Prefix caching on (the engine's default), six requests that share their first three pages, a pool so small
+    that requests are evicted: a request that is fed again finds pages of its own tokens (the shared prefix, or what
+    it had published itself) and must still give the plain model's tokens. Chunked under two budgets and whole
+    prompts first, steps run ahead or not."""
+    folder = folders("A")
+    shared = helpers.random_ids(48, 256, 340)
+    prompts = [shared + helpers.random_ids(n, 256, 341 + n) for n in (5, 20, 9, 30, 14, 3)]
+    for options in (dict(max_num_batched_tokens=16), dict(max_num_batched_tokens=64),
+                    dict(max_num_batched_tokens=128, enable_chunked_prefill=False)):
+        for run_ahead in (True, False):
+            llm = make(folder, kvcache_block_size=16, num_kvcache_blocks=10, max_num_seqs=4, max_model_len=128,
+                       enable_prefix_caching=True, run_ahead=run_ahead, **options)
+            assert llm.manager.prefix_caching
+            outs = llm.generate(prompts, _greedy(24), use_tqdm=False)
+            what = f"prefix cache + eviction {options} run_ahead={run_ahead}"
+            assert llm.scheduler.num_preemptions > 0, f"{what}: nobody was evicted"
+            assert llm.scheduler.num_prefix_hits_after_eviction > 0, f"{what}: no request that was fed again found cached pages"
+            helpers.assert_greedy_like_plain(folder, prompts, [o["token_ids"] for o in outs], exact, what)
+            llm.manager.check_invariants()
+            assert llm.manager.num_free_pages() == 10
+
+
+def sampled_tokens_follow_their_keys(make, folders, exact):
+    """Temperature 0.8: output number i of request r is argmax(plain logits / T - log E) with the noise E keyed by
+    (seed, r's noise stream, i), the key derived here by the test's own code. A key that left out the seed, the
+    request or the output index would give other tokens. Prompts are chunked under a budget of 16 and one request
+    brings a seed of its own."""
+    import torch
+    import kernel_twins
+    import plain_qwen3
+    from mini_engine_amd import SamplingParams
+    folder = folders("B")
+    cfg, w = plain_qwen3.read_model_folder(folder, torch.float64)
+    prompts = [helpers.random_ids(n, 384, 960 + n) for n in (1, 9, 24, 40)]
+    T = 0.8
+    sps = [SamplingParams(temperature=T, max_tokens=10, ignore_eos=True, seed=(77 if i == 2 else None)) for i in range(4)]
+    llm = make(folder, kvcache_block_size=8, num_kvcache_blocks=64, max_num_seqs=4, max_num_batched_tokens=16,
+               max_model_len=128, seed=3)
+    outs = [o["token_ids"] for o in llm.generate(prompts, sps, use_tqdm=False)]
+    seen_keys = set()
+    not_greedy = 0
+    for r, (prompt, out) in enumerate(zip(prompts, outs)):
+        ids = list(prompt)
+        for i, tok in enumerate(out):
+            z = plain_qwen3.logits(cfg, w, ids)[-1]
+            key = kernel_twins.row_key(77 if r == 2 else 3, r, i)
+            seen_keys.add(key)
+            keys = torch.tensor([key], dtype=torch.int64).to(torch.int32)      # the words' bits, as the kernel takes them
+            score = kernel_twins.sample_scores(z.float()[None, :], torch.tensor([T]), keys)[0].double()
+            best = int(score.argmax())
+            not_greedy += tok != int(z.argmax())
+            # the engine's logits differ from the plain model's within its tolerance; a token other than the best
+            # passes only where the two scores lie closer than that
+            tol = (helpers.TOL_F32 if exact else helpers.TOL_BF16) * float(z.abs().max()) / T
+            assert tok == best or float(score[best] - score[tok]) <= tol, \
+                f"request {r}, output {i}: sampled {tok}, the keyed noise on the plain logits gives {best}"
+            ids.append(tok)
+    assert len(seen_keys) == 40
+    assert not_greedy >= 10, "the noise changed next to nothing: the case tests nothing"
+
+
+ALL = [eviction_with_prefix_cache, sampled_tokens_follow_their_keys, priority_policy, priority_order, long_prefill_threshold, prefill_first, many_live_requests, windowed_model]

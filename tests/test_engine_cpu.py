@@ -266,6 +266,53 @@ def test_padded_decode_layout_without_capture(folders, plain_backend, name):
         assert helpers.rel_err(got, helpers.plain_logits(folder, ids[r][:got.shape[0]])) <= helpers.TOL_F32, r
 
 
+@pytest.mark.parametrize("limit", [100, 43])
+def test_fixed_layouts_with_a_longest_context_that_is_no_multiple_of_8(folders, plain_backend, limit):
+    """The fixed layouts round their block tables up; what they tell the kernels about the longest context must
+    not go beyond the engine's limit, which is where the position encoding's table ends (the twins assert it)."""
+    V, page, folder = helpers.CONFIGS["A"]["vocab_size"], helpers.PAGE["A"], folders("A")
+    model = load_model(folder, "cpu", torch.float32, limit)
+    assert model.layers[0].mixer.position.rotary_table().shape[0] == limit
+    manager = CacheManager(20, page, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, torch.float32, "cpu", limit, poison_cache=True, use_graphs=True,
+                         mixed_graphs_after=0, mixed_graphs_max_tokens=4096)
+    ids = helpers.random_ids(limit, V, 77)
+    d = helpers.Driver(runner, manager)
+    d.step({"r": ids[:limit - 6]})
+    for t in range(limit - 6, limit):
+        d.step({"r": ids[t:t + 1]})
+    assert runner.graphs.replays == 6
+    assert all(c.context().max_decode_context <= limit for c in runner.graphs.captured.values())
+    assert helpers.rel_err(d.result("r"), helpers.plain_logits(folder, ids)) <= helpers.TOL_F32
+
+
+def test_a_padding_request_longer_than_the_longest_context_is_not_made(folders, plain_backend):
+    """Three prompts of 43 tokens under a limit of 64: rounded up to 256 tokens the padding request would hold 126
+    tokens, at positions the engine does not have. Such a step runs exactly sized instead."""
+    from mini_engine_amd.engine.packing import exact_layout, pack_step
+    import numpy as np
+    V, page, folder = helpers.CONFIGS["A"]["vocab_size"], helpers.PAGE["A"], folders("A")
+    model = load_model(folder, "cpu", torch.float32, 64)
+    manager = CacheManager(20, page, ModelRunner.windows_of(model), enable_prefix_caching=False)
+    runner = ModelRunner(model, manager, torch.float32, "cpu", 64, poison_cache=True, use_graphs=True,
+                         mixed_graphs_after=0, mixed_graphs_max_tokens=4096)
+    ids = {r: helpers.random_ids(43, V, 80 + i) for i, r in enumerate("abc")}
+    d = helpers.Driver(runner, manager)
+    d.step(ids)
+    assert runner.mixed_graphs.replays == 0
+    d.step({"a": [5, 6]})                      # a small step still takes a padded layout
+    assert runner.mixed_graphs.replays == 1
+    for r in "abc":
+        assert helpers.rel_err(d.result(r)[:43], helpers.plain_logits(folder, ids[r])) <= helpers.TOL_F32, r
+    # and the packing itself refuses a padding request whose pages do not fit the layout's tables
+    exact = exact_layout([43], [0], [[[0, 1, 2]]], 0, lambda *a: False)
+    import dataclasses
+    wide = dataclasses.replace(exact, prefill_reqs=2, prefill_tokens=43 + 100)
+    with pytest.raises(ValueError, match="padding request"):
+        pack_step(wide, np.zeros(wide.segments()[1], dtype=np.int32), [list(range(43))], [0], [[[0, 1, 2]]], [-1], [],
+                  page, [9], 0, V)
+
+
 def test_decode_rows_follow_a_request_that_was_fed_again(folders, plain_backend):
     """Decode steps that continue the one before carry their tables and slots on; a request that gave
     its pages back and was fed again sits at the same positions on other pages, and must be looked up."""

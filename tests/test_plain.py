@@ -4,7 +4,10 @@ that reduce to library routines, and invariants, each chosen so that a plausible
 
 The reference publishes no test vectors (its checks are git-ignored, reference .gitignore:10-12),
 so none can be used here: parity with its numbers is unpinned, parity with its formulas is
-what these tests hold.
+what these tests hold. The model code of installed packages is no source for this repository
+(neither read, imported nor run), so no test compares with one; what stands in for it: the
+attention scale is the library routine's own default, the rotation's frequencies are literals
+worked out by hand, the rotation is a complex product, the window is a band matrix written out.
 """
 import math
 
@@ -41,11 +44,32 @@ def test_add_rms_norm_returns_sum_as_residual():
     assert torch.allclose(y, P.rms_norm(x + r, w, 1e-6))
 
 
+def test_rope_frequencies_by_hand():
+    """The frequencies worked out by hand, not by the formula's own expression. Head size 8, theta 10^4: pair i
+    turns by theta^(-2i/8) per position = 1, 1/10, 1/100, 1/1000 (an exponent of i/D, (2i+1)/D or 2i/(D-2) gives
+    other numbers); head size 4, theta 10^6: 1 and 1/1000. The cos/sin literals are those of 3, 0.3, 0.03, 0.003."""
+    cos, sin = P.rope_tables(8, 4, 10000.0)
+    want_cos = [-0.9899924966004454, 0.955336489125606, 0.9995500337489875, 0.9999955000033750]
+    want_sin = [0.1411200080598672, 0.29552020666133955, 0.02999550020249566, 0.0029999955000020250]
+    assert torch.allclose(cos[3, :4], torch.tensor(want_cos, dtype=D64), atol=1e-14)
+    assert torch.allclose(sin[3, :4], torch.tensor(want_sin, dtype=D64), atol=1e-14)
+    assert torch.equal(cos[:, :4], cos[:, 4:]) and torch.equal(sin[:, :4], sin[:, 4:])    # both halves carry the same angle
+    cos, sin = P.rope_tables(4, 2001, 1e6)
+    # one position turns pair 1 by a thousandth of a radian: after 2,000 positions it has turned by 2 radians
+    assert torch.allclose(cos[2000, 1], torch.tensor(-0.4161468365471424, dtype=D64), atol=1e-12)
+    assert torch.allclose(sin[1, 0], torch.tensor(0.8414709848078965, dtype=D64), atol=1e-14)       # pair 0: one radian
+
+
 def test_rope_tables_and_pairing():
     Dh, n, theta = 16, 50, 10000.0
     cos, sin = P.rope_tables(Dh, n, theta)
-    inv = theta ** (-torch.arange(0, Dh, 2, dtype=D64) / Dh)
-    ang = torch.outer(torch.arange(n, dtype=D64), inv)
+    # the angle of pair i grows linearly with the position, pair 0 by one radian a position, and the pairs'
+    # rates form a geometric sequence that ends one step (a factor theta^(2/D)) above 1/theta
+    ang = torch.atan2(sin[1, :Dh // 2], cos[1, :Dh // 2])          # position 1: all angles are below pi
+    assert torch.allclose(ang[0], torch.tensor(1.0, dtype=D64))
+    assert torch.allclose(ang[1:] / ang[:-1], torch.full((Dh // 2 - 1,), theta ** (-2 / Dh), dtype=D64))
+    assert torch.allclose(ang[-1] * theta ** (-2 / Dh), torch.tensor(1 / theta, dtype=D64))
+    ang = torch.outer(torch.arange(n, dtype=D64), ang)
     assert torch.allclose(cos[:, :Dh // 2], ang.cos()) and torch.allclose(cos[:, Dh // 2:], ang.cos())
     assert torch.allclose(sin[:, Dh // 2:], ang.sin())
     x = torch.randn(n, 3, Dh, dtype=D64)
@@ -76,10 +100,11 @@ def test_rope_scores_depend_only_on_distance():
 def test_attention_is_library_causal_attention(Hq, Hkv):
     T, Dh = 19, 16
     q, k, v = torch.randn(T, Hq, Dh, dtype=D64), torch.randn(T, Hkv, Dh, dtype=D64), torch.randn(T, Hkv, Dh, dtype=D64)
-    got = P.causal_attention(q, k, v, Dh ** -0.5)
+    got = P.causal_attention(q, k, v, 0.37)
     ref = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
-                                         is_causal=True, scale=Dh ** -0.5, enable_gqa=True)[0].transpose(0, 1)
+                                         is_causal=True, scale=0.37, enable_gqa=True)[0].transpose(0, 1)
     assert torch.allclose(got, ref, atol=1e-12)
+    got = P.causal_attention(q, k, v, Dh ** -0.5)
     # grouped heads == every kv head repeated for its consecutive query heads
     rep = Hq // Hkv
     full = P.causal_attention(q, k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1), Dh ** -0.5)
@@ -100,6 +125,14 @@ def test_attention_special_cases():
     assert torch.allclose(outw[4, 0], v[3:5, 0].mean(0))
     # a window as long as the sequence changes nothing
     assert torch.allclose(P.causal_attention(q, k, v, 0.3, window=5), out)
+    # the library routine with the band written out: query i sees keys i - w + 1 .. i
+    T, w = 23, 6
+    q, k, v = torch.randn(T, 2, Dh, dtype=D64), torch.randn(T, 2, Dh, dtype=D64), torch.randn(T, 2, Dh, dtype=D64)
+    band = torch.ones(T, T, dtype=torch.bool).tril().triu(-(w - 1))
+    assert band[10].nonzero().flatten().tolist() == [5, 6, 7, 8, 9, 10]
+    ref = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                         attn_mask=band, scale=0.3)[0].transpose(0, 1)
+    assert torch.allclose(P.causal_attention(q, k, v, 0.3, window=w), ref, atol=1e-12)
 
 
 def test_far_key_dominates():
@@ -140,8 +173,11 @@ def test_model_reduces_to_hand_composition(tmp_path):
     k = F.rms_norm(k, (Dh,), w[p + "self_attn.k_norm.weight"], eps)
     cos, sin = P.rope_tables(Dh, 11, cfg["rope_theta"])
     q, k = P.apply_rope(q, cos, sin, torch.arange(11)), P.apply_rope(k, cos, sin, torch.arange(11))
+    # no scale is handed to the library: its default, 1 / sqrt(head size), is what the model's attention must use
+    # (reference models/qwen3.py:25 hands head_dim ** -0.5 to its kernels; a scale of 1 / head size, or 1 /
+    # sqrt(hidden / heads) where that differs from the head size as it does here (80 / 6), fails this)
     o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
-                                       is_causal=True, scale=Dh ** -0.5, enable_gqa=True)[0].transpose(0, 1)
+                                       is_causal=True, enable_gqa=True)[0].transpose(0, 1)
     res = h + F.linear(o.reshape(11, -1), w[p + "self_attn.o_proj.weight"])
     x = F.rms_norm(res, (res.shape[-1],), w[p + "post_attention_layernorm.weight"], eps)
     m = F.linear(F.silu(F.linear(x, w[p + "mlp.gate_proj.weight"])) * F.linear(x, w[p + "mlp.up_proj.weight"]),

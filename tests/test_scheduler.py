@@ -260,3 +260,20 @@ def test_random_traffic_keeps_every_invariant():
             assert r.done and 1 <= r.num_generated <= r.params.max_tokens
             if r.num_generated < r.params.max_tokens:
                 assert r.tokens[-1] == 5 and not r.params.ignore_eos
+
+
+def test_noise_keys_depend_on_seed_request_and_output_index():
+    """The sampler's key against the test's own derivation (tests/kernel_twins.py), against SplitMix64's
+    published first output for state 0, and: no two of (seed, request, output index) in a small cube share a key."""
+    import kernel_twins
+    from mini_engine_amd.sampling.sampler import _splitmix64, row_key
+    assert _splitmix64(0) == 0xE220A8397B1DCDAF
+    seen = set()
+    for seed in (0, 3, 2**31, 2**63 + 5):
+        for request in (0, 1, 7, 2**40):
+            for index in range(6):
+                key = row_key(seed, request, index)
+                assert key == kernel_twins.row_key(seed, request, index)
+                assert all(0 <= word < 2**32 for word in key)
+                seen.add(key)
+    assert len(seen) == 4 * 4 * 6

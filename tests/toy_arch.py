@@ -26,17 +26,28 @@ from mini_engine_amd.registry import build_model, register_architecture
 from mini_engine_amd.weights.random_init import fill_random, write_random_model
 
 
+PRIOR_COUNT = 2.0      # the running mean starts as if it had seen this many zero vectors
+
+
+def half_to_one(shape, generator, device):
+    """An init function of a part's own: uniform in [0.5, 1)."""
+    return 0.5 + 0.5 * torch.rand(shape, generator=generator, dtype=torch.float32, device=device)
+
+
 @register_part("mixer", "toy_running_mean")
 class RunningMean(Mixer):
-    """y_t = W . mean(x_0..x_t). State per request: [hidden + 1] = (sum of inputs, count)."""
+    """y_t = W . (gain * (x_0 + .. + x_t) / (t + 1 + PRIOR_COUNT)). State per request: [hidden + 1] = (sum of
+    inputs, count); the count of a request that has seen nothing is PRIOR_COUNT, not zero (`StateNeed.initial`),
+    and `gain` is drawn by a function of this file (`ParamSpec.init`)."""
 
     def __init__(self, hidden_size):
         super().__init__()
         self.hidden_size = hidden_size
         self.add_param("weight", ParamSpec((hidden_size, hidden_size), init="matrix", dtype="compute"))
+        self.add_param("gain", ParamSpec((hidden_size,), init=half_to_one, dtype="float32"))
 
     def state_need(self):
-        return StateNeed((self.hidden_size + 1,), "float32")
+        return StateNeed((self.hidden_size + 1,), "float32", initial=(0.0,) * self.hidden_size + (PRIOR_COUNT,))
 
     def forward(self, x, step, cache, state):
         T = x.shape[0]
@@ -50,7 +61,7 @@ class RunningMean(Mixer):
         counts = held[seq, -1] + (torch.arange(T, device=x.device) - first + 1).float()
         last = cu[1:] - 1
         state.index_copy_(0, slots, torch.cat([sums[last], counts[last, None]], 1))
-        return (sums / counts[:, None]).to(x.dtype) @ self.weight.T
+        return (self.gain * sums / counts[:, None]).to(x.dtype) @ self.weight.T
 
 
 @register_part("mixer", "toy_latent_mean")
@@ -196,7 +207,8 @@ def _toy_plain(model, ids, margins=None):
         res = res + h
         a = norm(layer.norm1, res)
         if isinstance(layer.mixer, RunningMean):
-            a = (a.cumsum(0) / torch.arange(1, T + 1, dtype=torch.float64)[:, None]) @ W(layer.mixer.weight).T
+            count = torch.arange(1, T + 1, dtype=torch.float64) + PRIOR_COUNT
+            a = (W(layer.mixer.gain) * a.cumsum(0) / count[:, None]) @ W(layer.mixer.weight).T
         elif isinstance(layer.mixer, LatentMean):
             z = a @ W(layer.mixer.w_in).T
             a = (z.cumsum(0) / torch.arange(1, T + 1, dtype=torch.float64)[:, None]) @ W(layer.mixer.w_out).T
@@ -243,11 +255,11 @@ def run_toy(device, dtype, tol):
     manager = CacheManager(8, 8, ModelRunner.windows_of(model), num_state_slots=3)
     runner = ModelRunner(model, manager, dtype, device, 128, poison_cache=True)
     assert runner.pool.states[0] is not runner.pool.states[2]      # each call of layer 0 has state of its own
-    a, b = helpers.random_ids(30, 50, 50), helpers.random_ids(12, 50, 34)     # seeds with clear routing, see below
+    a, b = helpers.random_ids(30, 50, 54), helpers.random_ids(12, 50, 34)     # seeds with clear routing, see below
     d = helpers.Driver(runner, manager)
     d.step({"a": a[:11]}); d.step({"a": a[11:12], "b": b[:5]}); d.step({"b": b[5:6], "a": a[12:29]})
     d.step({"a": a[29:], "b": b[6:]}, end=["a"])
-    c = helpers.random_ids(9, 50, 44)                                # takes over a's slot: must start from zero state
+    c = helpers.random_ids(9, 50, 46)                                # takes over a's slot: must start from zero state
     d.step({"c": c}, end=["b", "c"])
     margins = []
     for ids, rid in ((a, "a"), (b, "b"), (c, "c")):
