@@ -57,70 +57,121 @@ def poisson_arrivals(num: int, rate: float, long_frac: float, vocab: int, scale:
     return out
 
 
-def apply_setting(engine, name: str) -> None:
-    """`pf`: whole prompts first, 16,384 tokens a step. `c<N>`: chunked prefill under N tokens a step."""
-    sched = engine.scheduler
-    if name == "pf":
-        sched.chunked, sched.token_budget = False, ENGINE_BUDGET
-    elif name.startswith("c") and name[1:].isdigit() and 0 < int(name[1:]) <= ENGINE_BUDGET:
-        sched.chunked, sched.token_budget = True, int(name[1:])
-    else:
+@dataclass(frozen=True)
+class Setting:
+    """How prompts enter the steps: whole prompts first (`pf`), or in portions beside the decoding requests
+    under a budget of tokens a step (`c<tokens>`); reference bench_latency.py:41-51 names them so."""
+
+    name: str
+    chunked: bool
+    budget: int
+
+    @classmethod
+    def parse(cls, name: str) -> "Setting":
+        if name == "pf":
+            return cls(name, False, ENGINE_BUDGET)
+        if name[:1] == "c" and name[1:].isdigit() and 0 < int(name[1:]) <= ENGINE_BUDGET:
+            return cls(name, True, int(name[1:]))
         raise ValueError(f"setting {name!r}: expected 'pf' or 'c<tokens>' with at most {ENGINE_BUDGET} tokens")
-    if name == "pf" and ENGINE_BUDGET < sched.max_model_len:
-        raise ValueError(f"setting 'pf' needs a whole prompt in one step: max_model_len {sched.max_model_len} > {ENGINE_BUDGET}")
-    if sched.token_budget < sched.max_live:
-        raise ValueError(f"setting {name!r}: the budget must cover one token for each of {sched.max_live} requests")
-    engine.manager.forget_prefixes()
+
+    def check(self, scheduler) -> None:
+        if not self.chunked and self.budget < scheduler.max_model_len:
+            raise ValueError(f"setting 'pf' needs a whole prompt in one step: max_model_len {scheduler.max_model_len} > {self.budget}")
+        if self.budget < scheduler.max_live:
+            raise ValueError(f"setting {self.name!r}: the budget must cover one token for each of {scheduler.max_live} requests")
+
+    def switch(self, engine) -> None:
+        """Put the engine's scheduler into this setting; what earlier settings left published in the cache is forgotten."""
+        self.check(engine.scheduler)
+        engine.scheduler.chunked = self.chunked
+        engine.scheduler.token_budget = self.budget
+        engine.manager.forget_prefixes()
 
 
-def percentile_ms(values, q: float):
-    import numpy as np
-    return round(float(np.percentile(values, q)) * 1e3, 1) if len(values) else None
+class TokenTimes:
+    """When every request came and when each of its tokens left the engine; the latency figures follow from that."""
+
+    def __init__(self):
+        self.came: dict = {}
+        self.out: dict = {}
+        self.long: set = set()
+
+    def request(self, rid, at: float, is_long: bool) -> None:
+        self.came[rid] = at
+        self.out[rid] = []
+        if is_long:
+            self.long.add(rid)
+
+    def tokens(self, rids, at: float) -> None:
+        for rid in rids:
+            self.out[rid].append(at)
+
+    @staticmethod
+    def _ms(values, q: float):
+        import numpy as np
+        return round(float(np.percentile(values, q)) * 1e3, 1) if len(values) else None
+
+    def figures(self) -> dict:
+        import numpy as np
+        answered = {rid: ts for rid, ts in self.out.items() if ts}
+        to_first = {rid: ts[0] - self.came[rid] for rid, ts in answered.items()}
+        every = list(to_first.values())
+        long = [t for rid, t in to_first.items() if rid in self.long]
+        short = [t for rid, t in to_first.items() if rid not in self.long]
+        streams = [np.asarray(ts) for ts in answered.values() if len(ts) > 1]
+        between = np.concatenate([np.diff(ts) for ts in streams]) if streams else np.zeros(0)
+        per_token = [float(ts[-1] - ts[0]) / (len(ts) - 1) for ts in streams]
+        ms = self._ms
+        return {
+            "ttft_p50_ms": ms(every, 50), "ttft_p99_ms": ms(every, 99), "ttft_short_p99_ms": ms(short, 99),
+            "ttft_long_p50_ms": ms(long, 50), "ttft_long_p99_ms": ms(long, 99),
+            "itl_p50_ms": ms(between, 50), "itl_p99_ms": ms(between, 99), "itl_p999_ms": ms(between, 99.9),
+            "itl_max_ms": ms(between, 100),
+            "tpot_mean_ms": round(float(np.mean(per_token)) * 1e3, 1) if per_token else None,
+            "output_tokens": sum(len(ts) for ts in self.out.values()), "num_long": len(long),
+        }
 
 
 def serve(engine, arrivals: list, sampling_params_of) -> dict:
-    """Feeds the arrivals at their times, steps the engine in between, and notes when each request's
-    tokens come out (reference bench_latency.py:54-96)."""
-    import numpy as np
-    preempted_before = engine.scheduler.num_preemptions
-    due, stamps, came, is_long = 0, {}, {}, {}
+    """Serves `arrivals` (sorted by time) in real time: a request enters the engine once its time has come, the
+    engine steps whenever it holds a request, and sleeps until the next arrival when it holds none. Returns the
+    latency figures of the run (the quantities of reference bench_latency.py:78-96)."""
+    from collections import deque
+    waiting = deque(arrivals)
+    times = TokenTimes()
+    evictions_at_start = engine.scheduler.num_preemptions
     steps = 0
-    start = time.perf_counter()
-    while due < len(arrivals) or not engine.is_finished():
-        now = time.perf_counter() - start
-        while due < len(arrivals) and arrivals[due].at <= now:
-            a = arrivals[due]
-            rid = engine.add_request(a.prompt, sampling_params_of(a))
-            came[rid], stamps[rid], is_long[rid] = start + a.at, [], a.long
-            due += 1
-        if engine.is_finished():                                   # idle until the next arrival
-            time.sleep(max(0.0, arrivals[due].at - (time.perf_counter() - start)))
-            continue
-        _, _, _, emitted = engine.step()
-        steps += 1
-        t = time.perf_counter()
-        for rid in emitted:
-            stamps[rid].append(t)
-    wall = time.perf_counter() - start
+    t0 = time.perf_counter()
+    while True:
+        elapsed = time.perf_counter() - t0
+        while waiting and waiting[0].at <= elapsed:
+            a = waiting.popleft()
+            times.request(engine.add_request(a.prompt, sampling_params_of(a)), t0 + a.at, a.long)
+        if not engine.is_finished():
+            produced = engine.step()[3]
+            steps += 1
+            times.tokens(produced, time.perf_counter())
+        elif waiting:
+            pause = waiting[0].at - (time.perf_counter() - t0)
+            if pause > 0:
+                time.sleep(pause)
+        else:
+            break
+    wall = time.perf_counter() - t0
+    row = times.figures()
+    row.update(out_tok_s=round(row["output_tokens"] / wall, 1), wall_s=round(wall, 1), steps=steps,
+               preemptions=engine.scheduler.num_preemptions - evictions_at_start)
+    return row
 
-    first = {rid: ts[0] - came[rid] for rid, ts in stamps.items() if ts}
-    gaps = np.concatenate([np.diff(ts) for ts in stamps.values() if len(ts) > 1] or [np.zeros(0)])
-    per_token = [(ts[-1] - ts[0]) / (len(ts) - 1) for ts in stamps.values() if len(ts) > 1]
-    ttft_all = list(first.values())
-    ttft_long = [v for rid, v in first.items() if is_long[rid]]
-    ttft_short = [v for rid, v in first.items() if not is_long[rid]]
-    return {
-        "ttft_p50_ms": percentile_ms(ttft_all, 50), "ttft_p99_ms": percentile_ms(ttft_all, 99),
-        "ttft_short_p99_ms": percentile_ms(ttft_short, 99),
-        "ttft_long_p50_ms": percentile_ms(ttft_long, 50), "ttft_long_p99_ms": percentile_ms(ttft_long, 99),
-        "itl_p50_ms": percentile_ms(gaps, 50), "itl_p99_ms": percentile_ms(gaps, 99),
-        "itl_p999_ms": percentile_ms(gaps, 99.9),
-        "itl_max_ms": round(float(gaps.max()) * 1e3, 1) if len(gaps) else None,
-        "tpot_mean_ms": round(float(np.mean(per_token)) * 1e3, 1) if per_token else None,
-        "output_tokens": sum(len(ts) for ts in stamps.values()),
-        "out_tok_s": round(sum(len(ts) for ts in stamps.values()) / wall, 1), "wall_s": round(wall, 1), "steps": steps,
-        "preemptions": engine.scheduler.num_preemptions - preempted_before, "num_long": len(ttft_long),
-    }
+
+def sweep(engine, settings: list, rates: list, workload, num_reqs: int, sampling_params_of, emit) -> None:
+    """Every setting at every rate, the same arrivals for all settings of a rate; `emit(rate, setting, figures)`
+    takes each result as it is ready."""
+    for rate in rates:
+        arrivals = workload(num_reqs, rate)
+        for setting in settings:
+            setting.switch(engine)
+            emit(rate, setting, serve(engine, arrivals, sampling_params_of))
 
 
 def main(argv=None) -> int:
@@ -164,27 +215,31 @@ def main(argv=None) -> int:
                  max_num_batched_tokens=ENGINE_BUDGET, dtype=args.dtype, seed=args.seed)
     vocab = engine.model.embedding.vocab_size
     params_of = lambda a: SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=a.max_tokens)
-    settings = [s for s in args.configs.split(",") if s]
+    settings = [Setting.parse(name) for name in args.configs.split(",") if name]
+    for setting in settings:
+        setting.check(engine.scheduler)
     if int(7680 * args.scale) + int(256 * args.scale) > engine.scheduler.max_model_len:
         p.error(f"the longest request ({int(7680 * args.scale)} + {int(256 * args.scale)} tokens) exceeds "
                 f"max_model_len {engine.scheduler.max_model_len}: lower --scale")
     workload = lambda num, rate: poisson_arrivals(num, rate, args.long_frac, vocab, args.scale)
 
-    apply_setting(engine, "c2048")                   # warm-up: kernels, graphs and library plans
-    serve(engine, workload(20, 20.0), params_of)
+    # before anything is measured: a short, dense run that meets the kernels, graphs and library plans (reference :99-100)
+    sweep(engine, [Setting.parse("c2048")], [20.0], workload, 20, params_of, lambda *ignored: None)
 
     os.makedirs(os.path.dirname(args.out) or ".", exist_ok=True)
-    for rate in (float(r) for r in args.rates.split(",") if r):
-        arrivals = workload(args.num_reqs, rate)
-        for name in settings:
-            apply_setting(engine, name)
-            row = {"engine": "mini_engine_amd", "label": args.label, "config": name, "rate": rate,
-                   "num_reqs": args.num_reqs, "long_frac": args.long_frac, **serve(engine, arrivals, params_of),
-                   "model": args.random_weights or path, "dtype": args.dtype, "gpu": torch.cuda.get_device_name(0),
-                   "torch": torch.__version__, "time": datetime.now().isoformat(timespec="seconds")}
-            print(json.dumps(row), flush=True)
-            with open(args.out, "a") as f:
-                f.write(json.dumps(row) + "\n")
+    about = {"model": args.random_weights or path, "dtype": args.dtype, "gpu": torch.cuda.get_device_name(0),
+             "torch": torch.__version__}
+
+    def emit(rate, setting, figures):
+        row = {"engine": "mini_engine_amd", "label": args.label, "config": setting.name, "rate": rate,
+               "num_reqs": args.num_reqs, "long_frac": args.long_frac, **figures, **about,
+               "time": datetime.now().isoformat(timespec="seconds")}
+        text = json.dumps(row)
+        print(text, flush=True)
+        with open(args.out, "a") as f:
+            f.write(text + "\n")
+
+    sweep(engine, settings, [float(r) for r in args.rates.split(",") if r], workload, args.num_reqs, params_of, emit)
     if tmp is not None:
         tmp.cleanup()
     return 0

@@ -68,6 +68,7 @@ _CORE_PROTOS = {
     "me_gemm_mid_bf16": [P, L, P, L, P, L, I, I, I, I, I, I, P],
     "me_gemm_library_bf16": [P, L, P, L, P, L, I, P, ctypes.c_size_t, I, I, I, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
+    "me_sample_static": [P, L, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
     "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, I, P, P, I, P],
@@ -349,7 +350,9 @@ class HipBackend:
             col_tiles = prefill_col_tiles(max_prefill_context, win, Tp, Hq, D)
             seg_keys, max_segs = prefill_segments(max_prefill_context, win, Tp, Hq, D, col_tiles)
             waves = prefill_waves(max_prefill_context, Tp, B - num_decodes, Hq, Hkv, col_tiles, max_segs)
-            pf = torch.empty((Tp * Hq * max_segs * (D + 2),), dtype=torch.float32, device=q.device) if max_segs > 1 else None
+            # the segments' partial results: in a buffer that is kept between steps (a step's decode rows have
+            # finished with theirs before, on the same stream, but the two are kept apart all the same)
+            pf = _scratch(Tp * Hq * max_segs * (D + 2), q.device, "prefill") if max_segs > 1 else None
             lib.call("me_attn_prefill", q.data_ptr() + num_decodes * q.stride(0) * es, q.stride(0),
                      out.data_ptr() + num_decodes * out.stride(0) * es, out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
@@ -555,7 +558,13 @@ class HipBackend:
                "sample: temperatures must be float32 [S]")
         _check(keys.dtype == torch.int32 and keys.shape == (S, 2) and keys.is_contiguous(), "sample: keys must be int32 [S, 2]")
         out = torch.empty((S,), dtype=torch.int32, device=logits.device)
-        scratch = torch.empty((2 * S * 32,), dtype=torch.int32, device=logits.device)
+        if S <= SAMPLE_STATIC_MAX_ROWS:
+            # the per-chunk partial results stay in a device array of the library: nothing is allocated for them.
+            # (All calls on a GPU share that array; the engine samples on one stream, one call after the other.)
+            core().call("me_sample_static", logits.data_ptr(), logits.stride(0), temperatures.data_ptr(), keys.data_ptr(),
+                        out.data_ptr(), S, V, _stream())
+            return out
+        scratch = _scratch(2 * S * 32, logits.device, "sample")
         core().call("me_sample", logits.data_ptr(), logits.stride(0), temperatures.data_ptr(), keys.data_ptr(),
                     out.data_ptr(), scratch.data_ptr(), S, V, _stream())
         return out
@@ -630,17 +639,22 @@ _DECODE_WHOLE_MAX_KEYS = 4096
 _DECODE_EVEN_WHOLE_WORKGROUPS = 192
 _DECODE_EVEN_WHOLE_MAX_KEYS = 8192
 _DECODE_MAX_PARTITION = 2048
+SAMPLE_STATIC_MAX_ROWS = 1024     # ME_SAMPLE_STATIC_MAX_ROWS of csrc/sampling.h
 _scratch_buf: dict = {}
 _scratch_retired: list = []      # outgrown buffers stay alive: a captured graph may still write to them
 
 
-def _scratch(num_floats: int, device) -> torch.Tensor:
-    buf = _scratch_buf.get(device)
+def _scratch(num_floats: int, device, use: str = "decode") -> torch.Tensor:
+    """Device memory for a kernel's partial results (4-byte words), kept between calls: one buffer per device
+    and use, grown when a call needs more (by half as much again, so that a slowly growing need does not
+    allocate at every step), never shrunk."""
+    key = (device, use)
+    buf = _scratch_buf.get(key)
     if buf is None or buf.numel() < num_floats:
         if buf is not None:
             _scratch_retired.append(buf)
-        buf = torch.empty((max(2 * num_floats, 1 << 22),), dtype=torch.float32, device=device)
-        _scratch_buf[device] = buf
+        buf = torch.empty((max(num_floats + num_floats // 2, 1 << 20),), dtype=torch.float32, device=device)
+        _scratch_buf[key] = buf
     return buf
 
 

@@ -52,13 +52,16 @@ def _engine(folder, **kw):
 
 def test_settings_switch_the_scheduler_and_refuse_what_it_cannot_do(folders, plain_backend):
     llm = _engine(folders("B"))
-    cli_latency.apply_setting(llm, "c16")
+    Setting = cli_latency.Setting
+    assert Setting.parse("c16") == Setting("c16", True, 16) and Setting.parse("pf") == Setting("pf", False, cli_latency.ENGINE_BUDGET)
+    Setting.parse("c16").switch(llm)
     assert llm.scheduler.chunked and llm.scheduler.token_budget == 16
-    cli_latency.apply_setting(llm, "pf")
+    Setting.parse("pf").switch(llm)
     assert not llm.scheduler.chunked and llm.scheduler.token_budget == cli_latency.ENGINE_BUDGET
     for bad in ("c0", "c99999", "x12", "c", "c2"):     # c2: fewer tokens than requests that may decode
         with pytest.raises(ValueError):
-            cli_latency.apply_setting(llm, bad)
+            Setting.parse(bad).switch(llm)
+    assert not llm.scheduler.chunked and llm.scheduler.token_budget == cli_latency.ENGINE_BUDGET       # a refused setting changes nothing
 
 
 def test_serving_arrivals_gives_every_request_its_tokens_and_times(folders, plain_backend):
@@ -75,7 +78,7 @@ def test_serving_arrivals_gives_every_request_its_tokens_and_times(folders, plai
     params_of = lambda a: SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=a.max_tokens)
     rows = {}
     for name in ("c16", "pf"):
-        cli_latency.apply_setting(llm, name)
+        cli_latency.Setting.parse(name).switch(llm)
         r = rows[name] = cli_latency.serve(llm, arrivals, params_of)
         assert not llm.manager.held
         llm.manager.check_invariants()
@@ -85,6 +88,20 @@ def test_serving_arrivals_gives_every_request_its_tokens_and_times(folders, plai
         assert 0 <= r["ttft_p50_ms"] <= r["ttft_p99_ms"] and 0 <= r["itl_p50_ms"] <= r["itl_p99_ms"] <= r["itl_max_ms"]
         assert r["ttft_long_p50_ms"] is not None and r["ttft_short_p99_ms"] is not None and r["tpot_mean_ms"] >= 0
     assert rows["c16"]["steps"] >= 90 // 16                  # the longest prompt alone needs that many portions
+
+
+def test_token_times_give_the_figures_of_a_known_run():
+    """Two requests with hand-made times: first tokens after 10 and 30 ms, gaps of 2 ms and 4 ms."""
+    t = cli_latency.TokenTimes()
+    t.request("a", 100.0, False)
+    t.request("b", 100.5, True)
+    t.request("c", 101.0, False)                              # never answered: counts nowhere
+    t.tokens(["a"], 100.010); t.tokens(["a", "b"], 100.530); t.tokens(["b"], 100.534); t.tokens(["b"], 100.538)
+    f = t.figures()
+    assert f["output_tokens"] == 5 and f["num_long"] == 1
+    assert f["ttft_p50_ms"] == 20.0 and f["ttft_long_p50_ms"] == 30.0 and f["ttft_short_p99_ms"] == 10.0
+    assert f["itl_max_ms"] == 520.0 and f["itl_p50_ms"] == 4.0
+    assert f["tpot_mean_ms"] == round((520.0 + 4.0) / 2, 1)
 
 
 @pytest.mark.gpu

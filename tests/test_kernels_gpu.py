@@ -772,6 +772,35 @@ def test_sample_frequencies_follow_softmax():
     assert chi2 < 40.0, f"chi-square {chi2:.1f} with 11 degrees of freedom"   # p < 1e-4 under the null
 
 
+def test_kernels_allocate_nothing_beside_their_results(monkeypatch):
+    """The kernels' own scratch memory (partial results of split decode attention, of prefill attention cut into
+    segments, of the sampler's chunks) is kept between calls or lives in the library: once a shape has run, a call
+    asks the allocator for its result and nothing else."""
+    def allocations(fn):
+        fn()                                                  # the first call of a shape may size the kept buffers
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_stats()["allocation.all.allocated"]
+        out = fn()
+        torch.cuda.synchronize()
+        return torch.cuda.memory_stats()["allocation.all.allocated"] - before, out
+
+    logits = torch.randn(40, 20011, device=DEV)
+    temps = torch.full((40,), 0.7, device=DEV)
+    keys = torch.randint(-2 ** 31, 2 ** 31 - 1, (40, 2), device=DEV, dtype=torch.int32)
+    n, tokens = allocations(lambda: hip().sample(logits, temps, keys))
+    assert n == 1 and tokens.shape == (40,)
+    big = torch.randn(1030, 300, device=DEV)                  # more rows than the library's array holds: the kept buffer
+    n, tokens = allocations(lambda: hip().sample(big, torch.zeros(1030, device=DEV), keys[:1].expand(1030, 2).contiguous()))
+    assert n == 1 and tokens.tolist() == big.argmax(-1).tolist()
+    # prefill attention cut into segments, decode attention in partitions, both in one step
+    monkeypatch.setattr(ops, "PREFILL_SEGMENT_KEYS", 64)
+    args = _attention_case(torch.bfloat16, 16, 8, 128, 16, [(700, 1), (300, 1), (400, 130), (90, 7)], seed=5)
+    assert ops.decode_partitions(2, 16, 8, 700)[1] > 1 and ops.prefill_segments(400, 0, 137, 16)[1] > 1
+    n, out = allocations(lambda: hip().paged_attention(*args))
+    assert n == 1
+    close(out, twin.paged_attention(*args), 1.5e-2)
+
+
 def test_kernels_refuse_what_they_cannot_do():
     with pytest.raises(ops.KernelError, match="dtype"):
         hip().silu_and_mul(torch.zeros(2, 4, device=DEV, dtype=torch.float16))
