@@ -9,7 +9,10 @@ SIZES = {
     # name: (layers, hidden, q heads, kv heads, head_dim, intermediate, vocab, tied)
     "tinyA": (2, 64, 4, 2, 16, 128, 256, True),
     "0.6b": (28, 1024, 16, 8, 128, 3072, 151936, True),
+    "1.7b": (28, 2048, 16, 8, 128, 6144, 151936, True),
+    "4b": (36, 2560, 32, 8, 128, 9728, 151936, True),
     "8b": (36, 4096, 32, 8, 128, 12288, 151936, False),
+    "14b": (40, 5120, 40, 8, 128, 17408, 151936, False),
     "32b": (64, 5120, 64, 8, 128, 25600, 151936, False),
 }
 

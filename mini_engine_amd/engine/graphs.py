@@ -397,7 +397,13 @@ class MixedGraphs:
     few, and a step that the host bounds loses nothing by the padding. A layout that has come up
     `capture_after` times is captured on its next appearance and replayed from then on; larger steps, and
     layouts that come up once, stay eager and exactly sized. The captured work is the model's own forward pass
-    over the padded step."""
+    over the padded step.
+
+    Steps beyond `max_tokens` and up to `max_exact_tokens` (six times as many: up to there the host's launches
+    still leave gaps between the GPU's kernels) take a layout with the step's own token and request counts and
+    only the context cap and the rows of logits rounded: a prompt of 2,048 tokens alone, or a prompt's portions
+    under a fixed budget beside a constant number of decoding requests, come up again and again exactly so, and
+    nothing is lost to padding when they do not."""
 
     def __init__(self, runner, max_rows: int, capture: bool = True, capture_after: int = 4, max_graphs: int = 48,
                  max_tokens: int | None = None):
@@ -407,6 +413,7 @@ class MixedGraphs:
         self.capture_after = capture_after
         self.max_graphs = max_graphs
         self.max_tokens = host_bound_tokens(runner.model) if max_tokens is None else max_tokens
+        self.max_exact_tokens = 6 * self.max_tokens
         self.captured: dict = {}
         self.sightings: dict = {}
         self.pool = runner.graph_pool() if capture else None
@@ -415,9 +422,18 @@ class MixedGraphs:
     def padded(self, exact: StepLayout) -> StepLayout | None:
         r = self.runner
         tokens = exact.decode_rows + exact.prefill_tokens
-        if (exact.prefill_reqs == 0 or exact.rows > self.max_rows or tokens >= self.max_tokens or r.vocab_size is None
+        if (exact.prefill_reqs == 0 or exact.rows > self.max_rows or tokens >= self.max_exact_tokens or r.vocab_size is None
                 or not (r.device.type == "cuda" or not self.capture)):
             return None
+        ps = r.manager.page_size
+        if tokens >= self.max_tokens:
+            # the step's own counts; only what differs from step to step of a repeating pattern is rounded
+            cap = min(max(1024, _pow2_at_least(max(exact.decode_ctx, exact.prefill_ctx))), r.max_positions)
+            return StepLayout(
+                decode_rows=exact.decode_rows, prefill_reqs=exact.prefill_reqs, prefill_tokens=exact.prefill_tokens,
+                rows=bucket_of(exact.rows) if exact.rows else 0,
+                max_blocks=tuple(max(mb, -(-cap // ps)) for mb in exact.max_blocks),
+                decode_ctx=cap if exact.decode_rows else 0, prefill_ctx=cap, even=exact.even)
         decode_rows = bucket_of(exact.decode_rows) if exact.decode_rows else 0
         need = decode_rows + exact.prefill_tokens + 1
         total = max(32, _pow2_at_least(need)) if need <= 256 else _round_up(need, 64 if need <= 1024 else 128)
@@ -425,7 +441,6 @@ class MixedGraphs:
         if pad > r.max_positions:
             return None       # the padding request would stand at positions the engine does not have: run as it is
         cap = min(max(1024, _pow2_at_least(max(exact.decode_ctx, exact.prefill_ctx, pad))), r.max_positions)
-        ps = r.manager.page_size
         return StepLayout(
             decode_rows=decode_rows, prefill_reqs=exact.prefill_reqs + 1, prefill_tokens=total - decode_rows,
             rows=bucket_of(exact.rows) if exact.rows else 0,

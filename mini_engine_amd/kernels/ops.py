@@ -570,47 +570,19 @@ class HipBackend:
         return out
 
 
-# Rows up to which the skinny MFMA kernel beats the library product. Measured at Qwen3-0.6B sizes
-# (us, skinny / library): 32 rows qkv 4096x1024 6.0 / 11.2, gate_up 6144x1024 8.8 / 11.5; 64 rows
-# qkv 8.1 / 11.6 but gate_up 14.3 / 11.8, hence the smaller limit for weights above
-# SKINNY_WIDE_MAX_WEIGHT elements. Split over K with the sum left to the norm kernel
-# (product + norm): 64 rows o 1024x2048 10.6 / 11.3, down 1024x3072 11.9 / 14.3.
-SKINNY_MAX_M = 32
-SKINNY_WIDE_MAX_M = 64
+# Dispatch rules. Every threshold below was measured on one MI355X at the layer sizes of Qwen3-0.6B, 8B and 32B;
+# the tables behind each constant are kept in the repository's design notes, one line of reason here.
+SKINNY_MAX_M = 32                          # rows up to which the skinny kernel beats the library product
+SKINNY_WIDE_MAX_M = 64                     # ... for weights of up to SKINNY_WIDE_MAX_WEIGHT elements
 SKINNY_WIDE_MAX_WEIGHT = 5 * 1024 * 1024
-PARTIALS_MAX_M = 64      # rows up to which a product split over K (float32 partial sums) pays
-# Outputs this wide (the head over the vocabulary, gate/up of the largest sizes) go to the library, except up to
-# WIDE_OUTPUT_SKINNY_ROWS rows where the skinny kernel's wide loads apply (us, skinny to float32 / library: 151936 x 1024
-# at 1 / 8 / 12 / 16 rows 47.8 / 59.9, 51.0 / 62.3, 60.1 / 64.4, 67.9 / 66.3; 151936 x 2560 125 / 249, 141 / 246, 165 / 246,
-# 187 / 246; 151936 x 4096 182 / 252 (6.8 TB/s), 199 / 252, 224 / 257, 253 / 259; 151936 x 5120 231 / 308, 261 / 305, 306 /
-# 313, 355 / 318)
-LIBRARY_MIN_N = 32768
-WIDE_OUTPUT_SKINNY_ROWS = 12
-# Large weights go to the library from a row count on: every workgroup of the skinny kernel reads all of x, which
-# at 8 to 16 rows is as much traffic as the weights themselves. With its wide loads (skinny_wide: K in whole steps
-# of 128, up to 16 rows) the skinny kernel streams a large weight at 5.3-6.0 TB/s where the library reaches 4-5, and
-# stays ahead up to 16 rows over a K of up to 4,096 and up to 10 rows over a longer K. Measured with weights streamed
-# from HBM (us, skinny / library; gate_up with the gating: in the epilogue / a kernel behind the library's product):
-#   rows   qkv 6144x4096   o 4096x4096 (slices)   gate_up 24576x4096   down 4096x12288 (slices)
-#     1    11.3 / 14.5        7.9 / 15.4             33.6 / 48.8          18.2 / 21.8
-#     4    11.6 / 14.6        8.0 / 15.5             33.6 / 47.1          18.2 / 21.7
-#     8    12.4 / 14.5        8.2 / 15.5             34.6 / 47.0          19.0 / 21.7
-#    12    13.3 / 14.5        8.5 / 15.6             38.0 / 47.4          20.3 / 21.9
-#    16    14.6 / 14.5        9.0 / 15.5             42.2 / 47.3          22.6 / 22.3
-#   rows   qkv 10240x5120  o 5120x8192 (slices)   gate_up 51200x5120   gate_up 34816x5120   down 5120x25600 (slices)
-#     4    20.2 / 23.3       17.0 / 19.7             85.7 / 98.1          60.8 / 86.5          43.7 / 137
-#     8    22.4 / 23.7       17.3 / 20.2             94.8 / 98.5          64.3 / 80.2          47.3 / 138
-#    12    25.2 / 24.1       18.2 / 20.6            104.1 / 95.0          73.4 / 79.7          52.5 / 139
-#    16    29.0 / 24.5       19.7 / 21.2            119.8 / 95.4          84.0 / 81.0          60.5 / 140
-# (the library's choice for a very long K is poor, hence LIBRARY_MAX_K). Without the wide loads (K no multiple of
-# 128, or 17 rows and more) the library is level from 4 rows on: 6144x4096 at 4 / 8 / 16 / 32 rows 14.9 / 14.4,
-# 15.6 / 14.4, 18.3 / 14.5, 27.2 / 15.2; 24576x4096 42.4 / 45.7, 47.1 / 46.3, 55.1 / 46.3. All Qwen3-0.6B products
-# favour the skinny kernel (3.3-5.5 us against 7.4-12 us).
-LIBRARY_MIN_ROWS = 4
-LIBRARY_MIN_ROWS_WIDE = 17          # with the wide loads, K up to 4,096: never within their 16 rows
-LIBRARY_MIN_ROWS_WIDE_LONG_K = 11   # ... over a longer K
+PARTIALS_MAX_M = 64                        # rows up to which a product split over K (float32 partial sums) pays
+LIBRARY_MIN_N = 32768                      # outputs this wide (the head over the vocabulary) go to the library ...
+WIDE_OUTPUT_SKINNY_ROWS = 12               # ... except up to this many rows, where the skinny kernel's wide loads win
+LIBRARY_MIN_ROWS = 4                       # large weights go to the library from this many rows on ...
+LIBRARY_MIN_ROWS_WIDE = 17                 # ... with the wide loads and K up to 4,096: never within their 16 rows
+LIBRARY_MIN_ROWS_WIDE_LONG_K = 11          # ... over a longer K
 LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
-LIBRARY_MAX_K = 16384
+LIBRARY_MAX_K = 16384                      # the library's choice for a longer K is poor
 ROWS_MIN_WEIGHT = 16 * 1024 * 1024
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 # prefill attention, keys and values shared by a workgroup's waves through LDS: 0 never, 1 wherever it fits (written there
@@ -626,10 +598,7 @@ FUSE_NORM_INTO_LINEAR = True   # False: the norm kernel and the product behind i
 NORM_FUSE_MAX_M = 2
 NORM_FUSE_MAX_WEIGHT = 8 << 20
 FUSE_DECODE_STEP = True        # False: pure decode steps run norm/rotation/cache write and attention as two launches
-# The fused form evaluates the gate in every workgroup (N/16 of them), which is free while the
-# product waits for its weights but not over a long K: at 4096x12288, one row, fused 63 us against
-# 27 us for the plain product after a separate gating kernel (3 us).
-GATED_MAX_K = 4096
+GATED_MAX_K = 4096             # the gating in front of the down product is formed in every workgroup: not over a longer K
 GATED_MAX_M = 16
 _COMPUTE_UNITS = 256
 _DECODE_WORKGROUPS = 4096
@@ -662,9 +631,7 @@ def prefill_col_tiles(max_context: int, window: int, num_tokens: int, Hq: int, D
     """Column tiles (of 16 (token, head) pairs) per wave of the prefill kernel: 2 halves the reads of keys and
     values per product but needs twice the columns per workgroup, so it is for launches with many columns (32,768
     or more: 2,048 tokens of 16 heads), and for portions of 256 tokens or more of a prompt over 4,096 keys or
-    more, where each tile walks a long range and `prefill_segments` cuts that range into enough workgroups
-    (us at 16x128 heads, one tile / two: 512 tokens over 8,192 keys 96 / 65, over 16,384 172 / 120; 1,024 over
-    8,192 142 / 116; 256 over 32,768 176 / 128; 512 over 2,048 and 400 over 3,000 level: left at one).
+    more, where each tile walks a long range and `prefill_segments` cuts that range into enough workgroups.
     PREFILL_COL_TILES forces it."""
     if PREFILL_COL_TILES in (1, 2):
         return PREFILL_COL_TILES
@@ -680,17 +647,13 @@ def prefill_segments(max_context: int, window: int, num_tokens: int, Hq: int, D:
 
     A tile's key range grows with its position, and a step with few new tokens over a long context
     gives the kernel few workgroups, each walking the whole context. Cutting the ranges into
-    segments of at least 512 keys (1,024 over ranges beyond 4,096), run by different workgroups and merged by a second kernel,
-    evens the work out and fills the GPU: two segments for launches of 257 to 640 workgroups; three
+    segments of at least 512 keys (1,024 over ranges beyond 4,096), run by different workgroups and merged by a
+    second kernel, evens the work out and fills the GPU: two segments for launches of 257 to 640 workgroups; three
     for 129 to 256 when the ranges start short (a prompt from its beginning: tiles of 64 to all keys,
     which thirds balance better than halves) and two when they are all long (a later portion of a
     prompt: twice the workgroups fill the slots evenly); as many as give 768 workgroups below that.
-    Measured at 16x128 heads (us, whole / cut): 64 tokens over 32,768 keys 1406 / 99, 1,024 over 4,096
-    116 / 86, 2,048 over 8,192 333 / 237, one prompt of 4,096 tokens 166 / 135, of 2,048 86 / 56, of
-    1,536 52 / 43, of 1,024 36 / 33, 512 over 2,048 62 / 37. A portion of a prompt that runs with two column
-    tiles per wave before its launch has 32,768 columns (`prefill_col_tiles`) gets segments of 512 to 1,024
-    keys, as many as give about 512 workgroups (512 tokens over 8,192 keys: segments of 512 / 1,024 / 1,376
-    keys 80 / 65 / 74 us; 256 over 8,192: 49 / 61 / 61; 1,024 over 4,096: 77 / 63 / 87).
+    A portion of a prompt that runs with two column tiles per wave before its launch has 32,768 columns
+    (`prefill_col_tiles`) gets segments of 512 to 1,024 keys, as many as give about 512 workgroups.
     PREFILL_SEGMENT_KEYS forces a size."""
     span = min(max_context, window + 256) if window else max_context
     if PREFILL_SEGMENT_KEYS is not None:
@@ -732,10 +695,7 @@ def skinny_wide(N: int, K: int) -> int:
     """Whether the skinny product reads a weight [N, K] with its wide loads: a wave's load takes 256 contiguous bytes
     of each of four rows, marked as not to be kept by the caches, and the pieces reach their lanes through LDS. For
     weights of SKINNY_WIDE_MIN_WEIGHT elements or more (the kernel applies them to up to 16 rows and a K in whole
-    steps of 128). us, plain / wide, weights cold, the same bits: 24576 x 4096 with the gating at 1 / 3 / 8 rows
-    39.0 / 33.6, 41.1 / 33.9, 47.2 / 36.0; 4096 x 12288 in slices 21.8 / 18.8, 22.1 / 18.9; 5120 x 25600 53.0 / 44.5,
-    57.2 / 44.8; 6144 x 4096 13.1 / 11.2; 4096 x 4096 in slices 8.3 / 7.8; 6144 x 1024 at 1 / 8 rows 4.8 / 4.6, 5.4 /
-    5.0; 4096 x 1024 3.7 / 3.7 (small weights are over before the mark matters)."""
+    steps of 128); small weights are over before the mark matters."""
     return 1 if N * K >= SKINNY_WIDE_MIN_WEIGHT else 0
 
 
@@ -759,13 +719,7 @@ def library_splits(M: int, N: int, K: int) -> int:
     shapes); as a strided batch over slices of K it runs the same large-tile kernels on 2-8 times the
     tiles. From 33 rows (below, the skinny and the rows kernel are as fast or faster) to 1,024 (above,
     the tiles suffice and the partial sums, S x M x N x 4 bytes written and read again, cost more than
-    the split gains), for weights of 16 M elements or more. Measured, us (plain call / slices), weights
-    from HBM:
-      4096 x 4096:    48 rows 13.9 / 12.4 (8),  128 rows 24.4 / 15.3 (8),  256 rows 22.7 / 20.0 (8),  1024 rows 44.4 / 38.6 (2)
-      4096 x 12288:   48 rows 33.6 / 25.7 (8),  128 rows 67.4 / 29.2 (8),  256 rows 55.3 / 34.5 (8),  512 rows 83.1 / 52.9 (4)
-      5120 x 8192:    48 rows 42.8 / 25.2 (8),  128 rows 44.7 / 29.9 (8),  256 rows 74.2 / 34.0 (8),  512 rows 68.0 / 46.5 (4)
-      5120 x 25600:   48 rows 152 / 55.9 (8),   128 rows 182 / 65.9 (8),   256 rows 263 / 80.2 (8),   1024 rows 350 / 222 (2)
-    (the rows kernel at 48 and 64 rows of 5120 x 25600: 82 and 87)."""
+    the split gains), for weights of 16 M elements or more."""
     if not (LIBRARY_SPLIT_MIN_ROWS <= M <= LIBRARY_SPLIT_MAX_ROWS) or N * K < LIBRARY_SPLIT_MIN_WEIGHT:
         return 1
     if not library_is_direct():
@@ -781,14 +735,7 @@ def rows_takes(M: int, N: int, K: int) -> bool:
     workgroup, the tokens staged once per workgroup in LDS, K split over up to 8 workgroups): large
     weights with 17 to 64 rows, where the skinny kernel reads the tokens again for every 16 features and
     the library streams at 1.7-3.5 TB/s, and from 8 rows on over a K too long for the library that is no multiple
-    of 128 (otherwise the skinny kernel's wide loads are ahead up to 16 rows: 5120 x 25600 at 8 / 16 rows 47.3 / 60.5
-    us against 63.2 here at 8).
-    Measured, us (rows kernel / best of library and skinny), weights from HBM:
-      4096 x 4096:   24 rows 10.6 / 13.2,  48 rows 13.5 / 13.6,  64 rows 14.6 / 15.0
-      4096 x 12288:  24 rows 25.0 / 26.9,  48 rows 30.2 / 33.6,  64 rows 31.7 / 37.3
-      5120 x 8192:   24 rows 23.3 / 26.0,  48 rows 28.0 / 43.1,  64 rows 33.3 / 29.2 (left to the library)
-      5120 x 25600:   8 rows 63.2 / 66.8,  32 rows 70.7 / 109,   64 rows 86.6 / 157
-      2560 x 9728:   24 rows 19.2 / 19.1,  48 rows 26.4 / 20.5 (left to the library)"""
+    of 128 (otherwise the skinny kernel's wide loads are ahead up to 16 rows)."""
     if N * K < ROWS_MIN_WEIGHT or K < 4096 or K % 8 or M > 64 or library_splits(M, N, K) > 1:
         return False
     if M > 16:
@@ -800,10 +747,7 @@ def rows_wide(M: int, N: int, ksplit: int) -> int:
     """Whether the rows kernel reads its weights with the wide loads of the skinny kernel (`skinny_wide`): up to 32
     rows and with two workgroups or more to a compute unit. The pass through LDS lengthens a wave's chain from load
     to product, which other workgroups on the compute unit must fill, and the wave tiles' 17 KB beside 48-64 KB of
-    staged tokens leave room for one workgroup only. us, plain / wide, in 8 slices of K: 4096 x 4096 at 17 / 32 rows
-    10.4 / 9.8, 11.4 / 10.8; 4096 x 12288 24.2 / 22.3, 25.7 / 23.8; 5120 x 8192 22.4 / 19.3, 24.2 / 21.6; 5120 x 25600
-    67.5 / 53.8, 69.8 / 56.5; at 48 / 64 rows 4096 x 12288 30.0 / 29.4, 31.5 / 46.3; unsplit (96-384 workgroups):
-    6144 x 4096 at 17 rows 26.2 / 33.3, 24576 x 4096 52.2 / 49.0, at 64 rows 63.8 / 108."""
+    staged tokens leave room for one workgroup only."""
     return 1 if M <= 32 and -(-N // 64) * ksplit >= 2 * _COMPUTE_UNITS else 0
 
 
@@ -817,7 +761,8 @@ def rows_ksplit(K: int) -> int:
 
 
 def library_streams_better(M: int, N: int, K: int) -> bool:
-    """Whether a product of few rows goes to the library rather than the skinny kernel."""
+    """Whether a product of few rows goes to the library rather than the skinny kernel: every workgroup of the
+    skinny kernel reads all of x, which at 8 to 16 rows is as much traffic as a large weight itself."""
     if N * K < LIBRARY_MIN_WEIGHT or K > LIBRARY_MAX_K:
         return False
     if K % 128 == 0 and M <= 16 and skinny_wide(N, K):
@@ -833,11 +778,7 @@ def choose_ksplit(M: int, N: int, K: int) -> int:
     that the consumer reads. The split with the least of that is taken, each split keeping 512 of K or more (4
     steps of 128, one per wave); with 256 feature tiles or more only over a K of 4,096 or more, where an uneven
     count (320 tiles: one round and a quarter) costs a quarter of the stream, and only up to 32 rows (beyond, the
-    library is level or ahead). Measured, product + norm in us by splits 1 / 2 / 3 / 4 / 6 / 8, one row:
-      1024 x 2048 (64 tiles):    6.8 / 5.6 / 5.5 / 5.3 / 5.7 / 5.6      1024 x 3072:  8.1 / 6.4 / 5.9 / 5.9 / 6.1 / 6.0
-      2048 x 6144 (128 tiles):   11.7 / 9.0 / 10.9 / 10.2 / 9.2 / 9.5   2560 x 9728 (160): 16.1 / 17.9 / 14.4 / 15.7 / 15.8 / 15.2
-      4096 x 12288 (256 tiles):  23.9 / 24.6 / 25.6 / 24.9 / 24.9 / 28.4
-      5120 x 8192 (320 tiles):   29.1 / 24.0 / 22.7 / 22.2 / 24.1 / 23.8   5120 x 25600: 73.3 / 60.4 / 56.8 / 52.1 / 54.4 / 53.7"""
+    library is level or ahead)."""
     tiles = -(-N // 16) * -(-M // 64)
     if tiles >= _COMPUTE_UNITS and (K < 4096 or M > SKINNY_MAX_M):
         return 1
@@ -854,15 +795,9 @@ def choose_ksplit(M: int, N: int, K: int) -> int:
 def mid_takes(M: int, N: int, K: int, partials: bool) -> int:
     """Whether the product of M rows against a bfloat16 weight [N, K] goes to the own kernel for a few hundred rows
     over small weights (csrc/gemm_mid.hip), and in how many slices of K: 0 no, 1 one result, 4 float32 partial
-    sums over four slices (only when the consumer adds them, `partials`).
-
-    Its time is 7 us whatever the row count up to 256 (tiles of 64 x 64, one workgroup to a compute unit), where
-    the library's grows with the rows. us, own / library, weights warm, replayed: 4096 x 1024 at 65 / 128 / 192 /
-    256 / 384 rows 7.2 / 7.2 / 7.4 / 7.5 / 9.1 against 6.9 / 8.7 / 10.2 / 8.1 / 9.2; 6144 x 1024 7.2 / 7.3 / 8.8 /
-    9.3 / 11.9 against 7.7 / 8.6 / 10.3 / 11.9 / 12.2; with few output features and a long K in four slices:
-    1024 x 2048 at 65 / 256 / 512 rows 5.1 / 5.5 / 7.2 against 6.4 / 7.2 / 9.0, 1024 x 3072 6.1 / 6.6 / 9.3 against
-    6.7 / 8.7 / 11.5. Beyond 8 M weight elements (4096 x 2048 and up) and beyond these row counts the library's
-    larger tiles win (6144 x 1024 at 512 rows 14.6 against 12.7, 12288 x 2048 at 256 rows 23.5 against 23.0)."""
+    sums over four slices (only when the consumer adds them, `partials`). Its time is 7 us whatever the row count
+    up to 256 (tiles of 64 x 64, one workgroup to a compute unit), where the library's grows with the rows; beyond
+    8 M weight elements and beyond these row counts the library's larger tiles win."""
     if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 256 or N * K > MID_MAX_WEIGHT or M <= 32:
         return 0
     if partials and N <= 2048 and K >= 2048 and M <= 512:
@@ -876,13 +811,8 @@ def prefill_waves(max_context: int, num_tokens: int, num_seqs: int, Hq: int, Hkv
     Three waves of 168 registers where two column tiles per wave are in use, the tiles are left whole, there are
     2,048 workgroups or more, and the prompts start at their beginning (the longest context at most twice the mean
     number of new tokens per sequence): tiles of all lengths are then under way at once and the third wave fills
-    the others' waits. us, two / three waves, the best of four runs taken in turn: one prompt at 16 query heads of
-    8,192 tokens 277 / 300, of 16,384 1,014 / 986, of 32,768 3,977 / 3,760; at 32 heads 8,192 tokens 511 / 504,
-    16,384 1,995 / 1,890; at 64 heads 4,096 tokens 282 / 271, 8,192 1,028 / 967, 16,384 3,994 / 3,751 (the
-    crossing lies at about 2,000 workgroups in each case). Portions over a long prefix, whose tiles are equally
-    long and walk the same keys together, run better with two waves and 205 registers (2,048 tokens over 8,192
-    keys at 64 heads 475 / 533, over 6,000 keys 333 / 377), and so do launches of few workgroups (512 tokens over
-    8,192 keys 56 / 64)."""
+    the others' waits. Portions over a long prefix, whose tiles are equally long and walk the same keys together,
+    run better with two waves and 205 registers, and so do launches of few workgroups."""
     if col_tiles != 2 or max_segs != 1 or num_seqs < 1 or max_context <= 0:
         return 2
     group = max(1, Hq // max(1, Hkv))
@@ -901,20 +831,14 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
     heads x partitions) already gives several workgroups per compute unit, or to keep the
     number of partitions to merge at 64 or less. A partition holds at most 2,048 keys (as long as 64
     partitions cover the context): a workgroup goes through its keys round by round, so in a batch with
-    a few long contexts among short ones the long partitions are what is still running at the end
-    (128 sequences, four of 16 k keys among 100-2,048: 4096 x 4 311 us, 2048 x 8 283 us, 1024 x 16 280 us).
+    a few long contexts among short ones the long partitions are what is still running at the end.
     From 768 workgroups on (96 sequences x 8 kv heads) a context up to 2,048 keys (4,096 from 2,048 workgroups
-    on) is one partition and needs no reduce kernel (us, split / whole: 256 x 4,096 keys 752 / 719; 256 x 100-600 keys 83 / 74; contexts
-    of 100-2,048 keys: 192 sequences 159 / 145, 128 sequences 107 / 98, 100 of 600-2,048 keys 105 / 95; below, 40
-    sequences of 1,000-2,048 keys 41.6 / 44.2 and 64 of 100-2,048
-    56.1 / 55.8, hence the 768). `even` (the contexts are equally long, `decode_contexts_even`): from 192 workgroups on (24
-    sequences x 8 kv heads) a context up to 8,192 keys is one partition: every workgroup then has the same
-    work, none waits for another's partial results and no reduce kernel follows (us, default split / one
-    partition: 24 x 2,048 keys 34.2 / 32.9, 32 x 2,048 44.1 / 39.6, 64 x 2,048 104.9 / 97.3, 64 x 512
-    25.9 / 21.7, 32 x 8,192 196.5 / 182.0, 128 x 2,048 201.8 / 187.7; 16 x 2,048 25.3 / 31.0, hence the
-    192; contexts of 100-2,048 keys gain nothing from it and long ones among short ones lose, hence only
-    for equal ones). (The reference's rule: layers/ops.py:44-51, split when sequences x kv heads cannot
-    fill the SMs, 256-key partitions.)"""
+    on) is one partition and needs no reduce kernel. `even` (the contexts are equally long,
+    `decode_contexts_even`): from 192 workgroups on (24 sequences x 8 kv heads) a context up to 8,192 keys is one
+    partition: every workgroup then has the same work, none waits for another's partial results and no reduce
+    kernel follows; contexts of different lengths gain nothing from it and long ones among short ones lose.
+    (The reference's rule: layers/ops.py:44-51, split when sequences x kv heads cannot fill the SMs, 256-key
+    partitions.)"""
     col_tiles = (Hq // Hkv + 15) // 16
     base = max(1, num_seqs * Hkv * col_tiles)
     ctx = max(1, max_context)
@@ -932,24 +856,20 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
 def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     """Whether `rows` rows against the packed gate/up weight w [2 I, K] are few enough, and w of a kind, for the
     gating to happen in the product's epilogue: a bfloat16 product that the unsplit skinny kernel takes, up to
-    GATED_EPILOGUE_MAX_M rows, or one of 33-256 rows that the tiled kernel for small weights takes (`mid_takes`). At
-    the 0.6B widths the gating in front of the down product costs every one of that product's workgroups about 2 us;
-    behind gate/up every gate is formed once. At 33-256 rows the gating was a kernel of its own: a layer's feed-forward,
-    us, apart / in the epilogue: 40 rows 17.5 / 14.8, 64 rows 18.8 / 15.9, 128 rows 20.6 / 17.5, 256 rows 24.6 / 20.4."""
+    GATED_EPILOGUE_MAX_M rows, or one of 17-256 rows that the tiled kernel for small weights takes (`mid_takes`).
+    In front of the down product the gating costs every one of that product's workgroups about 2 us; behind
+    gate/up every gate is formed once."""
     if not FUSE_GATE_INTO_GATE_UP or w.dtype != torch.bfloat16 or w.dim() != 2:
         return False
     N, K = w.shape
     # over large weights the library takes the product from a row count on (library_streams_better), and the gating is
     # then a kernel of its own; without the skinny kernel's wide loads (K no multiple of 128) the skinny kernel with the
-    # gating in its epilogue is still ahead of the two up to 8 rows over a K of 4,096 (4096 -> 24576, us: 4 rows 38.9 /
-    # 45.5, 8 rows 43.9 / 45.5, 12 rows 49.2 / 46.2)
+    # gating in its epilogue is still ahead of the two up to 8 rows over a K of 4,096
     takes = skinny_takes(rows, N, K) or (rows <= 8 and K <= 4096 and N < LIBRARY_MIN_N and rows <= SKINNY_MAX_M)
     aligned = N % 2 == 0 and K % 8 == 0 and w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
     if rows > GATED_EPILOGUE_MAX_M:
-        # a few hundred rows over a small weight: the kernel that takes the product (mid_takes) gates in its epilogue too,
-        # in place of a kernel of its own behind it; and from 17 rows on, where the skinny kernel would have the product
-        # itself: a layer's feed-forward at the 0.6B sizes, us, skinny product + gating + down / tiled product with the
-        # gating + down: 17 rows 14.1 / 13.6, 24 rows 14.8 / 13.8, 32 rows 15.9 / 14.1
+        # the kernel for a few hundred rows over a small weight gates in its epilogue too, in place of a kernel of
+        # its own behind it; and from 17 rows on, where the skinny kernel would have the product itself
         if not (aligned and N % 8 == 0):
             return False
         if rows <= 32:
@@ -968,10 +888,7 @@ def norm_linear_fuses(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether `norm_linear` takes rows x ([M, K], or float32 partial sums [S, M, K]) and weight w: a
     bfloat16 weight that the unsplit skinny kernel would take, one or two rows, a weight of at most
     NORM_FUSE_MAX_WEIGHT elements. Every workgroup forms the normed rows for itself, which costs each about
-    2 us; the norm kernel costs 3 us in a chain of decode kernels. Measured, us (two launches / one):
-    1024 -> 4096 with 4 partial sums: 1 row 6.4 / 5.4, 2 rows 6.3 / 5.7, 3 rows 6.4 / 7.5, 8 rows 6.6 / 11.2;
-    1024 -> 6144 with 6: 1 row 7.7 / 6.7, 2 rows 7.7 / 6.9, 4 rows 7.8 / 9.7; 4096 -> 6144: 1 row 16.5 / 15.7,
-    2 rows 16.2 / 16.2; 4096 -> 24576: 1 row 41.4 / 44.8 (the prologue delays the weight stream)."""
+    2 us; the norm kernel costs 3 us in a chain of decode kernels, so it pays for one and two rows only."""
     if not FUSE_NORM_INTO_LINEAR or w.dtype != torch.bfloat16 or w.dim() != 2 or x.dim() not in (2, 3):
         return False
     S = x.shape[0] if x.dim() == 3 else 1
@@ -996,10 +913,8 @@ def decode_step_fuses(dtype: torch.dtype, D: int, page: int) -> bool:
 def decode_contexts_even(num_seqs: int, min_context: int, max_context: int) -> bool:
     """Whether the decode kernel may keep each request's work on one XCD (8 requests or more whose
     contexts differ by 5 % at most), or has to spread every request over the XCDs. With all of a request
-    on one XCD, the XCD that draws the long contexts finishes last: 64 contexts of 100-2,048 keys took
-    58.6 us against 48.5 us spread, and one of 32 k keys among 255 short ones 434 against 138 us; with
-    equal contexts the spread costs 1-3 % (decode of 64 x 2,048 keys at the 8B sizes: 8.9 against 8.6 ms
-    a step), for the block-table reads that a request's heads no longer share in one L2."""
+    on one XCD, the XCD that draws the long contexts finishes last; with equal contexts the spread costs
+    1-3 % for the block-table reads that a request's heads no longer share in one L2."""
     return num_seqs >= 8 and min_context > 0 and (max_context - min_context) * 20 <= max_context
 
 

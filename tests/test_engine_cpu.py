@@ -18,10 +18,11 @@ from mini_engine_amd.weights.loader import load_model
 class Env:
     device, dtype, tol = "cpu", torch.float32, helpers.TOL_F32
 
-    def __init__(self, folders, graphs=False):
+    def __init__(self, folders, graphs=False, padded_up_to=4096):
         self.folders = folders
         self.models = {}
         self.graphs = graphs           # every step through the fixed layouts (padded; captured where there is a GPU)
+        self.padded_up_to = padded_up_to
 
     def runner(self, name, pages):
         folder = self.folders(name)
@@ -29,7 +30,7 @@ class Env:
             self.models[name] = load_model(folder, self.device, self.dtype, 512)
         model = self.models[name]
         manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
-        options = dict(use_graphs=True, mixed_graphs_after=0, mixed_graphs_max_tokens=4096) if self.graphs else {}
+        options = dict(use_graphs=True, mixed_graphs_after=0, mixed_graphs_max_tokens=self.padded_up_to) if self.graphs else {}
         return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True, **options), manager, folder
 
 
@@ -50,6 +51,17 @@ def test_cuts_through_padded_layouts(folders, plain_backend, case, name):
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_padded_layouts_are_used(folders, plain_backend, name):
     engine_cases.padded_layouts_are_used(Env(folders, graphs=True), name, captured=False)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_exactly_sized_layouts_are_used(folders, plain_backend, name):
+    engine_cases.exactly_sized_layouts_are_used(Env(folders, graphs=True, padded_up_to=16), name, captured=False)
+
+
+@pytest.mark.parametrize("name", ["B"])
+@pytest.mark.parametrize("case", [engine_cases.changing_portions, engine_cases.mixed_with_reuse], ids=lambda c: c.__name__)
+def test_cuts_through_exactly_sized_layouts(folders, plain_backend, case, name):
+    case(Env(folders, graphs=True, padded_up_to=16), name)
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])

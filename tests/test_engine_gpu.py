@@ -18,6 +18,7 @@ class Env:
 
     def __init__(self, folders, dtype, graphs=False):
         self.folders, self.dtype = folders, dtype
+        self.padded_up_to = 4096
         self.graphs = graphs           # every step through a captured graph of its padded layout
         self.tol = helpers.TOL_F32 if dtype == torch.float32 else helpers.TOL_BF16
         self.models = {}
@@ -28,7 +29,7 @@ class Env:
             self.models[name] = load_model(folder, self.device, self.dtype, 512)
         model = self.models[name]
         manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
-        options = dict(use_graphs=True, mixed_graphs_after=0, mixed_graphs_max_tokens=4096) if self.graphs else {}
+        options = dict(use_graphs=True, mixed_graphs_after=0, mixed_graphs_max_tokens=self.padded_up_to) if self.graphs else {}
         return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True, **options), manager, folder
 
 
@@ -59,6 +60,14 @@ def test_padded_layouts_are_captured_and_replayed(env, name):
     graphs = Env(env.folders, env.dtype, graphs=True)
     graphs.models = env.models
     engine_cases.padded_layouts_are_used(graphs, name, captured=True)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_exactly_sized_layouts_are_captured_and_replayed(env, name):
+    graphs = Env(env.folders, env.dtype, graphs=True)
+    graphs.models, graphs.padded_up_to = env.models, 16
+    engine_cases.exactly_sized_layouts_are_used(graphs, name, captured=True)
+    engine_cases.mixed_with_reuse(graphs, name)
 
 
 def test_hip_libraries_are_the_ones_running(env):

@@ -790,7 +790,8 @@ def test_kernels_allocate_nothing_beside_their_results(monkeypatch):
     n, tokens = allocations(lambda: hip().sample(logits, temps, keys))
     assert n == 1 and tokens.shape == (40,)
     big = torch.randn(1030, 300, device=DEV)                  # more rows than the library's array holds: the kept buffer
-    n, tokens = allocations(lambda: hip().sample(big, torch.zeros(1030, device=DEV), keys[:1].expand(1030, 2).contiguous()))
+    no_noise, same_keys = torch.zeros(1030, device=DEV), keys[:1].expand(1030, 2).contiguous()
+    n, tokens = allocations(lambda: hip().sample(big, no_noise, same_keys))
     assert n == 1 and tokens.tolist() == big.argmax(-1).tolist()
     # prefill attention cut into segments, decode attention in partitions, both in one step
     monkeypatch.setattr(ops, "PREFILL_SEGMENT_KEYS", 64)
