@@ -448,14 +448,17 @@ class HipBackend:
             core().call("me_gemm_rows_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
                         ME_F32, parts.data_ptr(), ksplit, M, N, K, rows_wide(M, N, ksplit), _stream())
             return parts
-        ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype
+        # 33-64 rows over few output features and a long K: the tiled kernel's four slices are ahead of the skinny split
+        mid_first = allow_partials and out_dtype == x.dtype and mid_takes(M, N, K, True) == 4
+        ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype and not mid_first
+                                            and (M <= SKINNY_MAX_M or N * K <= SKINNY_WIDE_MAX_WEIGHT)
                                             and not library_streams_better(M, N, K)) else 1
         if ksplit > 1:
             parts = torch.empty((ksplit, M, N), dtype=torch.float32, device=x.device)
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
                         ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, 0, skinny_wide(N, K), _stream())
             return parts
-        if skinny_takes(M, N, K):
+        if skinny_takes(M, N, K) and not mid_first:
             y = new()
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), None, 1, M, N, K, 0, 0, skinny_wide(N, K), _stream())
@@ -581,9 +584,10 @@ WIDE_OUTPUT_SKINNY_ROWS = 12               # ... except up to this many rows, wh
 LIBRARY_MIN_ROWS = 4                       # large weights go to the library from this many rows on ...
 LIBRARY_MIN_ROWS_WIDE = 17                 # ... with the wide loads and K up to 4,096: never within their 16 rows
 LIBRARY_MIN_ROWS_WIDE_LONG_K = 11          # ... over a longer K
-LIBRARY_MIN_WEIGHT = 20 * 1024 * 1024
+LIBRARY_MIN_WEIGHT = 15 * 1024 * 1024
 LIBRARY_MAX_K = 16384                      # the library's choice for a longer K is poor
-ROWS_MIN_WEIGHT = 16 * 1024 * 1024
+ROWS_MIN_WEIGHT = 10 * 1024 * 1024
+ROWS_FEW_FEATURES = 3072
 PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forces that many keys per segment (0: never cut)
 # prefill attention, keys and values shared by a workgroup's waves through LDS: 0 never, 1 wherever it fits (written there
 # by the loads themselves at head size 128 and pages of 16 keys or more), 2 as 1 but always staged through registers
@@ -592,6 +596,7 @@ PREFILL_COL_TILES = 0     # 0: chosen by prefill_col_tiles(); 1 or 2 force the c
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
 USE_MID_PRODUCT = True          # False: products of 33-512 rows over small weights go to the library like the larger ones
 MID_MAX_WEIGHT = 8 << 20
+MID_SMALL_WEIGHT = 13 << 19     # 6.5 M elements: gate/up at the 0.6B sizes (6.3 M) keeps the own kernel and its gating epilogue
 FUSE_GATE_INTO_GATE_UP = True  # False: silu(gate) * up is formed in front of the down product, not behind gate_up
 GATED_EPILOGUE_MAX_M = 16
 FUSE_NORM_INTO_LINEAR = True   # False: the norm kernel and the product behind it always run as two launches
@@ -709,7 +714,8 @@ def skinny_takes(M: int, N: int, K: int) -> bool:
 
 LIBRARY_SPLIT_MIN_ROWS = 33
 LIBRARY_SPLIT_MAX_ROWS = 1024
-LIBRARY_SPLIT_MIN_WEIGHT = 16 << 20
+LIBRARY_SPLIT_MIN_WEIGHT = 10 << 20
+LIBRARY_SPLIT_SURE_WEIGHT = 16 << 20
 
 
 def library_splits(M: int, N: int, K: int) -> int:
@@ -719,8 +725,12 @@ def library_splits(M: int, N: int, K: int) -> int:
     shapes); as a strided batch over slices of K it runs the same large-tile kernels on 2-8 times the
     tiles. From 33 rows (below, the skinny and the rows kernel are as fast or faster) to 1,024 (above,
     the tiles suffice and the partial sums, S x M x N x 4 bytes written and read again, cost more than
-    the split gains), for weights of 16 M elements or more."""
+    the split gains), for weights of 10 M elements or more."""
     if not (LIBRARY_SPLIT_MIN_ROWS <= M <= LIBRARY_SPLIT_MAX_ROWS) or N * K < LIBRARY_SPLIT_MIN_WEIGHT:
+        return 1
+    if N * K < LIBRARY_SPLIT_SURE_WEIGHT and K < 6144 and M < 128:
+        return 1          # the smaller of these weights over a short K: the plain call is ahead below 128 rows
+    if rows_has_few_features(M, N, K):
         return 1
     if not library_is_direct():
         return 1
@@ -730,13 +740,24 @@ def library_splits(M: int, N: int, K: int) -> int:
     return splits
 
 
+def rows_has_few_features(M: int, N: int, K: int) -> bool:
+    """33 to 64 rows over a weight of up to ROWS_FEW_FEATURES output features and a K of 8,192 or more (down at the 4B
+    sizes): the rows kernel's own split over K is ahead of the library's slices and of its plain call."""
+    return 32 < M <= 64 and N <= ROWS_FEW_FEATURES and K >= 8192 and K % 8 == 0 and N * K >= ROWS_MIN_WEIGHT
+
+
 def rows_takes(M: int, N: int, K: int) -> bool:
     """Whether a product whose consumer adds float32 partial sums goes to the rows kernel (64 features per
     workgroup, the tokens staged once per workgroup in LDS, K split over up to 8 workgroups): large
     weights with 17 to 64 rows, where the skinny kernel reads the tokens again for every 16 features and
     the library streams at 1.7-3.5 TB/s, and from 8 rows on over a K too long for the library that is no multiple
-    of 128 (otherwise the skinny kernel's wide loads are ahead up to 16 rows)."""
-    if N * K < ROWS_MIN_WEIGHT or K < 4096 or K % 8 or M > 64 or library_splits(M, N, K) > 1:
+    of 128 (otherwise the skinny kernel's wide loads are ahead up to 16 rows); and 33 to 64 rows over a weight with
+    few output features (up to ROWS_FEW_FEATURES) and a K of 8,192 or more, where the library's slices of K are poor."""
+    if N * K < ROWS_MIN_WEIGHT or K < 4096 or K % 8 or M > 64:
+        return False
+    if rows_has_few_features(M, N, K):
+        return True       # few output features over a long K: the library's slices have too few tiles here too
+    if library_splits(M, N, K) > 1:
         return False
     if M > 16:
         return M <= 32 or K >= 12288
@@ -800,8 +821,10 @@ def mid_takes(M: int, N: int, K: int, partials: bool) -> int:
     8 M weight elements and beyond these row counts the library's larger tiles win."""
     if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 256 or N * K > MID_MAX_WEIGHT or M <= 32:
         return 0
-    if partials and N <= 2048 and K >= 2048 and M <= 512:
+    if partials and N <= 2048 and K >= 2048 and M <= (512 if N <= 1024 else 256):
         return 4
+    if N * K > MID_SMALL_WEIGHT and M < 128:
+        return 0          # the larger of the small weights with few rows: the library's tiles are ahead
     return 1 if M <= 256 else 0
 
 

@@ -135,10 +135,10 @@ def test_library_slices_of_k_for_o_and_down_at_many_rows():
     assert ops.library_splits(256, 5120, 25600) == 8 and ops.library_splits(257, 5120, 25600) == 4
     assert ops.library_splits(512, 5120, 8192) == 4 and ops.library_splits(1024, 5120, 8192) == 2
     assert ops.library_splits(1025, 5120, 8192) == 1
-    assert ops.library_splits(128, 1024, 3072) == 1 and ops.library_splits(128, 2048, 8192) == 8   # 16 M elements or more
+    assert ops.library_splits(128, 1024, 3072) == 1 and ops.library_splits(128, 2048, 8192) == 8   # 10 M elements or more
     assert ops.library_splits(64, 1400, 12296) == 1      # 12296 = 8 x 1537: no two equal slices of a multiple of 8
     assert ops.library_splits(64, 4096, 4096 + 32) == 4  # 4128 = 4 x 1032
-    for M, N, K in ((100, 4096, 4096), (300, 5120, 17408), (40, 2560, 9728)):
+    for M, N, K in ((100, 4096, 4096), (300, 5120, 17408), (100, 2560, 9728)):
         s = ops.library_splits(M, N, K)
         assert s > 1 and K % (8 * s) == 0 and K // s >= 512
 
@@ -148,3 +148,31 @@ def test_requests_stay_on_one_xcd_only_when_their_contexts_are_equally_long():
     assert not ops.decode_contexts_even(64, 1900, 2100) and not ops.decode_contexts_even(256, 100, 2048)
     assert not ops.decode_contexts_even(7, 2048, 2048)          # fewer requests than XCDs: spread
     assert not ops.decode_contexts_even(8, 0, 0)                # unknown
+
+
+def test_rules_at_the_layer_sizes_between_the_measured_ones():
+    """What was corrected after the products of the 1.7B (2048 / 6144), 4B (2560 / 9728) and 14B (5120 / 17408) layer sizes
+    were timed beside every other kernel: each line is a place where the rule had picked the slower one."""
+    # down at the 1.7B sizes (12.6 M elements): the library's slices of K from 33 rows (64 rows: 16.9 -> 9.0 us), the rows
+    # kernel at 17-32 (32 rows: 11.0 -> 9.1)
+    assert ops.library_splits(64, 2048, 6144) == 8 and ops.library_splits(512, 2048, 6144) == 4
+    assert ops.rows_takes(32, 2048, 6144) and not ops.rows_takes(64, 2048, 6144)
+    # o at the 4B sizes (10.5 M elements over a K of 4,096): slices only from 128 rows, the plain call below (64 rows: 17.1
+    # -> 11.5 us), and no skinny split beyond 32 rows over a weight this large
+    assert ops.library_splits(64, 2560, 4096) == 1 and ops.library_splits(128, 2560, 4096) == 8
+    assert ops.rows_takes(32, 2560, 4096) and not ops.rows_takes(48, 2560, 4096)
+    # down at the 4B sizes (2560 features over a K of 9,728): the rows kernel at 33-64 rows, where the library's slices take
+    # 48 us and its plain call 29 (64 rows: -> 21 us); the slices again beyond
+    assert ops.rows_takes(64, 2560, 9728) and ops.library_splits(64, 2560, 9728) == 1 and ops.library_splits(128, 2560, 9728) == 8
+    assert not ops.rows_has_few_features(64, 5120, 17408) and ops.library_splits(64, 5120, 17408) == 8     # 14B: stays with the slices
+    # qkv at the 4B sizes (15.7 M elements): the library from 17 rows (32 rows: 18.8 -> 10.4 us), the skinny kernel's wide loads below
+    assert ops.library_streams_better(32, 6144, 2560) and not ops.library_streams_better(16, 6144, 2560)
+    assert not ops.skinny_takes(32, 6144, 2560) and ops.skinny_takes(16, 6144, 2560)
+    # qkv at the 1.7B sizes (8.4 M elements) at 64 rows: the library's tiles, not the tiled kernel for small weights (12.2 -> 9.8 us);
+    # from 128 rows the two are level and the own kernel stays
+    assert ops.mid_takes(64, 4096, 2048, False) == 0 and ops.mid_takes(128, 4096, 2048, False) == 1
+    assert ops.mid_takes(64, 4096, 1024, False) == 1                     # the 0.6B sizes keep theirs
+    # o at the 1.7B sizes at 33-64 rows: the tiled kernel's four slices of K, not the skinny split (64 rows: 7.9 -> 5.9 us);
+    # beyond 1,024 features only up to 256 rows (512 rows: 13.1 -> 11.7 with the library)
+    assert ops.mid_takes(64, 2048, 2048, True) == 4 and ops.mid_takes(256, 2048, 2048, True) == 4
+    assert ops.mid_takes(512, 2048, 2048, True) == 0 and ops.mid_takes(512, 1024, 2048, True) == 4

@@ -678,6 +678,32 @@ def test_linear_a_few_hundred_rows_over_small_weights(M, N, K):
         close(parts, ref, 6e-3)
 
 
+@pytest.mark.parametrize("M,N,K,route", [(48, 1024, 2048, "mid"), (64, 2048, 2048, "mid"), (64, 2560, 9728, "rows"), (40, 2560, 9728, "rows"),
+                                         (64, 2048, 6144, "slices"), (128, 2560, 4096, "slices"), (64, 2560, 4096, "plain"),
+                                         (32, 2560, 4096, "rows"), (32, 6144, 2560, "plain"), (64, 4096, 2048, "plain")])
+def test_linear_routes_at_the_sizes_between_the_measured_ones(M, N, K, route):
+    """Products of the 1.7B, 4B layer sizes at row counts where the rules were corrected: the route the rules name
+    is the one that runs, and it gives the exact product."""
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+    ref = x.double() @ w.double().t()
+    parts = hip().linear(x, w, None, allow_partials=True)
+    if route == "mid":
+        assert ops.mid_takes(M, N, K, True) == 4 and parts.shape == (4, M, N)
+    elif route == "rows":
+        assert ops.rows_takes(M, N, K) and parts.shape == (ops.rows_ksplit(K), M, N)
+    elif route == "slices":
+        assert parts.shape == (ops.library_splits(M, N, K), M, N) and parts.shape[0] > 1
+    else:
+        assert parts.dim() == 2 and not ops.skinny_takes(M, N, K) and ops.mid_takes(M, N, K, False) == 0
+    if parts.dim() == 3:
+        assert parts.dtype == torch.float32
+        close(parts.sum(0), ref, 2e-5)
+    else:
+        close(parts, ref, 6e-3)
+    close(hip().linear(x, w), ref, 6e-3)
+
+
 @pytest.mark.parametrize("M,N,K", [(200, 384, 80), (2048, 1024, 1024), (65, 100, 200), (70, 96, 44)])
 def test_linear_large_and_odd_bf16(M, N, K):
     """Above the skinny range the library product runs; K not a multiple of 8 takes the FMA kernel."""
@@ -717,7 +743,7 @@ def test_library_product_is_called_directly(M, N, K):
         close(ops.library_product(x, w, torch.float32), x.double() @ w.double().t(), 2e-5)
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 4096, 4096), (128, 4096, 4096), (200, 2560, 9728), (300, 4096, 12288), (700, 5120, 8192), (64, 1368, 12288 + 64)])
+@pytest.mark.parametrize("M,N,K", [(33, 4096, 4096), (128, 4096, 4096), (200, 2560, 9728), (300, 4096, 12288), (700, 5120, 8192), (100, 1368, 12288 + 64)])
 def test_linear_library_slices_of_k(M, N, K):
     """o and down at 33 to 1,024 rows over large weights: the library runs slices of K as one strided batch
     and the consumer adds the float32 partial sums."""
