@@ -609,6 +609,7 @@ _COMPUTE_UNITS = 256
 _DECODE_WORKGROUPS = 4096
 _PREFILL_THREE_WAVES_WORKGROUPS = 2048
 _DECODE_WHOLE_WORKGROUPS = 768
+_DECODE_ONE_ROUND = 768           # workgroups of the decode kernel that run at once: three to a compute unit
 _DECODE_WHOLE_MAX_KEYS = 4096
 _DECODE_EVEN_WHOLE_WORKGROUPS = 192
 _DECODE_EVEN_WHOLE_MAX_KEYS = 8192
@@ -849,17 +850,21 @@ def prefill_waves(max_context: int, num_tokens: int, num_seqs: int, Hq: int, Hkv
 def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: bool = False) -> tuple:
     """(keys per partition, number of partitions) for the split decode kernel.
 
-    A workgroup's 4 waves take 32 keys each per round, so a partition of 128 keys is one round
-    with every load in flight at once; partitions grow beyond that only when (sequences x kv
-    heads x partitions) already gives several workgroups per compute unit, or to keep the
-    number of partitions to merge at 64 or less. A partition holds at most 2,048 keys (as long as 64
-    partitions cover the context): a workgroup goes through its keys round by round, so in a batch with
-    a few long contexts among short ones the long partitions are what is still running at the end.
+    A workgroup's 4 waves take the 32-key blocks of its partition in turn, and three workgroups share a compute
+    unit: 768 run at once. While (sequences x kv heads) stays below that, the partitions are sized so that all
+    workgroups run in one round (8 requests of 2,048 keys: 11 partitions of 192 keys, 704 workgroups; with
+    partitions of 128 keys 1,088 workgroups run in a round and a third, which costs a fifth more), at least 128
+    keys (one block per wave) and at most 512 (beyond, more and shorter workgroups stream better even in several
+    rounds), never more than 64 partitions to merge, and at most 2,048 keys as long as 64 partitions cover the
+    context: a workgroup goes through its keys round by round, so in a batch with a few long contexts among short
+    ones the long partitions are what is still running at the end.
     From 768 workgroups on (96 sequences x 8 kv heads) a context up to 2,048 keys (4,096 from 2,048 workgroups
     on) is one partition and needs no reduce kernel. `even` (the contexts are equally long,
-    `decode_contexts_even`): from 192 workgroups on (24 sequences x 8 kv heads) a context up to 8,192 keys is one
-    partition: every workgroup then has the same work, none waits for another's partial results and no reduce
-    kernel follows; contexts of different lengths gain nothing from it and long ones among short ones lose.
+    `decode_contexts_even`): from 192 workgroups on, a context up to 8,192 keys is one partition if the workgroups
+    then fill the compute units evenly (a multiple of 256: 32 or 64 requests x 8 kv heads; 24 or 48 requests leave
+    compute units idle or doubly loaded and run 12-14 % faster in partitions): every workgroup then has the same
+    work, none waits for another's partial results and no reduce kernel follows; contexts of different lengths
+    gain nothing from it and long ones among short ones lose.
     (The reference's rule: layers/ops.py:44-51, split when sequences x kv heads cannot fill the SMs, 256-key
     partitions.)"""
     col_tiles = (Hq // Hkv + 15) // 16
@@ -867,8 +872,14 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
     ctx = max(1, max_context)
     if base >= _DECODE_WHOLE_WORKGROUPS and ctx <= (_DECODE_WHOLE_MAX_KEYS if base >= 2048 else _DECODE_WHOLE_MAX_KEYS // 2):
         return -(-ctx // 128) * 128, 1
-    if even and base >= _DECODE_EVEN_WHOLE_WORKGROUPS and ctx <= _DECODE_EVEN_WHOLE_MAX_KEYS:
+    if even and base >= _DECODE_EVEN_WHOLE_WORKGROUPS and base % _COMPUTE_UNITS == 0 and ctx <= _DECODE_EVEN_WHOLE_MAX_KEYS:
         return -(-ctx // 128) * 128, 1
+    if base <= _DECODE_ONE_ROUND:
+        # one round of workgroups where the batch allows it
+        per = -(-ctx // max(1, _DECODE_ONE_ROUND // base))
+        part = min(512, max(128, -(-per // 64) * 64))
+        part = max(part, -(-(-(-ctx // 64)) // 128) * 128)          # 64 partitions at most
+        return part, max(1, -(-ctx // part))
     want = max(1, -(-_DECODE_WORKGROUPS // base), -(-ctx // _DECODE_MAX_PARTITION))
     want = min(64, want)
     part = max(128, -(-(-(-ctx // want)) // 128) * 128)

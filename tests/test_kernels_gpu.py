@@ -300,8 +300,9 @@ def test_decode_step_in_one_launch(Hq, Hkv, D, page, window):
 
 @pytest.mark.parametrize("Hq,Hkv,D,page", [(16, 8, 128, 16), (6, 2, 32, 8), (64, 8, 128, 16)])
 def test_attention_decode_equal_contexts_in_one_partition(Hq, Hkv, D, page):
-    """Equally long contexts with 192 workgroups or more: one partition each, no reduce kernel."""
-    n = -(-192 // Hkv)
+    """Equally long contexts whose workgroups fill the compute units evenly (256 of them): one partition each, no
+    reduce kernel."""
+    n = -(-256 // Hkv)
     seqs = [(1500 + i % 20, 1) for i in range(n)]
     assert ops.decode_partitions(n, Hq, Hkv, 1519, True)[1] == 1 and ops.decode_partitions(n, Hq, Hkv, 1519, False)[1] > 1
     args = _attention_case(torch.bfloat16, Hq, Hkv, D, page, seqs, seed=3, peak=700)
@@ -462,7 +463,7 @@ def test_decode_partitions_rule():
     for S, Hq, Hkv, ctx in ((1, 16, 8, 2048), (8, 16, 8, 2048), (64, 16, 8, 2304), (1, 32, 8, 100), (3, 6, 2, 130000),
                             (256, 16, 8, 4096), (256, 16, 8, 4097), (128, 16, 8, 16384)):
         part, parts = ops.decode_partitions(S, Hq, Hkv, ctx)
-        assert part % 128 == 0 and part * parts >= ctx and part * (parts - 1) < ctx
+        assert part % 64 == 0 and part >= 128 and part * parts >= ctx and part * (parts - 1) < ctx
 
 
 # ------------------------------------------------------------------------------- products
