@@ -44,6 +44,27 @@ extern "C" int me_gather_rows(const void* src, const int32_t* idx, void* out, in
   return 0;
 }
 
+// ------------------------------------------------------------------ tokens handed over on the device
+// tokens[r] = sampled[take[r]] for the rows whose take[r] >= 0; the other rows keep what they hold. A decode step
+// that is launched before the step in flight has delivered its tokens takes them so from the sampling kernel's
+// output (the reference fetches every token to the host first: engine/llm_engine.py:43-52).
+__global__ void take_tokens_kernel(int32_t* __restrict__ tokens, const int32_t* __restrict__ sampled,
+                                   const int32_t* __restrict__ take, int rows, int num_sampled) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  const int t = take[r];
+  if (t >= 0 && t < num_sampled) tokens[r] = sampled[t];
+}
+
+extern "C" int me_take_tokens(int32_t* tokens, const int32_t* sampled, const int32_t* take, int rows, int num_sampled,
+                              hipStream_t stream) {
+  if (rows <= 0) return 0;
+  ME_CHECK(tokens && sampled && take && num_sampled > 0, "take_tokens: missing operand");
+  take_tokens_kernel<<<dim3((rows + 255) / 256), dim3(256), 0, stream>>>(tokens, sampled, take, rows, num_sampled);
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------------------------------------ RMSNorm (+ residual)
 // r = x (+ res_in)           summed in float32, kept in float32 as the new residual
 // y = w * r * rsqrt(mean(r^2) + eps)

@@ -208,15 +208,9 @@ class DecodeGraphs:
 
     def _take_pending(self, cap: _Captured, take, B: int) -> None:
         """Copy the tokens that the last sampling call left on the device into the step's token rows
-        (after the upload, before the replay, on the same stream). `take` went up with the metadata."""
-        out = self.runner.last_sampled.out
-        tokens = cap.view("tokens")
-        if out.numel() == B and np.array_equal(take[:B], np.arange(B)):
-            tokens[:B].copy_(out)
-            return
-        t = cap.view("take")[:B].long()
-        picked = out.index_select(0, t.clamp(min=0)).to(tokens.dtype)
-        tokens[:B].copy_(torch.where(t >= 0, picked, tokens[:B]))
+        (after the upload, before the replay, on the same stream): one small kernel, rows whose `take` is
+        negative keep the token that went up with the metadata. `take` went up with the metadata too."""
+        ops.take_tokens(cap.view("tokens")[:B], self.runner.last_sampled.out, cap.view("take")[:B])
 
     def _continues(self, cap: _Captured, reqs: list, pos, B: int) -> bool:
         """Whether this step is the one before with every request one position on: the same

@@ -32,7 +32,7 @@ CORE_SOURCES = ["elementwise.hip", "rope_kv.hip", "attention_simple.hip",
                 "gemm.hip", "gemm_mid.hip", "gemm_library.hip", "sampling.hip"]
 ATTN_SOURCE = "attention_mfma.hip"
 HEADERS = ["common.h", "errors.inc", "sampling.h"]
-# Head sizes built by build_all(): the sizes of the benchmark models and of the test configurations.
+# Head sizes that build_all() compiles ahead of use; any other multiple of 16 up to 512 is compiled when a model first needs it.
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 128)
 
 _locks: dict = {}

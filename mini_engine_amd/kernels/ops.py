@@ -56,6 +56,7 @@ class _Lib:
 P, I, L, F = c_void_p, c_int, c_int64, c_float
 _CORE_PROTOS = {
     "me_gather_rows": [P, P, P, L, L, L, P],
+    "me_take_tokens": [P, P, P, I, I, P],
     "me_rms_norm": [P, I, I, L, P, P, P, P, I, L, I, F, P],
     "me_silu_and_mul": [P, P, I, L, I, P],
     "me_qk_norm_rope_store": [P, I, L, L, P, P, F, P, L, L, P, P, P, P, I, I, I, I, I, P],
@@ -211,6 +212,13 @@ class HipBackend:
         core().call("me_gather_rows", src.data_ptr(), idx.data_ptr(), out.data_ptr(), idx.numel(),
                     src.shape[1] * src.element_size(), src.shape[0], _stream())
         return out
+
+    def take_tokens(self, tokens: torch.Tensor, sampled: torch.Tensor, take: torch.Tensor) -> None:
+        """tokens[r] = sampled[take[r]] where take[r] >= 0, in place (int32 [R], [S], [R]): the tokens of the last
+        sampling call go into the rows of a step launched before they have reached the host."""
+        R = tokens.numel()
+        _check(_is_i32(tokens) and _is_i32(sampled) and _is_i32(take, R), "take_tokens: int32 tensors, one source row per token row")
+        core().call("me_take_tokens", tokens.data_ptr(), sampled.data_ptr(), take.data_ptr(), R, sampled.numel(), _stream())
 
     # -- norm ----------------------------------------------------------------------------
     def rms_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None,
@@ -972,6 +980,7 @@ def set_backend(b) -> None:
 
 
 def gather_rows(*a, **k): return backend().gather_rows(*a, **k)
+def take_tokens(*a, **k): return backend().take_tokens(*a, **k)
 def rms_norm(*a, **k): return backend().rms_norm(*a, **k)
 def silu_and_mul(*a, **k): return backend().silu_and_mul(*a, **k)
 def qk_norm_rope_store(*a, **k): return backend().qk_norm_rope_store(*a, **k)

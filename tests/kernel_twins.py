@@ -17,6 +17,11 @@ def gather_rows(src, idx):
     return src[idx.long()].clone()
 
 
+def take_tokens(tokens, sampled, take):
+    chosen = take.long() >= 0
+    tokens[chosen] = sampled[take.long()[chosen]].to(tokens.dtype)
+
+
 def rms_norm(x, weight, eps, residual, out_dtype, want_residual=True):
     r = x.float().sum(0) if x.dim() == 3 else x.float()
     if residual is not None:
@@ -83,11 +88,11 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
     T = q.shape[0]
     out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
     G = Hq // Hkv
+    seqs, where, lens = seq_of_token[:T].tolist(), positions[:T].tolist(), context_lens.tolist()      # one trip to the host
     for t in range(T):
-        b = int(seq_of_token[t])
-        pos = int(positions[t])
+        b, pos = seqs[t], where[t]
         lo = max(0, pos - window + 1) if window else 0
-        hi = min(pos + 1, int(context_lens[b]))            # a padding row (context 0) sees nothing
+        hi = min(pos + 1, lens[b])                         # a padding row (context 0) sees nothing
         if hi <= lo:
             out[t] = 0
             continue
@@ -97,12 +102,10 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
         offs = js % page
         k = k_cache[pages, :, offs, :].to(compute_dtype)             # [n, Hkv, D]
         v = v_cache[pages, :, :, offs].to(compute_dtype)             # [n, Hkv, D]
-        qt = q[t].to(compute_dtype).view(Hq, D)
-        for h in range(Hq):
-            kh = h // G
-            s = (k[:, kh, :] @ qt[h]) * scale
-            p = torch.softmax(s, dim=0)
-            out[t, h * D:(h + 1) * D] = (p @ v[:, kh, :]).to(q.dtype)
+        qt = q[t].to(compute_dtype).view(Hkv, G, D)                  # query head h belongs to key head h // G
+        s = torch.einsum("nkd,kgd->kgn", k, qt) * scale
+        p = torch.softmax(s, dim=-1)
+        out[t] = torch.einsum("kgn,nkd->kgd", p, v).reshape(Hq * D).to(q.dtype)
     return out
 
 
@@ -213,6 +216,7 @@ def sample(logits, temperatures, keys):
 class PlainBackend:
     name = "plain"
     gather_rows = staticmethod(gather_rows)
+    take_tokens = staticmethod(take_tokens)
     rms_norm = staticmethod(rms_norm)
     silu_and_mul = staticmethod(silu_and_mul)
     qk_norm_rope_store = staticmethod(qk_norm_rope_store)

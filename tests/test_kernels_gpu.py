@@ -32,6 +32,19 @@ def test_gather_rows(dtype, rows, width):
     assert torch.equal(hip().gather_rows(src, idx), twin.gather_rows(src, idx))
 
 
+def test_take_tokens():
+    """Rows that name a row of the sampling call's output take its token; rows that name none (-1) keep theirs."""
+    sampled = torch.randint(0, 1000, (37,), device=DEV, dtype=torch.int32)
+    for rows in (1, 8, 300):
+        tokens = torch.randint(1000, 2000, (rows,), device=DEV, dtype=torch.int32)
+        take = torch.randint(-1, 37, (rows,), device=DEV, dtype=torch.int32)
+        want = tokens.clone()
+        twin.take_tokens(want, sampled, take)
+        hip().take_tokens(tokens, sampled, take)
+        assert torch.equal(tokens, want)
+        assert torch.equal(tokens[take < 0], want[take < 0]) and (want[take >= 0] < 1000).all()
+
+
 @pytest.mark.parametrize("T,n", [(1, 80), (13, 1000), (64, 4096), (3, 5120), (300, 1024), (257, 72), (1000, 1028),
                                  (300, 520), (257, 4104), (256, 5120), (260, 5128)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
