@@ -65,15 +65,19 @@ def _used_per_call(model) -> dict:
 def _matrix_params(model) -> tuple:
     """(matrix elements multiplied per token in the layers, counting a layer once per run; elements of the head's matrix)."""
     runs = _used_per_call(model)
-    per_token = 0
+    tied = getattr(model.head, "tied_to", None) is model.embedding
+    per_token = head = 0
     for name, _, _, spec in model.named_specs():
-        if name.startswith("layers.") and len(spec.shape) >= 2:
-            n = 1
-            for d in spec.shape:
-                n *= int(d)
+        if len(spec.shape) < 2:
+            continue
+        n = 1
+        for d in spec.shape:
+            n *= int(d)
+        if name.startswith("layers."):
             per_token += n * runs.get(int(name.split(".")[1]), 0)
-    head = model.head.matrix() if hasattr(model.head, "matrix") else None
-    return per_token, (head.numel() if head is not None else 0)
+        elif name.startswith("head.") or (tied and name.startswith("embedding.")):
+            head += n
+    return per_token, head
 
 
 def cache_bytes_per_token(model, page: int, dtype) -> list:
