@@ -198,30 +198,38 @@ def padded_layouts_are_used(env, name, captured: bool):
 
 
 def exactly_sized_layouts_are_used(env, name, captured: bool):
-    """Steps beyond the size that is padded keep their own token and request counts in a fixed layout (only the
-    context cap and the rows of logits are rounded): a repeating pattern, portions of 40 tokens beside one decoding
-    request, goes through one layout again and again while the contexts grow; logits as ever. `env.runner` must have
-    made the runner with a small `mixed_graphs_max_tokens` (16) and `mixed_graphs_after=0`."""
-    runner, manager, folder = env.runner(name, 60)
+    """Steps beyond the size that is padded, in which nobody decodes, keep their own token and request counts in a
+    fixed layout (only the context cap and the rows of logits are rounded): a repeating pattern, portions of 40
+    tokens of one prompt beside 24 of another, goes through one layout again and again while the contexts grow;
+    logits as ever. `env.runner` must have made the runner with a small `mixed_graphs_max_tokens` (16) and
+    `mixed_graphs_after=0`."""
+    runner, manager, folder = env.runner(name, 90)
     mg = runner.mixed_graphs
     assert mg is not None and mg.capture_after == 0 and mg.max_tokens == 16 and mg.max_exact_tokens == 96
     V = _vocab(name)
-    a, b, c = helpers.random_ids(60, V, 811), helpers.random_ids(200, V, 812), helpers.random_ids(130, V, 813)
+    a, b, c = helpers.random_ids(130, V, 811), helpers.random_ids(201, V, 812), helpers.random_ids(130, V, 813)
     d = helpers.Driver(runner, manager)
-    d.step({"a": a[:50]})                                        # 50 tokens: its own layout
+    d.step({"c": c[:50]})                                        # 50 tokens: its own layout
     layouts = [set(mg.captured)]
-    for i in range(5):                                           # 1 + 40 tokens, five times: one layout
-        d.step({"a": a[50 + i:51 + i], "b": b[40 * i:40 * i + 40]})
+    for i in range(5):                                           # 24 + 40 tokens, five times: one layout
+        d.step({"a": a[24 * i:24 * i + 24], "b": b[40 * i:40 * i + 40]})
         layouts.append(set(mg.captured))
     assert len(layouts[1]) == 2 and all(l == layouts[1] for l in layouts[2:]), "the repeating step did not keep its layout"
     one = next(iter(layouts[1] - layouts[0]))
-    assert (one.decode_rows, one.prefill_reqs, one.prefill_tokens) == (1, 1, 40)      # nothing was padded
-    d.step({"c": c[:100]})                                       # 100 tokens: beyond what is replayed at all
+    assert (one.decode_rows, one.prefill_reqs, one.prefill_tokens) == (0, 2, 64)      # nothing was padded
     assert mg.replays == 6
-    d.step({"c": c[100:], "a": a[55:]})                          # 30 + 5 tokens: two portions, its own layout
-    assert mg.replays == 7 and len(mg.captured) == 3
+    d.step({"c": c[50:51], "a": a[120:]})                        # somebody decodes beside 10 tokens: a padded layout
+    d.step({"c": c[51:]})                                        # 79 tokens, nobody decodes: its own layout again
+    assert mg.replays == 8 and len(mg.captured) == 4
+    assert sorted(l.prefill_tokens for l in mg.captured if l.decode_rows == 0) == [50, 64, 79]
+    # so many tokens with a decoding request among them get no layout of their own: the step runs as it is
+    e = helpers.random_ids(41, V, 814)
+    d.step({"b": b[200:], "e": e[:40]})
+    assert mg.replays == 8 and len(mg.captured) == 4
+    d.step({"e": e[40:]})
     if captured:
         assert all(cap.graph is not None for cap in mg.captured.values())
     _check(env, folder, a, d.result("a"), "a through exactly sized layouts")
     _check(env, folder, b, d.result("b"), "b through exactly sized layouts")
     _check(env, folder, c, d.result("c"), "c through exactly sized layouts")
+    _check(env, folder, e, d.result("e"), "e beside a decoding request")
