@@ -73,8 +73,8 @@ _CORE_PROTOS = {
 }
 _ATTN_PROTOS = {
     "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, I, P, P, I, P],
-    "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, I, P],
-    "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, I, P],
+    "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, P, I, P],
+    "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, P, I, P],
 }
 
 _core: _Lib | None = None
@@ -351,6 +351,7 @@ class HipBackend:
             lib.call("me_attn_decode", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
                      num_decodes, Hq, Hkv, page, float(scale), win, part_size, num_parts, _ptr(scratch),
+                     _ptr(_part_counters(num_decodes * Hkv * -(-(Hq // Hkv) // 16), q.device) if num_parts > 1 else None),
                      0 if even_contexts else 1, _stream())
         if T > num_decodes:
             _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
@@ -405,7 +406,9 @@ class HipBackend:
                          _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0],
                          k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
                          context_lens.data_ptr(), int(max_context), B, Hq, Hkv, page, float(scale), int(window or 0),
-                         part_size, num_parts, _ptr(scratch), 0 if even_contexts else 1, _stream())
+                         part_size, num_parts, _ptr(scratch),
+                         _ptr(_part_counters(B * Hkv * -(-(Hq // Hkv) // 16), qkv.device) if num_parts > 1 else None),
+                         0 if even_contexts else 1, _stream())
         return out
 
     # -- matrix products -----------------------------------------------------------------
@@ -638,6 +641,24 @@ def _scratch(num_floats: int, device, use: str = "decode") -> torch.Tensor:
             _scratch_retired.append(buf)
         buf = torch.empty((max(num_floats + num_floats // 2, 1 << 20),), dtype=torch.float32, device=device)
         _scratch_buf[key] = buf
+    return buf
+
+
+PART_COUNTERS = 1 << 16
+MERGE_PARTITIONS_IN_KERNEL = True
+_part_counter_buf: dict = {}
+
+
+def _part_counters(count: int, device) -> torch.Tensor | None:
+    """Zeroed int32 counters, one per (request, block of heads), with which the decode kernel's workgroups find out
+    which of a context's partitions finishes last (that one merges them); the kernel leaves them zero. One array
+    per device, made once; a launch that would need more gets None and merges in a launch of its own. Launches
+    on different streams of one device would share them: the engine runs on one stream."""
+    if not MERGE_PARTITIONS_IN_KERNEL or count > PART_COUNTERS:
+        return None
+    buf = _part_counter_buf.get(device)
+    if buf is None:
+        buf = _part_counter_buf[device] = torch.zeros((PART_COUNTERS,), dtype=torch.int32, device=device)
     return buf
 
 
