@@ -1304,7 +1304,11 @@ __device__ __forceinline__ void decode_part_range(const AttnArgs& a, int L, int&
 #define ME_DECODE_STREAMS 1
 #endif
 constexpr bool DECODE_STREAMS = ME_DECODE_STREAMS != 0;
-template <bool PROLOGUE>
+// AHEAD (for partitions of at most 256 keys, i.e. one or two blocks to a wave): the keys of a wave's two blocks are
+// both asked for before the first is worked on, so the second block's keys do not wait for the first block's work.
+// (The values of both ahead as well need 197 registers, which leaves two workgroups to a compute unit instead of
+// three.)
+template <bool PROLOGUE, bool AHEAD = false>
 __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
   extern __shared__ float lds[];  // [4 waves][cols][HD + 2]; PROLOGUE: then bfloat16 [cols + 2][HD]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1393,7 +1397,20 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
   // and it is their interleaving that hides the load latency here (partitions are short).
   int t0 = p_lo + 32 * wave;
   const bool has_keys = t0 < p_hi;
-  KVBlock A;
+  const bool has_second = AHEAD && t0 + 128 < p_hi;
+  KVBlock A, A2;
+  // the first block of keys (AHEAD: and the second; both table reads go out before the keys they address)
+  auto first_keys = [&]() {
+    if constexpr (AHEAD) {
+      BlockPages pg, pg2;
+      lookup_pages(a, bt, t0, L, lo, n, g, pg);
+      if (has_second) lookup_pages(a, bt, t0 + 128, L, lo, n, g, pg2);
+      load_kv<DECODE_STREAMS>(a, pg, kvh, t0, L, n, g, A);
+      if (has_second) load_kv<DECODE_STREAMS>(a, pg2, kvh, t0 + 128, L, n, g, A2);
+    } else {
+      load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
+    }
+  };
   if (PROLOGUE) {
     // the wave's first head is asked for before the first block of keys, and worked on while those are on
     // their way; the heads after it (more than three query heads to a key head) one by one
@@ -1402,7 +1419,7 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     bf16_t new_v = static_cast<bf16_t>(0.f);
     const int vd = threadIdx.x < HD ? threadIdx.x : 0;
     if (holds_new) new_v = a.raw_v[t * a.q_stride + (int64_t)kvh * HD + vd];
-    if (has_keys) load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
+    if (has_keys) first_keys();
     if (wave < nheads) finish_head(wave, first);
     for (int h = wave + 4; h < nheads; h += 4) {
       RawHead r;
@@ -1420,16 +1437,15 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     }
     __syncthreads();
   } else if (has_keys) {
-    load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
+    first_keys();
   }
   if (has_keys) {
     bf16x8 qb[KS];
     if (PROLOGUE) load_q(q_s + (valid ? n : 0) * HD, valid, g, qb);
     else load_q(a.q + t * a.q_stride + (int64_t)head * HD, valid, g, qb);
     const int col_hi = valid ? pos : -1;
-    while (true) {
-      VBlock vb;
-      load_v<DECODE_STREAMS>(a, A, kvh, t0, L, n, g, vb);
+    // one block: what the new token brings comes from LDS, then scores, softmax and the weighted sum
+    auto work_on = [&](KVBlock& A, VBlock& vb, int t0) {
       if (holds_new && pos >= t0 && pos < t0 + 32) {
         // the block with the new token: its key row and its value column come from LDS
         const int rel = pos - t0;
@@ -1455,9 +1471,24 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
       }
       if (t0 + 32 <= L && t0 >= lo) attend_block<true>(a, A, vb, t0, qb, lo, col_hi, m, l, acc, g);
       else attend_block<false>(a, A, vb, t0, qb, lo, col_hi, m, l, acc, g);
+    };
+    if constexpr (AHEAD) {
+      VBlock vb;
+      load_v<DECODE_STREAMS>(a, A, kvh, t0, L, n, g, vb);
+      work_on(A, vb, t0);
+      if (has_second) {
+        load_v<DECODE_STREAMS>(a, A2, kvh, t0 + 128, L, n, g, vb);
+        work_on(A2, vb, t0 + 128);
+      }
+      t0 += 256;
+    }
+    while (t0 < p_hi) {           // AHEAD: only partitions of more than 256 keys get here
+      if (AHEAD) load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
+      VBlock vb;
+      load_v<DECODE_STREAMS>(a, A, kvh, t0, L, n, g, vb);
+      work_on(A, vb, t0);
       t0 += 128;
-      if (t0 >= p_hi) break;
-      load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
+      if (!AHEAD && t0 < p_hi) load_block<DECODE_STREAMS>(a, bt, kvh, t0, L, lo, n, g, A);
     }
   }
   l = column_sum(l);
@@ -1715,14 +1746,20 @@ static int launch_decode(AttnArgs& a, int num_seqs, int part_size, int num_parts
   const size_t lds = (size_t)4 * cmax * (HD + 2) * sizeof(float) + (prologue ? (size_t)(cmax + 2) * HD * sizeof(bf16_t) : 0);
   static size_t lds_allowed[2] = {64 * 1024, 64 * 1024};
   if (lds > lds_allowed[prologue]) {
-    hipError_t e = hipFuncSetAttribute(prologue ? (const void*)attn_decode_kernel<true> : (const void*)attn_decode_kernel<false>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    ME_CHECK(e == hipSuccess, "attention: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    for (const void* kernel : {prologue ? (const void*)attn_decode_kernel<true, false> : (const void*)attn_decode_kernel<false, false>,
+                               prologue ? (const void*)attn_decode_kernel<true, true> : (const void*)attn_decode_kernel<false, true>}) {
+      hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      ME_CHECK(e == hipSuccess, "attention: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    }
     lds_allowed[prologue] = lds;
   }
   const dim3 grid = a.spread_heads ? dim3(a.Hkv * col_tiles, num_seqs, num_parts) : dim3(num_seqs, a.Hkv * col_tiles, num_parts);
-  if (prologue) attn_decode_kernel<true><<<grid, dim3(256), lds, stream>>>(a);
-  else attn_decode_kernel<false><<<grid, dim3(256), lds, stream>>>(a);
+  // partitions of 129-256 keys: a wave has up to two blocks and asks for the keys of both at once
+  const bool ahead = num_parts > 1 && part_size > 128 && part_size <= 256;
+  if (prologue && ahead) attn_decode_kernel<true, true><<<grid, dim3(256), lds, stream>>>(a);
+  else if (prologue) attn_decode_kernel<true, false><<<grid, dim3(256), lds, stream>>>(a);
+  else if (ahead) attn_decode_kernel<false, true><<<grid, dim3(256), lds, stream>>>(a);
+  else attn_decode_kernel<false, false><<<grid, dim3(256), lds, stream>>>(a);
   ME_LAUNCH_CHECK();
   if (num_parts > 1 && a.part_counters == nullptr) {
     attn_reduce_kernel<<<dim3(num_seqs, a.Hq), dim3(128), 0, stream>>>(a);
