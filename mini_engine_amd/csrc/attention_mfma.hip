@@ -24,6 +24,7 @@
 // or beyond the context length are zeroed before the product, so a cache full of NaN outside
 // the owned range cannot leak.
 #include "common.h"
+#include <cstdlib>
 
 #ifndef ME_HEAD_DIM
 #error "compile with -DME_HEAD_DIM=<multiple of 16>"
@@ -64,8 +65,6 @@ struct AttnArgs {
   float* tmp_out;               // [num_seqs, Hq, num_parts, HD] unnormalised
   float* tmp_m;                 // [num_seqs, Hq, num_parts]
   float* tmp_l;
-  int32_t* part_counters;       // decode: [num_seqs, Hkv * column tiles], zero between launches, or nullptr (then
-                                // attn_reduce_kernel merges the partitions in a launch of its own)
   // prefill: a tile whose keys span more than seg_keys is cut into segments handled by different
   // workgroups (grid z); their partial results go to pf_scratch and are merged by a second kernel
   int seg_keys;                 // 0: no cutting; else a multiple of 32
@@ -1299,7 +1298,6 @@ __device__ __forceinline__ void decode_part_range(const AttnArgs& a, int L, int&
 // workgroups whose partition holds position L - 1 do the same for the new key and copy the new value: they
 // attend to both from LDS, in place of what the page holds there, and the first column tile's workgroup writes
 // them into the page. No workgroup reads what another one writes.
-#define RED_MAX_PARTS 64     // most partitions of a context
 #ifndef ME_DECODE_STREAMS
 #define ME_DECODE_STREAMS 1
 #endif
@@ -1521,68 +1519,15 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
       a.out[t * a.out_stride + (int64_t)hq * HD + d] = static_cast<bf16_t>(ls > 0.f ? o / ls : 0.f);
     } else {
       const int64_t row = ((int64_t)b * a.Hq + hq) * a.num_parts + part;
-      // written through to where every compute unit of the device reads it: the workgroup that merges the
-      // partitions may sit on another XCD, whose L2 does not see what this XCD's L2 still holds
-      __hip_atomic_store(a.tmp_out + row * HD + d, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (d == 0) {
-        __hip_atomic_store(a.tmp_m + row, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(a.tmp_l + row, ls, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      a.tmp_out[row * HD + d] = o;
+      if (d == 0) { a.tmp_m[row] = M; a.tmp_l[row] = ls; }
     }
-  }
-  if (a.num_parts == 1 || a.part_counters == nullptr) return;
-
-  // ---- the partitions of these heads are merged by whichever of their workgroups finishes last: each waits until
-  // its partial results (written through, above) have arrived, then takes a ticket; the one that draws the last
-  // ticket reads all the others' results past the caches, sets the counter back to zero for the next launch, and
-  // does what attn_reduce_kernel does, in the same order of sums. No workgroup waits for another. (A fence of
-  // device scope in place of the written-through stores writes back and drops the XCD's whole L2 per wave: with
-  // 704 workgroups finishing together that took 85 us a launch.)
-  __shared__ int is_last;
-  int part0, part_end;
-  decode_part_range(a, L, part0, part_end);
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __builtin_amdgcn_s_waitcnt(0);          // every counter at zero: the stores above have been acknowledged
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int32_t* counter = a.part_counters + (int64_t)b * (a.Hkv * col_tiles) + head_block;
-    const int ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    is_last = ticket == part_end - part0 - 1;
-    if (is_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
-  if (!is_last) return;
-  const int P = part_end - part0;
-  float* wgt = lds;                       // [ncols][RED_MAX_PARTS] weights of the partitions
-  float* inv_sum = lds + ncols * RED_MAX_PARTS;      // [ncols]
-  for (int c = wave; c < ncols; c += 4) {
-    const int64_t row0 = ((int64_t)b * a.Hq + kvh * a.G + ctile * 16 + c) * a.num_parts + part0;
-    const int pl = lane < P ? lane : 0;
-    const float mr = __hip_atomic_load(a.tmp_m + row0 + pl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const float lr = __hip_atomic_load(a.tmp_l + row0 + pl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const float mp = lane < P ? mr : NEG, lp = lane < P ? lr : 0.f;
-    const float M = wave_max(mp);
-    const float f = lane < P ? exp2f(mp - M) : 0.f;
-    const float ls = wave_sum(f * lp);
-    wgt[c * RED_MAX_PARTS + lane] = f;
-    if (lane == 0) inv_sum[c] = ls > 0.f ? 1.f / ls : 0.f;
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < ncols * HD; e += 256) {
-    const int c = e / HD, d = e - c * HD;
-    const int hq = kvh * a.G + ctile * 16 + c;
-    const int64_t row0 = ((int64_t)b * a.Hq + hq) * a.num_parts + part0;
-    float o = 0.f;
-#pragma unroll 8
-    for (int p = 0; p < P; ++p)
-      o += wgt[c * RED_MAX_PARTS + p] * __hip_atomic_load(a.tmp_out + (row0 + p) * HD + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    a.out[t * a.out_stride + (int64_t)hq * HD + d] = static_cast<bf16_t>(o * inv_sum[c]);
   }
 }
 
-// Reduce over partitions in a launch of its own (for callers without counters): out = sum_p e^{m_p - M} o_p /
-// sum_p e^{m_p - M} l_p. Grid (num_seqs, Hq);
+// Reduce over partitions: out = sum_p e^{m_p - M} o_p / sum_p e^{m_p - M} l_p. Grid (num_seqs, Hq);
 // the weights of the partitions are formed once, in LDS, then every thread sums its channel.
+#define RED_MAX_PARTS 64
 __global__ void __launch_bounds__(128) attn_reduce_kernel(AttnArgs a) {
   __shared__ float wgt[RED_MAX_PARTS];
   __shared__ float inv_s;
@@ -1721,10 +1666,8 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
 }
 
 // Scratch of the split decode path: num_seqs * Hq * num_parts * (HD + 2) floats (out, m, l per partition).
-// counters: num_seqs * Hkv * ceil(G / 16) int32, all zero (the kernel leaves them so), for the merge of the partitions
-// inside the decode kernel; nullptr: the merge is a launch of its own. Launches that share counters must not overlap.
-static int launch_decode(AttnArgs& a, int num_seqs, int part_size, int num_parts, float* scratch, int32_t* counters,
-                         int spread_heads, bool prologue, hipStream_t stream) {
+static int launch_decode(AttnArgs& a, int num_seqs, int part_size, int num_parts, float* scratch, int spread_heads,
+                         bool prologue, hipStream_t stream) {
   ME_CHECK(num_parts >= 1 && num_parts <= RED_MAX_PARTS, "attention: %d partitions outside 1..%d", num_parts, RED_MAX_PARTS);
   ME_CHECK(num_parts == 1 || (part_size >= 32 && part_size % 32 == 0),
            "attention: partition size %d must be a multiple of 32", part_size);
@@ -1736,13 +1679,10 @@ static int launch_decode(AttnArgs& a, int num_seqs, int part_size, int num_parts
     const int64_t rows = (int64_t)num_seqs * a.Hq * num_parts;
     a.tmp_out = scratch; a.tmp_m = scratch + rows * HD; a.tmp_l = a.tmp_m + rows;
   }
-  a.part_counters = num_parts > 1 ? counters : nullptr;
   const int col_tiles = (a.G + 15) / 16;
   ME_CHECK((int64_t)a.Hkv * col_tiles <= 65535 && num_seqs <= 65535,
            "attention: %d sequences or %d head blocks exceed one launch", num_seqs, a.Hkv * col_tiles);
   const int cmax = a.G < 16 ? a.G : 16;
-  // 4 * cmax * (HD + 2) floats hold the waves' results, and later the cmax * (RED_MAX_PARTS + 1) weights of the merge
-  static_assert(4 * (HD + 2) >= RED_MAX_PARTS + 1, "the merge's weights must fit where the waves' results lay");
   const size_t lds = (size_t)4 * cmax * (HD + 2) * sizeof(float) + (prologue ? (size_t)(cmax + 2) * HD * sizeof(bf16_t) : 0);
   static size_t lds_allowed[2] = {64 * 1024, 64 * 1024};
   if (lds > lds_allowed[prologue]) {
@@ -1755,13 +1695,14 @@ static int launch_decode(AttnArgs& a, int num_seqs, int part_size, int num_parts
   }
   const dim3 grid = a.spread_heads ? dim3(a.Hkv * col_tiles, num_seqs, num_parts) : dim3(num_seqs, a.Hkv * col_tiles, num_parts);
   // partitions of 129-256 keys: a wave has up to two blocks and asks for the keys of both at once
-  const bool ahead = num_parts > 1 && part_size > 128 && part_size <= 256;
+  static const bool ahead_allowed = []() { const char* v = getenv("ME_DECODE_KEYS_AHEAD"); return v == nullptr || v[0] != '0'; }();
+  const bool ahead = ahead_allowed && num_parts > 1 && part_size > 128 && part_size <= 256;
   if (prologue && ahead) attn_decode_kernel<true, true><<<grid, dim3(256), lds, stream>>>(a);
   else if (prologue) attn_decode_kernel<true, false><<<grid, dim3(256), lds, stream>>>(a);
   else if (ahead) attn_decode_kernel<false, true><<<grid, dim3(256), lds, stream>>>(a);
   else attn_decode_kernel<false, false><<<grid, dim3(256), lds, stream>>>(a);
   ME_LAUNCH_CHECK();
-  if (num_parts > 1 && a.part_counters == nullptr) {
+  if (num_parts > 1) {
     attn_reduce_kernel<<<dim3(num_seqs, a.Hq), dim3(128), 0, stream>>>(a);
     ME_LAUNCH_CHECK();
   }
@@ -1772,12 +1713,12 @@ extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_
                               const void* k_cache, const void* v_cache, const int32_t* block_tables,
                               int bt_stride, const int32_t* context_lens, int num_seqs, int Hq, int Hkv,
                               int page, float scale, int window, int part_size, int num_parts,
-                              float* scratch, int32_t* counters, int spread_heads, hipStream_t stream) {
+                              float* scratch, int spread_heads, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   AttnArgs a;
   if (fill_common(a, q, q_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
                   num_seqs, Hq, Hkv, page, scale, window)) return -1;
-  return launch_decode(a, num_seqs, part_size, num_parts, scratch, counters, spread_heads, false, stream);
+  return launch_decode(a, num_seqs, part_size, num_parts, scratch, spread_heads, false, stream);
 }
 
 // A whole decode step's attention from the packed projection rows [num_seqs, (Hq + 2 Hkv) * HD] (row r belongs
@@ -1791,7 +1732,7 @@ extern "C" int me_attn_decode_fused(const void* qkv, int64_t row_stride, void* o
                                     void* k_cache, void* v_cache, const int32_t* block_tables, int bt_stride,
                                     const int32_t* context_lens, int max_context, int num_seqs, int Hq, int Hkv,
                                     int page, float scale, int window, int part_size, int num_parts,
-                                    float* scratch, int32_t* counters, int spread_heads, hipStream_t stream) {
+                                    float* scratch, int spread_heads, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   AttnArgs a;
   if (fill_common(a, qkv, row_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
@@ -1805,5 +1746,5 @@ extern "C" int me_attn_decode_fused(const void* qkv, int64_t row_stride, void* o
   a.raw_v = a.raw_k + (int64_t)Hkv * HD;
   a.q_w = q_w; a.k_w = k_w; a.eps = eps; a.rope = rope;
   a.k_cache_w = (bf16_t*)k_cache; a.v_cache_w = (bf16_t*)v_cache;
-  return launch_decode(a, num_seqs, part_size, num_parts, scratch, counters, spread_heads, true, stream);
+  return launch_decode(a, num_seqs, part_size, num_parts, scratch, spread_heads, true, stream);
 }

@@ -73,8 +73,8 @@ _CORE_PROTOS = {
 }
 _ATTN_PROTOS = {
     "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, I, P, P, I, P],
-    "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, P, I, P],
-    "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, P, I, P],
+    "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, I, P],
+    "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, I, P],
 }
 
 _core: _Lib | None = None
@@ -351,7 +351,6 @@ class HipBackend:
             lib.call("me_attn_decode", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
                      num_decodes, Hq, Hkv, page, float(scale), win, part_size, num_parts, _ptr(scratch),
-                     _ptr(_part_counters(num_decodes * Hkv * -(-(Hq // Hkv) // 16), q.device) if num_parts > 1 else None),
                      0 if even_contexts else 1, _stream())
         if T > num_decodes:
             _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
@@ -406,9 +405,7 @@ class HipBackend:
                          _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(table), 0 if table is None else table.shape[0],
                          k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
                          context_lens.data_ptr(), int(max_context), B, Hq, Hkv, page, float(scale), int(window or 0),
-                         part_size, num_parts, _ptr(scratch),
-                         _ptr(_part_counters(B * Hkv * -(-(Hq // Hkv) // 16), qkv.device) if num_parts > 1 else None),
-                         0 if even_contexts else 1, _stream())
+                         part_size, num_parts, _ptr(scratch), 0 if even_contexts else 1, _stream())
         return out
 
     # -- matrix products -----------------------------------------------------------------
@@ -644,24 +641,6 @@ def _scratch(num_floats: int, device, use: str = "decode") -> torch.Tensor:
     return buf
 
 
-PART_COUNTERS = 1 << 16
-MERGE_PARTITIONS_IN_KERNEL = True
-_part_counter_buf: dict = {}
-
-
-def _part_counters(count: int, device) -> torch.Tensor | None:
-    """Zeroed int32 counters, one per (request, block of heads), with which the decode kernel's workgroups find out
-    which of a context's partitions finishes last (that one merges them); the kernel leaves them zero. One array
-    per device, made once; a launch that would need more gets None and merges in a launch of its own. Launches
-    on different streams of one device would share them: the engine runs on one stream."""
-    if not MERGE_PARTITIONS_IN_KERNEL or count > PART_COUNTERS:
-        return None
-    buf = _part_counter_buf.get(device)
-    if buf is None:
-        buf = _part_counter_buf[device] = torch.zeros((PART_COUNTERS,), dtype=torch.int32, device=device)
-    return buf
-
-
 def prefill_col_tiles(max_context: int, window: int, num_tokens: int, Hq: int, D: int = 128) -> int:
     """Column tiles (of 16 (token, head) pairs) per wave of the prefill kernel: 2 halves the reads of keys and
     values per product but needs twice the columns per workgroup, so it is for launches with many columns (32,768
@@ -876,15 +855,35 @@ def prefill_waves(max_context: int, num_tokens: int, num_seqs: int, Hq: int, Hkv
     return 3
 
 
+_DECODE_PART_SIZES = tuple(range(128, 577, 32)) + tuple(range(640, 1409, 64))
+
+
+def _decode_partition_cost(base: int, ctx: int, part: int) -> float:
+    """What a launch of the split decode kernel costs with partitions of `part` keys, in units of one key's work on a
+    compute unit: the keys of the busiest compute unit (its workgroups, each with about 64 keys' worth of work before
+    and after its keys; a few workgroups beyond a multiple of the 256 units already make some unit that busy), 80 for
+    every block that a wave takes after another (a trip to memory that nothing hides), and 300 for every round of
+    workgroups beyond the 768 that run at once. Fitted to 86 launches timed over all sizes (1-32 requests of 300-66,000
+    keys, 8 key heads with 2, 4 and 8 query heads each, 2 key heads of 64 channels): the size it puts first is 2 %
+    behind the fastest on average (12 % at worst)."""
+    parts = -(-ctx // part)
+    workgroups = base * parts
+    per_unit = workgroups / _COMPUTE_UNITS
+    busiest = int(per_unit) + min(1.0, (per_unit - int(per_unit)) * 3) if per_unit > 1 else 1.0
+    rounds = -(-workgroups // _DECODE_ONE_ROUND)
+    return busiest * (part + 64) + 80 * -(-part // 128) + 300 * (rounds - 1)
+
+
 def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: bool = False) -> tuple:
     """(keys per partition, number of partitions) for the split decode kernel.
 
     A workgroup's 4 waves take the 32-key blocks of its partition in turn, and three workgroups share a compute
-    unit: 768 run at once. While (sequences x kv heads) stays below that, the partitions are sized so that all
-    workgroups run in one round (8 requests of 2,048 keys: 11 partitions of 192 keys, 704 workgroups; with
-    partitions of 128 keys 1,088 workgroups run in a round and a third, which costs a fifth more), at least 128
-    keys (one block per wave) and at most 512 (beyond, more and shorter workgroups stream better even in several
-    rounds), never more than 64 partitions to merge, and at most 2,048 keys as long as 64 partitions cover the
+    unit: 768 run at once. While there are fewer (sequence, kv head) pairs than compute units, the partition size is
+    the one of 128, 160, ... 576, 640, ... 1,408 keys that `_decode_partition_cost` puts first (8 requests of 2,048
+    keys: 8 partitions of 256; of 2,070 keys: 11 of 192, 704 workgroups at once, where 17 of 128 keys, 1,088
+    workgroups in a round and a third, cost a fifth more; of 8,200 keys: 12 of 704), never more than 64 partitions to
+    merge. Beyond that list, and from 256 pairs on: one round of workgroups while the pairs stay below 768, at least
+    128 keys (one block per wave) and at most 512, and at most 2,048 keys as long as 64 partitions cover the
     context: a workgroup goes through its keys round by round, so in a batch with a few long contexts among short
     ones the long partitions are what is still running at the end.
     From 768 workgroups on (96 sequences x 8 kv heads) a context up to 2,048 keys (4,096 from 2,048 workgroups
@@ -903,6 +902,13 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
         return -(-ctx // 128) * 128, 1
     if even and base >= _DECODE_EVEN_WHOLE_WORKGROUPS and base % _COMPUTE_UNITS == 0 and ctx <= _DECODE_EVEN_WHOLE_MAX_KEYS:
         return -(-ctx // 128) * 128, 1
+    if base < _COMPUTE_UNITS:
+        # fewer (request, head block) pairs than compute units: the size that a simple reckoning of the launch's time
+        # puts first (sizes beyond the list only where 64 partitions of the largest do not cover the context)
+        sizes = [p for p in _DECODE_PART_SIZES if -(-ctx // p) <= 64]
+        if sizes:
+            part = min(sizes, key=lambda p: (_decode_partition_cost(base, ctx, p), -p))
+            return part, max(1, -(-ctx // part))
     if base <= _DECODE_ONE_ROUND:
         # one round of workgroups where the batch allows it
         per = -(-ctx // max(1, _DECODE_ONE_ROUND // base))

@@ -241,25 +241,28 @@ def test_pool_sizing_from_free_memory(folders):
     assert llm.config.num_kvcache_blocks == 4 * 8          # capped by what max_num_seqs requests can hold
     out = llm.generate([[1, 2, 3]], SamplingParams(temperature=0, max_tokens=3), use_tqdm=False)
     assert len(out[0]["token_ids"]) == 3
-    # Memory decides, not the cap: 256 requests of 4,096 tokens could hold 65,536 pages (256 MiB at this model's
-    # 4 KiB a page), and the share of the device the engine may use is set so that about 200 MiB are left for them.
+    # Memory decides, not the cap: 1,024 requests of 4,096 tokens could hold 262,144 pages (1 GiB at this model's
+    # 4 KiB a page), and the share of the device the engine may use is set so that about 1,000 MiB are left for them.
     del llm, out
     gc.collect()
     torch.cuda.empty_cache()
     free, total = torch.cuda.mem_get_info()
-    share = ((total - free) + (200 << 20)) / total
-    llm = LLM(folders("A"), max_num_seqs=256, max_num_batched_tokens=512, max_model_len=4096, gpu_memory_utilization=share)
+    share = ((total - free) + (1000 << 20)) / total
+    llm = LLM(folders("A"), max_num_seqs=1024, max_num_batched_tokens=1024, max_model_len=4096, gpu_memory_utilization=share)
     pages = llm.config.num_kvcache_blocks
     per_page = sum(page_bytes(llm.model.cache_plan(), 16, torch.bfloat16))
     assert per_page == 2 * 2 * 2 * 16 * 16 * 2              # layers x (keys, values) x kv heads x page x head size x bytes
-    assert 20000 < pages < 256 * 256, pages
+    assert 150000 < pages < 1024 * 256, pages
     free_now, _ = torch.cuda.mem_get_info()
     in_use = total - free_now                                # weights, workspace, the pool itself
     # what is in use and what is kept free for the steps add up to the share the engine was given: never more, and
-    # less only by what the allocator rounds (and a library workspace of 64 MiB that a first product may have brought)
+    # less only by what the allocator rounds, a library workspace of 64 MiB that a first product may have brought, and
+    # what the sizing steps held for a moment on top of what stays (scratch that grew in them: more after other tests
+    # of this process have run kernels with large scratch; 257 MiB seen): 384 MiB at most, where wrong arithmetic (a factor
+    # of two in a page's bytes, the weights counted twice) is off by the whole pool
     assert in_use + llm.reserved_bytes <= share * total + (8 << 20), (in_use, llm.reserved_bytes, share * total)
-    assert in_use + llm.reserved_bytes >= share * total - (96 << 20), (in_use, llm.reserved_bytes, share * total)
-    assert pages * per_page <= 200 << 20
+    assert in_use + llm.reserved_bytes >= share * total - (384 << 20), (in_use, llm.reserved_bytes, share * total)
+    assert pages * per_page <= 1000 << 20
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])

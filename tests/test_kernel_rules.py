@@ -8,17 +8,25 @@ def test_decode_partitions_cover_the_context():
     for S, Hq, Hkv, ctx in ((1, 16, 8, 2048), (8, 16, 8, 2048), (64, 16, 8, 2304), (1, 32, 8, 100), (3, 6, 2, 130000),
                             (256, 64, 8, 1), (1, 4, 4, 129), (24, 16, 8, 2070), (40, 16, 8, 3000), (95, 16, 8, 2048)):
         part, parts = ops.decode_partitions(S, Hq, Hkv, ctx)
-        assert part % 64 == 0 and part >= 128 and (parts <= 64 or part * 64 >= ctx)
+        assert part % 32 == 0 and part >= 128 and (parts <= 64 or part * 64 >= ctx)
         assert part * parts >= ctx and part * (parts - 1) < ctx
-    # while sequences x kv heads stay below the 768 workgroups that run at once: one round of workgroups (8 requests of
-    # 2,048 keys: 704 workgroups of 192 keys, 17.9 us where 1,088 of 128 keys took 20.5), partitions of 128 to 512 keys
-    assert ops.decode_partitions(8, 16, 8, 2048) == (192, 11) and ops.decode_partitions(16, 16, 8, 2070) == (384, 6)
-    assert ops.decode_partitions(12, 16, 8, 2070) == (320, 7) and ops.decode_partitions(8, 16, 8, 4100) == (384, 11)
+    # fewer (request, head block) pairs than compute units: the size that the reckoning of the launch's time puts
+    # first. 8 requests of 2,048 keys: 8 partitions of 256 keys are two workgroups to every compute unit, a few keys
+    # more and 11 of 192 (704 workgroups, all at once: 18.4 us where 1,088 of 128 keys took 20.5); longer contexts in
+    # one round of larger partitions (8 of 8,200 keys: 12 of 704, 48 us where 17 of 512 took 52)
+    assert ops.decode_partitions(8, 16, 8, 2048) == (256, 8) and ops.decode_partitions(8, 16, 8, 2070) == (192, 11)
+    assert ops.decode_partitions(16, 16, 8, 2070) == (352, 6) and ops.decode_partitions(12, 16, 8, 2070) == (416, 5)
+    assert ops.decode_partitions(8, 16, 8, 4100) == (352, 12) and ops.decode_partitions(8, 16, 8, 8200) == (704, 12)
     assert ops.decode_partitions(1, 16, 8, 2048) == (128, 16) and ops.decode_partitions(4, 16, 8, 2070) == (128, 17)
-    assert ops.decode_partitions(24, 16, 8, 2070) == (512, 5) and ops.decode_partitions(48, 16, 8, 2070, even=True) == (512, 5)
-    assert all(8 * S * ops.decode_partitions(S, 16, 8, 2070)[1] <= 768 for S in (1, 2, 3, 5, 8, 11, 16))
+    assert ops.decode_partitions(24, 16, 8, 2070) == (544, 4) and ops.decode_partitions(48, 16, 8, 2070, even=True) == (512, 5)
+    assert all(8 * S * ops.decode_partitions(S, 16, 8, 2070)[1] <= 768 for S in (1, 2, 3, 5, 8, 11, 16, 24, 31))
+    # the reckoning itself: a round more costs, a partition of a block more to a wave costs, and what counts of the
+    # workgroups is how many the busiest compute unit has
+    cost = ops._decode_partition_cost
+    assert cost(64, 2070, 128) > cost(64, 2070, 192) < cost(64, 2070, 256) and cost(64, 2048, 256) < cost(64, 2048, 192)
+    assert cost(64, 8200, 704) < cost(64, 8200, 512) and cost(8, 2048, 128) < cost(8, 2048, 256)
     # never more than 64 partitions; a partition holds at most 2,048 keys while 64 partitions cover the context
-    assert ops.decode_partitions(8, 16, 8, 32768) == (512, 64) and ops.decode_partitions(1, 16, 8, 70000) == (1152, 61)
+    assert ops.decode_partitions(8, 16, 8, 32768) == (1024, 32) and ops.decode_partitions(1, 16, 8, 70000) == (1152, 61)
     assert ops.decode_partitions(128, 16, 8, 16384) == (2048, 8) and ops.decode_partitions(256, 16, 8, 8192) == (2048, 4)
     assert ops.decode_partitions(3, 6, 2, 130000) == (2048, 64) and ops.decode_partitions(4, 16, 8, 1 << 20) == (16384, 64)
     # 768 workgroups without a split: contexts up to 4,096 keys stay whole

@@ -324,30 +324,6 @@ def test_attention_decode_equal_contexts_in_one_partition(Hq, Hkv, D, page):
     close(hip().paged_attention(*args, even_contexts=False), want, 1.5e-2)
 
 
-@pytest.mark.parametrize("Hq,Hkv,D,page", [(16, 8, 128, 16), (6, 2, 32, 8), (80, 1, 32, 16), (40, 8, 128, 16)])
-@pytest.mark.parametrize("window", [None, 100])
-def test_attention_decode_partitions_merged_by_the_last_workgroup(monkeypatch, Hq, Hkv, D, page, window):
-    """The partitions of a context are merged inside the decode kernel by whichever workgroup of theirs finishes last,
-    with counters that the kernel leaves at zero: the same bits as the merge in a launch of its own, launch after
-    launch (the counters are used again), with batches of different sizes and contexts with unequal numbers of
-    partitions, some without keys."""
-    counters = ops._part_counters(1, DEV)
-    assert counters is not None and int(counters.abs().sum()) == 0
-    cases = ([(3000, 1), (40, 1), (1, 1), (700, 1), (2049, 1), (128, 1), (2999, 1)], [(1500, 1)], [(2070 + i % 3, 1) for i in range(16)],
-             [(900, 1), (129, 1)])
-    for round_ in range(2):
-        for i, seqs in enumerate(cases):
-            args = _attention_case(torch.bfloat16, Hq, Hkv, D, page, seqs, window=window, seed=20 + i)
-            assert ops.decode_partitions(len(seqs), Hq, Hkv, max(L for L, _ in seqs), False)[1] > 1
-            monkeypatch.setattr(ops, "MERGE_PARTITIONS_IN_KERNEL", True)
-            merged = hip().paged_attention(*args)
-            assert int(counters.abs().sum()) == 0, "the kernel did not leave its counters at zero"
-            monkeypatch.setattr(ops, "MERGE_PARTITIONS_IN_KERNEL", False)
-            assert torch.equal(merged, hip().paged_attention(*args))
-            if round_ == 0:
-                close(merged, twin.paged_attention(*args), 1.5e-2)
-
-
 @pytest.mark.parametrize("window", [None, 100, 1000])
 def test_attention_decode_contexts_of_very_different_lengths(window):
     """One batch with contexts from 1 to 3,000 keys: the partitions are those of the longest, so most
@@ -500,7 +476,7 @@ def test_decode_partitions_rule():
     for S, Hq, Hkv, ctx in ((1, 16, 8, 2048), (8, 16, 8, 2048), (64, 16, 8, 2304), (1, 32, 8, 100), (3, 6, 2, 130000),
                             (256, 16, 8, 4096), (256, 16, 8, 4097), (128, 16, 8, 16384)):
         part, parts = ops.decode_partitions(S, Hq, Hkv, ctx)
-        assert part % 64 == 0 and part >= 128 and part * parts >= ctx and part * (parts - 1) < ctx
+        assert part % 32 == 0 and part >= 128 and part * parts >= ctx and part * (parts - 1) < ctx
 
 
 # ------------------------------------------------------------------------------- products
