@@ -324,6 +324,23 @@ def test_attention_decode_equal_contexts_in_one_partition(Hq, Hkv, D, page):
     close(hip().paged_attention(*args, even_contexts=False), want, 1.5e-2)
 
 
+@pytest.mark.parametrize("part", [128, 160, 192, 224, 256, 288, 352, 416, 544, 704, 1088, 1408])
+@pytest.mark.parametrize("window", [None, 300])
+def test_attention_decode_at_every_partition_size(monkeypatch, part, window):
+    """The partition sizes that `decode_partitions` chooses among (multiples of 32 keys; with 129-256 keys a wave asks
+    for the keys of its two blocks at once), forced one by one: contexts that end in a partition's first block, its
+    last, or exactly at its edge, a short one among them, the one key that matters in the last partition's first
+    block; at two shapes of heads."""
+    lens = [3000, part * 3, part * 2 + 1, part + 33, 40]
+    parts = -(-max(lens) // part)
+    monkeypatch.setattr(ops, "decode_partitions", lambda *a, **k: (part, parts))
+    peak = (3000 - 1) // part * part + 5
+    args = _attention_case(torch.bfloat16, 16, 8, 128, 16, [(L, 1) for L in lens], window=window, seed=part, peak=peak if window is None else None)
+    close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
+    args = _attention_case(torch.bfloat16, 6, 2, 64, 8, [(L, 1) for L in lens], window=window, seed=part + 1)
+    close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
+
+
 @pytest.mark.parametrize("window", [None, 100, 1000])
 def test_attention_decode_contexts_of_very_different_lengths(window):
     """One batch with contexts from 1 to 3,000 keys: the partitions are those of the longest, so most
