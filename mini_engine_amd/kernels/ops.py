@@ -419,8 +419,9 @@ class HipBackend:
         (library_streams_better), the FMA kernel for shapes the MFMA kernel refuses.
         With allow_partials the result may be float32 partial sums [S, M, N] over slices of K for a
         consumer that adds them: from the skinny kernel when the output features are few
-        (choose_ksplit), from the rows kernel for 17-32 rows over large weights (rows_takes), from the
-        library as a strided batch for 33-1,024 rows over large weights (library_splits).
+        (choose_ksplit), from the rows kernel for 17-32 rows over large weights (rows_takes), from the tiled
+        kernel for 33 to a few hundred rows over weights up to 27 M elements (mid_slices), from the
+        library as a strided batch for 33-1,024 rows over larger weights (library_splits).
         `out` (not with allow_partials): a contiguous [M, N] tensor of the output dtype to write into."""
         _check(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: {tuple(x.shape)} x {tuple(w.shape)}^T")
         _check(x.dtype == w.dtype, f"linear: activation {x.dtype} and weight {w.dtype} differ")
@@ -445,6 +446,12 @@ class HipBackend:
             core().call("me_gemm_tiled", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         ME_BF16, _code(out_dtype), M, N, K, _stream())
             return y
+        mid_parts = mid_takes(M, N, K, True) if (allow_partials and out_dtype == x.dtype) else 0
+        if mid_parts > 1:
+            parts = torch.empty((mid_parts, M, N), dtype=torch.float32, device=x.device)
+            core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), parts.data_ptr(), N,
+                        ME_F32, mid_parts, M, N, K, 0, _stream())
+            return parts
         splits = library_splits(M, N, K) if (allow_partials and out_dtype == x.dtype) else 1
         if splits > 1:
             parts = library_product(x, w, torch.float32, splits)
@@ -456,9 +463,7 @@ class HipBackend:
             core().call("me_gemm_rows_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
                         ME_F32, parts.data_ptr(), ksplit, M, N, K, rows_wide(M, N, ksplit), _stream())
             return parts
-        # 33-64 rows over few output features and a long K: the tiled kernel's four slices are ahead of the skinny split
-        mid_first = allow_partials and out_dtype == x.dtype and mid_takes(M, N, K, True) == 4
-        ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype and not mid_first
+        ksplit = choose_ksplit(M, N, K) if (allow_partials and M <= PARTIALS_MAX_M and out_dtype == x.dtype
                                             and (M <= SKINNY_MAX_M or N * K <= SKINNY_WIDE_MAX_WEIGHT)
                                             and not library_streams_better(M, N, K)) else 1
         if ksplit > 1:
@@ -466,18 +471,12 @@ class HipBackend:
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, N,
                         ME_F32, parts.data_ptr(), ksplit, M, N, K, 0, 0, skinny_wide(N, K), _stream())
             return parts
-        if skinny_takes(M, N, K) and not mid_first:
+        if skinny_takes(M, N, K):
             y = new()
             core().call("me_gemm_skinny_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), None, 1, M, N, K, 0, 0, skinny_wide(N, K), _stream())
             return y
-        mid = mid_takes(M, N, K, allow_partials and out_dtype == x.dtype)
-        if mid > 1:
-            parts = torch.empty((mid, M, N), dtype=torch.float32, device=x.device)
-            core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), parts.data_ptr(), N,
-                        ME_F32, mid, M, N, K, 0, _stream())
-            return parts
-        if mid == 1:
+        if mid_takes(M, N, K, False) == 1:
             y = new()
             core().call("me_gemm_mid_bf16", x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), y.data_ptr(), N,
                         _code(out_dtype), 1, M, N, K, 0, _stream())
@@ -822,16 +821,57 @@ def choose_ksplit(M: int, N: int, K: int) -> int:
     return best
 
 
+MID_SLICES_MAX_WEIGHT = 27 << 20
+
+
+def mid_slices(M: int, N: int, K: int) -> int:
+    """In how many slices of K (2, 4 or 8; 1: not so) the tiled kernel of csrc/gemm_mid.hip computes M rows against a
+    weight [N, K] as float32 partial sums for a consumer that adds them: o and down of a layer at 33 to a few hundred
+    rows. A tile of 64 x 64 is one workgroup, and a compute unit that draws its operands alone gets them slowly, so
+    what counts is how many workgroups there are: as many slices as keep tiles x slices within 384 workgroups, each
+    slice with 8 steps of 64 or more (4 where the workgroups are 128 at most). Where it is ahead of the skinny split,
+    the rows kernel and the library's strided batch (us with the norm that adds the slices behind, this / those): weights
+    up to 8 M elements with up to 2,048 features (1024 x 3072 at 64 rows in 8 slices 8.3 / 9.4 in 4); up to 13 M and
+    2,560 features at up to 256 rows (2048 x 6144 at 64 rows 11.6 / 14.7, 2560 x 4096 at 128 rows 13.7 / 20.9); up to 27 M
+    at up to 128 rows with 4,096 features or fewer (2560 x 9728 at 64 rows 21.3 / 24.7, 4096 x 4096 at 64 rows 14.3 /
+    17.2) and up to 64 rows with 5,120 (5120 x 5120 at 40 rows 21.3 / 24.0). Beyond (4096 x 12288, 5120 x 17408, more
+    rows) the library's larger tiles are level or ahead."""
+    weight = N * K
+    if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 2048 or M <= 32 or weight > MID_SLICES_MAX_WEIGHT:
+        return 1
+    if weight <= MID_MAX_WEIGHT:
+        if N > 2048 or M > (512 if N <= 1024 else 256):
+            return 1
+        if M > 256:
+            return 4
+    elif weight <= 13 << 20:
+        if N > 2560 or M > 256:
+            return 1
+    elif N > 5120 or M > (128 if N <= 4096 else 64):
+        return 1
+    tiles = -(-N // 64) * -(-M // 64)
+    steps = K // 64
+    for slices in (8, 4, 2):
+        per = -(-steps // slices)                       # steps of a slice; the last may have fewer, none has none
+        if tiles * slices <= 384 and (slices - 1) * per < steps and (per >= 8 or (per >= 4 and tiles * slices <= 128)):
+            return slices
+    return 1
+
+
 def mid_takes(M: int, N: int, K: int, partials: bool) -> int:
     """Whether the product of M rows against a bfloat16 weight [N, K] goes to the own kernel for a few hundred rows
-    over small weights (csrc/gemm_mid.hip), and in how many slices of K: 0 no, 1 one result, 4 float32 partial
-    sums over four slices (only when the consumer adds them, `partials`). Its time is 7 us whatever the row count
-    up to 256 (tiles of 64 x 64, one workgroup to a compute unit), where the library's grows with the rows; beyond
-    8 M weight elements and beyond these row counts the library's larger tiles win."""
-    if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 256 or N * K > MID_MAX_WEIGHT or M <= 32:
+    (csrc/gemm_mid.hip), and in how many slices of K: 0 no, 1 one result, 2, 4 or 8 float32 partial sums over
+    that many slices (only when the consumer adds them, `partials`: `mid_slices`). One result: its time is 7 us
+    whatever the row count up to 256 (tiles of 64 x 64, one workgroup to a compute unit), where the library's grows
+    with the rows; beyond 8 M weight elements and beyond these row counts the library's larger tiles win."""
+    if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 256 or M <= 32:
         return 0
-    if partials and N <= 2048 and K >= 2048 and M <= (512 if N <= 1024 else 256):
-        return 4
+    if partials:
+        slices = mid_slices(M, N, K)
+        if slices > 1:
+            return slices
+    if N * K > MID_MAX_WEIGHT:
+        return 0
     if N * K > MID_SMALL_WEIGHT and M < 128:
         return 0          # the larger of the small weights with few rows: the library's tiles are ahead
     return 1 if M <= 256 else 0

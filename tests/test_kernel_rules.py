@@ -66,6 +66,7 @@ def test_a_few_hundred_rows_over_small_weights_go_to_the_own_product():
     assert ops.mid_takes(257, 6144, 1024, False) == 0                   # more rows: the library's larger tiles
     assert ops.mid_takes(32, 4096, 1024, False) == 0                    # few rows: the skinny kernels
     assert ops.mid_takes(128, 1024, 2048, True) == 4 and ops.mid_takes(512, 1024, 3072, True) == 4
+    assert ops.mid_takes(64, 1024, 2048, True) == 8 and ops.mid_takes(64, 1024, 3072, True) == 8       # one tile of rows: 128 workgroups
     assert ops.mid_takes(513, 1024, 3072, True) == 0 and ops.mid_takes(128, 1024, 2048, False) == 1
     assert ops.mid_takes(128, 4096, 1024, True) == 1                    # many features: no slices of K
     assert ops.mid_takes(128, 12288, 2048, False) == 0                  # beyond 8 M weight elements
@@ -179,6 +180,15 @@ def test_rules_at_the_layer_sizes_between_the_measured_ones():
     # down at the 4B sizes (2560 features over a K of 9,728): the rows kernel at 33-64 rows, where the library's slices take
     # 48 us and its plain call 29 (64 rows: -> 21 us); the slices again beyond
     assert ops.rows_takes(64, 2560, 9728) and ops.library_splits(64, 2560, 9728) == 1 and ops.library_splits(128, 2560, 9728) == 8
+    # ... and ahead of both, with the norm that adds the slices counted in: the tiled kernel in 8 slices (64 rows: 24.7 ->
+    # 21.3 us) and in 4 at 128 rows (35.1 -> 31.5); o at the 8B sizes likewise up to 128 rows (64 rows: 17.2 -> 14.3), at
+    # the 14B sizes up to 64; down at the 8B and 14B sizes stays with the library's slices
+    assert ops.mid_takes(64, 2560, 9728, True) == 8 and ops.mid_takes(128, 2560, 9728, True) == 4 and ops.mid_takes(256, 2560, 9728, True) == 0
+    assert ops.mid_takes(64, 4096, 4096, True) == 4 and ops.mid_takes(128, 4096, 4096, True) == 2 and ops.mid_takes(256, 4096, 4096, True) == 0
+    assert ops.mid_takes(64, 5120, 5120, True) == 4 and ops.mid_takes(128, 5120, 5120, True) == 0
+    assert ops.mid_takes(64, 4096, 12288, True) == 0 and ops.mid_takes(64, 5120, 17408, True) == 0
+    assert ops.mid_takes(64, 2048, 6144, True) == 8 and ops.mid_takes(128, 2560, 4096, True) == 4       # 1.7B down, 4B o
+    assert all(ops.mid_takes(M, N, K, False) == 0 for M, N, K in ((64, 2560, 9728), (64, 4096, 4096), (64, 2048, 6144)))
     assert not ops.rows_has_few_features(64, 5120, 17408) and ops.library_splits(64, 5120, 17408) == 8     # 14B: stays with the slices
     # qkv at the 4B sizes (15.7 M elements): the library from 17 rows (32 rows: 18.8 -> 10.4 us), the skinny kernel's wide loads below
     assert ops.library_streams_better(32, 6144, 2560) and not ops.library_streams_better(16, 6144, 2560)
@@ -188,6 +198,7 @@ def test_rules_at_the_layer_sizes_between_the_measured_ones():
     assert ops.mid_takes(64, 4096, 2048, False) == 0 and ops.mid_takes(128, 4096, 2048, False) == 1
     assert ops.mid_takes(64, 4096, 1024, False) == 1                     # the 0.6B sizes keep theirs
     # o at the 1.7B sizes at 33-64 rows: the tiled kernel's four slices of K, not the skinny split (64 rows: 7.9 -> 5.9 us);
-    # beyond 1,024 features only up to 256 rows (512 rows: 13.1 -> 11.7 with the library)
-    assert ops.mid_takes(64, 2048, 2048, True) == 4 and ops.mid_takes(256, 2048, 2048, True) == 4
+    # beyond 1,024 features only up to 256 rows (512 rows: 13.1 -> 11.7 with the library), and there in two slices
+    # (128 tiles: 256 workgroups)
+    assert ops.mid_takes(64, 2048, 2048, True) == 4 and ops.mid_takes(256, 2048, 2048, True) == 2
     assert ops.mid_takes(512, 2048, 2048, True) == 0 and ops.mid_takes(512, 1024, 2048, True) == 4

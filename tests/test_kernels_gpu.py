@@ -702,16 +702,18 @@ def test_linear_a_few_hundred_rows_over_small_weights(M, N, K):
         close(hip().linear(xs, w), xs.double() @ w.double().t(), 6e-3)
     parts = hip().linear(x, w, None, allow_partials=True)
     if N <= 2048 and K >= 2048:
-        assert ops.mid_takes(M, N, K, True) == 4 and parts.shape == (4, M, N) and parts.dtype == torch.float32
+        slices = ops.mid_takes(M, N, K, True)
+        assert slices in (2, 4, 8) and parts.shape == (slices, M, N) and parts.dtype == torch.float32
         close(parts.sum(0), ref, 2e-5)
     else:
         assert parts.dim() == 2
         close(parts, ref, 6e-3)
 
 
-@pytest.mark.parametrize("M,N,K,route", [(48, 1024, 2048, "mid"), (64, 2048, 2048, "mid"), (64, 2560, 9728, "rows"), (40, 2560, 9728, "rows"),
-                                         (64, 2048, 6144, "slices"), (128, 2560, 4096, "slices"), (64, 2560, 4096, "plain"),
-                                         (32, 2560, 4096, "rows"), (32, 6144, 2560, "plain"), (64, 4096, 2048, "plain")])
+@pytest.mark.parametrize("M,N,K,route", [(48, 1024, 2048, "mid"), (64, 2048, 2048, "mid"), (64, 2560, 9728, "mid"), (40, 2560, 9728, "mid"),
+                                         (64, 2048, 6144, "mid"), (128, 2560, 4096, "mid"), (64, 2560, 4096, "mid"), (128, 4096, 4096, "mid"),
+                                         (64, 5120, 5120, "mid"), (200, 2560, 9728, "slices"), (64, 4096, 12288, "slices"),
+                                         (32, 2560, 9728, "rows"), (32, 2560, 4096, "rows"), (32, 6144, 2560, "plain"), (64, 4096, 2048, "plain")])
 def test_linear_routes_at_the_sizes_between_the_measured_ones(M, N, K, route):
     """Products of the 1.7B, 4B layer sizes at row counts where the rules were corrected: the route the rules name
     is the one that runs, and it gives the exact product."""
@@ -720,7 +722,7 @@ def test_linear_routes_at_the_sizes_between_the_measured_ones(M, N, K, route):
     ref = x.double() @ w.double().t()
     parts = hip().linear(x, w, None, allow_partials=True)
     if route == "mid":
-        assert ops.mid_takes(M, N, K, True) == 4 and parts.shape == (4, M, N)
+        assert ops.mid_takes(M, N, K, True) in (2, 4, 8) and parts.shape == (ops.mid_takes(M, N, K, True), M, N)
     elif route == "rows":
         assert ops.rows_takes(M, N, K) and parts.shape == (ops.rows_ksplit(K), M, N)
     elif route == "slices":
@@ -774,12 +776,13 @@ def test_library_product_is_called_directly(M, N, K):
         close(ops.library_product(x, w, torch.float32), x.double() @ w.double().t(), 2e-5)
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 4096, 4096), (128, 4096, 4096), (200, 2560, 9728), (300, 4096, 12288), (700, 5120, 8192), (100, 1368, 12288 + 64)])
+@pytest.mark.parametrize("M,N,K", [(33, 4096, 12288), (256, 4096, 4096), (200, 2560, 9728), (300, 4096, 12288), (700, 5120, 8192), (200, 1368, 12288 + 64)])
 def test_linear_library_slices_of_k(M, N, K):
-    """o and down at 33 to 1,024 rows over large weights: the library runs slices of K as one strided batch
-    and the consumer adds the float32 partial sums."""
+    """o and down at 33 to 1,024 rows over large weights (where the tiled kernel's slices are not ahead): the library
+    runs slices of K as one strided batch and the consumer adds the float32 partial sums."""
     from mini_engine_amd.kernels import ops
     splits = ops.library_splits(M, N, K)
+    assert ops.mid_takes(M, N, K, True) == 0
     assert splits == (8 if M <= 256 else 4 if M <= 512 else 2) and K % (8 * splits) == 0
     x = torch.randn(M, K, device=DEV).bfloat16()
     w = (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
