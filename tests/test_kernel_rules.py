@@ -202,3 +202,24 @@ def test_rules_at_the_layer_sizes_between_the_measured_ones():
     # (128 tiles: 256 workgroups)
     assert ops.mid_takes(64, 2048, 2048, True) == 4 and ops.mid_takes(256, 2048, 2048, True) == 2
     assert ops.mid_takes(512, 2048, 2048, True) == 0 and ops.mid_takes(512, 1024, 2048, True) == 4
+
+
+def test_slices_of_the_tiled_kernel_fit_what_the_kernel_and_the_norm_take():
+    """Whatever sizes come: the slices that `mid_slices` names leave no slice without steps (the kernel refuses that),
+    are at most the 8 partial sums that the norm kernel adds, and only K in whole steps of 64 is sliced."""
+    import random
+    rng = random.Random(5)
+    seen = set()
+    for _ in range(20000):
+        M, N, K = rng.randint(1, 700), 4 * rng.randint(1, 1600), 64 * rng.randint(1, 300)
+        if rng.random() < 0.2:
+            K += rng.choice([8, 16, 32])
+        slices = ops.mid_slices(M, N, K)
+        seen.add(slices)
+        assert slices in (1, 2, 4, 8)
+        if slices > 1:
+            steps = K // 64
+            per = -(-steps // slices)
+            assert K % 64 == 0 and M > 32 and (slices - 1) * per < steps and N * K <= ops.MID_SLICES_MAX_WEIGHT
+            assert ops.mid_takes(M, N, K, True) == slices and ops.mid_takes(M, N, K, False) in (0, 1)
+    assert seen == {1, 2, 4, 8}
