@@ -13,15 +13,14 @@
 // partial sums [S, M, N] for a consumer that adds them. Workgroups that share weight rows run on the same XCD.
 // An iteration is a chain of wait, barrier, LDS reads and 8 products (about 500 cycles for 128 cycles of matrix
 // work), so the kernel takes 7 us whatever the row count up to 256 and loses to the library's larger tiles
-// beyond; the caller (ops.mid_takes) knows where it is ahead.
+// beyond; the caller (ops.mid_takes) knows where it is ahead. Where K is a multiple of 128 an iteration walks 128 of
+// K instead (BK = 128: rows of 256 bytes, 16 pieces, piece c of row R at position c ^ (R & 15); 96 KB of LDS for
+// the three stages): half as many iterations, each with 16 products behind the same wait and barrier.
 #include "common.h"
 
 #define MID_TM 64
 #define MID_TN 64
-#define MID_BK 64
-#define MID_NB 3                                      // stages in LDS (48 KB): two asked for ahead of the one in use
-#define MID_STAGE ((MID_TM + MID_TN) * 2 * MID_BK)   // bytes
-#define MID_DMA_PER_WAVE ((MID_TM + MID_TN) / 8 / 4)  // instructions of 8 rows, per wave and stage
+#define MID_NB 3                                      // stages in LDS (48 or 96 KB): two asked for ahead of the one in use
 
 // gbase and lds_addr are the same in every lane; the first lane's values are taken so that they lie in scalar
 // registers whatever the compiler has concluded about them. The write to m0 needs one wait state before an
@@ -39,11 +38,17 @@ __device__ __forceinline__ void mid_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // ACT: w is a packed gate/up weight [2 I, K] (gate rows first, N = 2 I); the tile's 64 weight rows are 32 gate rows and
 // the 32 up rows that go with them, a wave's two feature tiles are 16 gate features and their up features, and what
 // is written is silu(gate) * up [M, I], formed from the unrounded sums (reference layers/activation.py:5-7).
-template <typename TO, bool PARTIAL, bool ACT>
+template <typename TO, bool PARTIAL, bool ACT, int MID_BK>
 __global__ void __launch_bounds__(256)
 gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, int64_t ldw,
                 TO* __restrict__ y, int64_t ldy, int M, int N, int K, int steps_per_split, int m_tiles, int n_tiles) {
   extern __shared__ __align__(16) unsigned char mid_lds[];   // [MID_NB][MID_STAGE]
+  static_assert(MID_BK == 64 || MID_BK == 128, "a row of a stage is 128 or 256 bytes");
+  constexpr int ROW = 2 * MID_BK;                                    // bytes of a row in LDS
+  constexpr int MID_STAGE = (MID_TM + MID_TN) * ROW;                // bytes
+  constexpr int ROWS_PER_DMA = 1024 / ROW;                           // rows that one instruction of a wave brings
+  constexpr int MID_DMA_PER_WAVE = (MID_TM + MID_TN) / ROWS_PER_DMA / 4;
+  constexpr int PIECES = ROW / 16;                                   // 16-byte pieces of a row
   constexpr int PD = MID_NB - 1;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -68,10 +73,10 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
   bool is_x[MID_DMA_PER_WAVE];
 #pragma unroll
   for (int q = 0; q < MID_DMA_PER_WAVE; ++q) {
-    const int inst = wave + 4 * q;                 // 0 .. (TM + TN) / 8 - 1; the first TM / 8 hold token rows
-    const int R = 8 * inst + (lane >> 3);
-    const int c = (lane & 7) ^ ((R >> 1) & 7);
-    is_x[q] = inst < MID_TM / 8;
+    const int inst = wave + 4 * q;                 // 0 .. (TM + TN) / rows per instruction - 1; token rows first
+    const int R = ROWS_PER_DMA * inst + lane / PIECES;
+    const int c = (lane % PIECES) ^ (MID_BK == 64 ? (R >> 1) & 7 : R & 15);
+    is_x[q] = inst < MID_TM / ROWS_PER_DMA;
     const int wr = R - MID_TM;                      // weight row of the tile
     const int64_t row = is_x[q] ? min(m0 + R, M - 1)
                         : ACT ? (wr < 32 ? min(n0 + wr, I - 1) : I + min(n0 + wr - 32, I - 1))
@@ -88,12 +93,13 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
   };
   // where this lane reads its operands: token rows of the wave's half, weight rows of its half
   const int wm = wave >> 1, wn = wave & 1;
-  const int swz = (n >> 1) & 7;
-  uint32_t rd_b[2], rd_a[2];
+  const int swz = MID_BK == 64 ? (n >> 1) & 7 : n;
+  constexpr int KS = MID_BK / 32;                  // matrix instructions' steps of 32 along K in a stage
+  uint32_t rd_b[KS], rd_a[KS];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    rd_b[s] = (wm * 32 + n) * 128 + (((4 * s + g) ^ swz) * 16);
-    rd_a[s] = (MID_TM + wn * (ACT ? 16 : 32) + n) * 128 + (((4 * s + g) ^ swz) * 16);
+  for (int s = 0; s < KS; ++s) {
+    rd_b[s] = (wm * 32 + n) * ROW + (((4 * s + g) ^ swz) * 16);
+    rd_a[s] = (MID_TM + wn * (ACT ? 16 : 32) + n) * ROW + (((4 * s + g) ^ swz) * 16);
   }
   f32x4 acc[2][2];
 #pragma unroll
@@ -112,12 +118,12 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
     if (k + PD < nsteps) stage(s_lo + k + PD, cur == 0 ? MID_NB - 1 : cur - 1);
     const unsigned char* buf = mid_lds + cur * MID_STAGE;
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < KS; ++s) {
       bf16x8 a[2], b[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const bf16x8*>(buf + rd_a[s] + (ACT ? 4096 : 2048) * i);
+      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const bf16x8*>(buf + rd_a[s] + (ACT ? 32 : 16) * ROW * i);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) b[j] = *reinterpret_cast<const bf16x8*>(buf + rd_b[s] + 2048 * j);
+      for (int j = 0; j < 2; ++j) b[j] = *reinterpret_cast<const bf16x8*>(buf + rd_b[s] + 16 * ROW * j);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -168,14 +174,17 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restr
 extern "C" int me_gemm_mid_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, void* y, int64_t ldy,
                                 int out_dtype, int ksplit, int M, int N, int K, int act, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
-  ME_CHECK(K >= MID_BK && K % MID_BK == 0, "mid gemm: K=%d must be a multiple of %d", K, MID_BK);
+  ME_CHECK(K >= 64 && K % 64 == 0, "mid gemm: K=%d must be a multiple of 64", K);
   ME_CHECK(N % 4 == 0 && ldy % 4 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "mid gemm: N=%d and the row strides must keep 16-byte pieces whole", N);
   ME_CHECK((reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0) &&
                (reinterpret_cast<uintptr_t>(y) % 16 == 0), "mid gemm: operands must be 16-byte aligned");
   ME_CHECK((int64_t)M * ldx * 2 < (1ll << 32) && (int64_t)N * ldw * 2 < (1ll << 32), "mid gemm: an operand beyond 4 GB");
-  const int steps = K / MID_BK;
-  ME_CHECK(ksplit >= 1 && ksplit <= steps, "mid gemm: %d slices of %d steps", ksplit, steps);
+  ME_CHECK(ksplit >= 1 && ksplit <= K / 64, "mid gemm: %d slices of %d steps", ksplit, K / 64);
   ME_CHECK(ksplit == 1 || out_dtype == ME_F32, "mid gemm: partial sums are float32");
+  // steps of 128 where K is in whole steps of 128 and every slice still gets one; else steps of 64
+  bool wide_steps = K % 128 == 0 && (int64_t)(ksplit - 1) * ((K / 128 + ksplit - 1) / ksplit) < K / 128;
+  const int bk = wide_steps ? 128 : 64;
+  const int steps = K / bk;
   const int steps_per_split = (steps + ksplit - 1) / ksplit;
   ME_CHECK((int64_t)(ksplit - 1) * steps_per_split < steps, "mid gemm: ksplit %d leaves a slice without work", ksplit);
   ME_CHECK(!act || (ksplit == 1 && out_dtype == ME_BF16 && N % 8 == 0), "mid gemm: the gating wants one bfloat16 result and I a multiple of 4");
@@ -183,15 +192,31 @@ extern "C" int me_gemm_mid_bf16(const void* x, int64_t ldx, const void* w, int64
   const int64_t ids = (int64_t)((n_tiles + 7) / 8) * 8 * m_tiles;
   ME_CHECK(ids < (1ll << 31), "mid gemm: too many tiles");
   const dim3 grid((unsigned)ids, 1, ksplit), block(256);
-  const size_t lds = (size_t)MID_NB * MID_STAGE;
+  const size_t lds = (size_t)MID_NB * (MID_TM + MID_TN) * 2 * bk;
+#define MID_LAUNCH1(TO, P, A, BK)                                                                                        \
+  gemm_mid_kernel<TO, P, A, BK><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, ldy, \
+                                                             M, N, K, steps_per_split, m_tiles, n_tiles)
 #define MID_LAUNCH(TO, P, A)                                                                                       \
-  gemm_mid_kernel<TO, P, A><<<grid, block, lds, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TO*)y, ldy, M, \
-                                                         N, K, steps_per_split, m_tiles, n_tiles)
+  do {                                                                                                             \
+    if (wide_steps) {                                                                                              \
+      static bool allowed = false;                   /* 96 KB of LDS: more than a kernel may have unasked */       \
+      if (!allowed) {                                                                                              \
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_mid_kernel<TO, P, A, 128>,                            \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                  \
+        ME_CHECK(e == hipSuccess, "mid gemm: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));         \
+        allowed = true;                                                                                            \
+      }                                                                                                            \
+      MID_LAUNCH1(TO, P, A, 128);                                                                                  \
+    } else {                                                                                                       \
+      MID_LAUNCH1(TO, P, A, 64);                                                                                   \
+    }                                                                                                              \
+  } while (0)
   if (act) MID_LAUNCH(bf16_t, false, true);
   else if (ksplit > 1) MID_LAUNCH(float, true, false);
   else if (out_dtype == ME_F32) MID_LAUNCH(float, false, false);
   else MID_LAUNCH(bf16_t, false, false);
 #undef MID_LAUNCH
+#undef MID_LAUNCH1
   ME_LAUNCH_CHECK();
   return 0;
 }
