@@ -144,6 +144,27 @@ def batch_of_decodes(env, name):
         _check(env, folder, ids[r], d.result(r), f"{name} decode batch request {r}")
 
 
+def many_rows_at_real_layer_sizes(env, name="R"):
+    """Batches of 40, 12 and 3 requests at the layer sizes of a real model: their prompts in one step (a few thousand
+    rows: the library's products, prefill attention at head size 128), then decode steps of as many rows (40: o and
+    down in slices of K by the tiled kernel, gate/up with the gating in its epilogue; 12 and 3: the skinny products and
+    their split of K, the norm inside the product), contexts in several partitions."""
+    page = helpers.PAGE[name]
+    V = _vocab(name)
+    for count, base, steps in ((40, 90, 4), (12, 500, 4), (3, 1500, 3)):
+        lens = {f"r{i}": base + 7 * i for i in range(count)}
+        ids = {r: random_ids(n + steps, V, 900 + count + i) for i, (r, n) in enumerate(lens.items())}
+        runner, manager, folder = env.runner(name, sum(-(-(n + steps) // page) for n in lens.values()))
+        d = Driver(runner, manager)
+        d.step({r: ids[r][:lens[r]] for r in lens}, want_all=False)
+        for t in range(steps):
+            d.step({r: ids[r][lens[r] + t: lens[r] + t + 1] for r in lens})
+        for r in list(lens)[::max(1, count // 6)]:
+            ref = plain_logits(folder, ids[r])[lens[r]:]
+            err = rel_err(d.result(r), ref)
+            assert err <= env.tol, f"{count} requests, request {r}: decode logits off by {err:.2e}"
+
+
 def first_tokens(env, name):
     """The first tokens of a sequence, one by one from position 0."""
     ids = random_ids(6, _vocab(name), 700)

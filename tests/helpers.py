@@ -23,9 +23,14 @@ CONFIGS = {
               rms_norm_eps=3e-6, rope_theta=50000.0, tie_word_embeddings=False, max_position_embeddings=4096,
               use_sliding_window=True, sliding_window=24,
               layer_types=["full_attention", "sliding_attention", "full_attention", "sliding_attention"]),
+    # R: two layers at the layer sizes of Qwen3-0.6B (bfloat16 only: the kernel forms that a real model runs through,
+    # which the tiny widths above never reach: products in slices of a long K, wide loads, head size 128)
+    "R": dict(architectures=["Qwen3ForCausalLM"], vocab_size=2048, hidden_size=1024, intermediate_size=3072,
+              num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+              rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True, max_position_embeddings=4096),
 }
-SEEDS = {"A": 0, "B": 1, "C": 2}
-PAGE = {"A": 16, "B": 8, "C": 16}
+SEEDS = {"A": 0, "B": 1, "C": 2, "R": 3}
+PAGE = {"A": 16, "B": 8, "C": 16, "R": 16}
 
 # float32: the engine against the float64 plain model, relative to the largest logit.
 TOL_F32 = 1e-5

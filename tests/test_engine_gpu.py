@@ -16,8 +16,8 @@ pytestmark = pytest.mark.gpu
 class Env:
     device = "cuda"
 
-    def __init__(self, folders, dtype, graphs=False):
-        self.folders, self.dtype = folders, dtype
+    def __init__(self, folders, dtype, graphs=False, max_positions=512):
+        self.folders, self.dtype, self.max_positions = folders, dtype, max_positions
         self.padded_up_to = 4096
         self.graphs = graphs           # every step through a captured graph of its padded layout
         self.tol = helpers.TOL_F32 if dtype == torch.float32 else helpers.TOL_BF16
@@ -26,11 +26,11 @@ class Env:
     def runner(self, name, pages):
         folder = self.folders(name)
         if name not in self.models:
-            self.models[name] = load_model(folder, self.device, self.dtype, 512)
+            self.models[name] = load_model(folder, self.device, self.dtype, self.max_positions)
         model = self.models[name]
         manager = CacheManager(pages, helpers.PAGE[name], ModelRunner.windows_of(model), enable_prefix_caching=False)
         options = dict(use_graphs=True, mixed_graphs_after=0, mixed_graphs_max_tokens=self.padded_up_to) if self.graphs else {}
-        return ModelRunner(model, manager, self.dtype, self.device, 512, poison_cache=True, **options), manager, folder
+        return ModelRunner(model, manager, self.dtype, self.device, self.max_positions, poison_cache=True, **options), manager, folder
 
 
 @pytest.fixture(scope="module", params=[torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -42,6 +42,20 @@ def env(request, folders):
 @pytest.mark.parametrize("case", engine_cases.ALL, ids=lambda c: c.__name__)
 def test_cuts(env, case, name):
     case(env, name)
+
+
+@pytest.mark.parametrize("captured", [False, True], ids=["eager", "graphs"])
+def test_many_rows_at_the_layer_sizes_of_a_real_model(folders, captured):
+    """Two layers at the Qwen3-0.6B layer sizes in bfloat16, batches of 40, 12 and 3 requests, against the plain
+    implementation: the tiny configurations never reach the products in slices of a long K, the wide loads, the
+    library's products or head size 128 inside the engine."""
+    from mini_engine_amd.kernels import ops
+    # what the 40 rows of a decode step go through at these sizes: o and down in eight slices by the tiled kernel, gate/up
+    # with the gating in that kernel's epilogue; 12 rows: the skinny kernel's split of K; contexts of 90-1,500 keys: partitions
+    assert ops.mid_takes(40, 1024, 2048, True) == 8 and ops.mid_takes(40, 1024, 3072, True) == 8
+    assert ops.mid_takes(40, 6144, 1024, False) == 1 and ops.choose_ksplit(12, 1024, 2048) > 1
+    assert ops.decode_partitions(12, 16, 8, 580)[1] > 1 and ops.decode_partitions(3, 16, 8, 1520)[1] > 1
+    engine_cases.many_rows_at_real_layer_sizes(Env(folders, torch.bfloat16, graphs=captured, max_positions=2048))
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
