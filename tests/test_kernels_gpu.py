@@ -339,6 +339,10 @@ def test_attention_decode_at_every_partition_size(monkeypatch, part, window):
     close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
     args = _attention_case(torch.bfloat16, 6, 2, 64, 8, [(L, 1) for L in lens], window=window, seed=part + 1)
     close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
+    if part in (160, 192, 256, 544):            # other head sizes, with and without the keys of two blocks ahead
+        for Hq, Hkv, D, page in ((4, 1, 48, 16), (4, 4, 256, 16), (10, 2, 80, 8), (2, 2, 16, 32)):
+            args = _attention_case(torch.bfloat16, Hq, Hkv, D, page, [(L, 1) for L in lens[1:]], window=window, seed=part + D)
+            close(hip().paged_attention(*args), twin.paged_attention(*args), 1.5e-2)
 
 
 @pytest.mark.parametrize("window", [None, 100, 1000])
