@@ -828,16 +828,19 @@ def mid_slices(M: int, N: int, K: int) -> int:
     """In how many slices of K (2, 4 or 8; 1: not so) the tiled kernel of csrc/gemm_mid.hip computes M rows against a
     weight [N, K] as float32 partial sums for a consumer that adds them: o and down of a layer at 33 to a few hundred
     rows. A tile of 64 x 64 is one workgroup, and a compute unit that draws its operands alone gets them slowly, so
-    what counts is how many workgroups there are: as many slices as keep tiles x slices within 384 workgroups, each
-    slice with 8 steps of 64 or more (4 where the workgroups are 128 at most). Where it is ahead of the skinny split,
-    the rows kernel and the library's strided batch (us with the norm that adds the slices behind, this / those): weights
-    up to 8 M elements with up to 2,048 features (1024 x 3072 at 64 rows in 8 slices 8.3 / 9.4 in 4); up to 13 M and
-    2,560 features at up to 256 rows (2048 x 6144 at 64 rows 11.6 / 14.7, 2560 x 4096 at 128 rows 13.7 / 20.9); up to 27 M
-    at up to 128 rows with 4,096 features or fewer (2560 x 9728 at 64 rows 21.3 / 24.7, 4096 x 4096 at 64 rows 14.3 /
-    17.2) and up to 64 rows with 5,120 (5120 x 5120 at 40 rows 21.3 / 24.0). Beyond (4096 x 12288, 5120 x 17408, more
-    rows) the library's larger tiles are level or ahead."""
+    what counts is how many workgroups there are: as many slices as keep tiles x slices within 256 workgroups (two
+    slices up to 320), each slice with 8 steps of 64 or more (4 where the workgroups are 128 at most). Where it is
+    ahead of the skinny split, the rows kernel and the library's strided batch (us with the norm that adds the slices
+    behind, this / those): weights up to 8 M elements with up to 2,048 features (1024 x 3072 at 64 rows in 8 slices
+    8.3 / 9.4 in 4); up to 13 M and 2,560 features at up to 256 rows (2048 x 6144 at 64 rows 11.6 / 14.7, 2560 x 4096 at
+    128 rows 13.7 / 20.9); up to 27 M and 4,096 features at up to 128 rows (2560 x 9728 at 64 rows 20.1 / 24.7, 4096 x
+    4096 at 64 rows 13.4 / 17.2). Beyond (4096 x 12288, 5120 x 5120, 5120 x 17408, more rows) the library's larger tiles
+    are level or ahead."""
     weight = N * K
-    if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 2048 or M <= 32 or weight > MID_SLICES_MAX_WEIGHT:
+    # from 17 rows over the larger weights (2048 x 6144 at 24 rows 10.2 / 12.0, 2560 x 4096 10.3 / 12.8, 2560 x 9728 17.6 /
+    # 20.3 with the rows kernel); over the small ones the skinny kernel's split keeps 17-32 rows (1024 x 2048: 6.8 / 7.2)
+    if (not USE_MID_PRODUCT or K % 64 or N % 4 or K < 2048 or M <= (32 if weight <= MID_MAX_WEIGHT else 16)
+            or weight > MID_SLICES_MAX_WEIGHT):
         return 1
     if weight <= MID_MAX_WEIGHT:
         if N > 2048 or M > (512 if N <= 1024 else 256):
@@ -847,13 +850,14 @@ def mid_slices(M: int, N: int, K: int) -> int:
     elif weight <= 13 << 20:
         if N > 2560 or M > 256:
             return 1
-    elif N > 5120 or M > (128 if N <= 4096 else 64):
+    elif N > 4096 or M > 128:
         return 1
     tiles = -(-N // 64) * -(-M // 64)
     steps = K // 64
     for slices in (8, 4, 2):
         per = -(-steps // slices)                       # steps of a slice; the last may have fewer, none has none
-        if tiles * slices <= 384 and (slices - 1) * per < steps and (per >= 8 or (per >= 4 and tiles * slices <= 128)):
+        fills = tiles * slices <= 256 or (slices == 2 and tiles <= 160)
+        if fills and (slices - 1) * per < steps and (per >= 8 or (per >= 4 and tiles * slices <= 128)):
             return slices
     return 1
 
@@ -864,12 +868,14 @@ def mid_takes(M: int, N: int, K: int, partials: bool) -> int:
     that many slices (only when the consumer adds them, `partials`: `mid_slices`). One result: its time is 7 us
     whatever the row count up to 256 (tiles of 64 x 64, one workgroup to a compute unit), where the library's grows
     with the rows; beyond 8 M weight elements and beyond these row counts the library's larger tiles win."""
-    if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 256 or M <= 32:
+    if not USE_MID_PRODUCT or K % 64 or N % 4 or K < 256 or M <= 16:
         return 0
     if partials:
         slices = mid_slices(M, N, K)
         if slices > 1:
             return slices
+    if M <= 32:
+        return 0
     if N * K > MID_MAX_WEIGHT:
         return 0
     if N * K > MID_SMALL_WEIGHT and M < 128:

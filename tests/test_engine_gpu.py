@@ -354,7 +354,7 @@ def test_wide_layer_sizes_take_the_products_with_partial_sums(tmp_path_factory, 
     """One layer of Qwen3-8B's width (hidden 4096, 32 query / 8 key heads of 128, intermediate 12288) and of
     Qwen3-32B's (hidden 5120, 64 query / 8 key heads: groups of 8, intermediate 25600): o and down are large
     enough for the forms that hand float32 partial sums over slices of K to the norm that follows (the library
-    as a strided batch at 300 and 127 rows, the rows kernel at 28), which the narrow test configurations never
+    as a strided batch at 300 and 127 rows, the rows kernel at 28 for down, the tiled kernel's slices for o), which the narrow test configurations never
     reach; then decoding; against the plain implementation."""
     from mini_engine_amd.config.model_config import Qwen3Config
     from mini_engine_amd.kernels import ops
