@@ -1695,6 +1695,7 @@ static int launch_decode(AttnArgs& a, int num_seqs, int part_size, int num_parts
   }
   const dim3 grid = a.spread_heads ? dim3(a.Hkv * col_tiles, num_seqs, num_parts) : dim3(num_seqs, a.Hkv * col_tiles, num_parts);
   // partitions of 129-256 keys: a wave has up to two blocks and asks for the keys of both at once
+  // (ME_DECODE_KEYS_AHEAD=0 in the environment leaves that form out, for timing one against the other)
   static const bool ahead_allowed = []() { const char* v = getenv("ME_DECODE_KEYS_AHEAD"); return v == nullptr || v[0] != '0'; }();
   const bool ahead = ahead_allowed && num_parts > 1 && part_size > 128 && part_size <= 256;
   if (prologue && ahead) attn_decode_kernel<true, true><<<grid, dim3(256), lds, stream>>>(a);
