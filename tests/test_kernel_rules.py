@@ -225,3 +225,21 @@ def test_slices_of_the_tiled_kernel_fit_what_the_kernel_and_the_norm_take():
             assert K % 64 == 0 and M > 16 and (slices - 1) * per < steps and N * K <= ops.MID_SLICES_MAX_WEIGHT
             assert ops.mid_takes(M, N, K, True) == slices and ops.mid_takes(M, N, K, False) in (0, 1)
     assert seen == {1, 2, 4, 8}
+
+
+def test_decode_partitions_always_fit_the_kernel():
+    """Whatever batch, heads and context come: partitions of a multiple of 32 keys, at least 128, that cover the
+    context without an empty last one, and at most the 64 that the merge takes unless even 64 of the largest size on
+    the list do not cover the context (then partitions of up to 16,384 keys, still 64)."""
+    import random
+    rng = random.Random(11)
+    for _ in range(20000):
+        Hkv = rng.choice([1, 2, 4, 8, 16])
+        Hq = Hkv * rng.choice([1, 2, 4, 5, 8, 20])
+        S = rng.choice([1, 2, 3, 5, 8, 13, 24, 31, 32, 64, 100, 300])
+        ctx = rng.choice([1, 17, 128, 129, 700, 2048, 2070, 5000, 33000, 140000, 1 << 20])
+        even = rng.random() < 0.5
+        part, parts = ops.decode_partitions(S, Hq, Hkv, ctx, even)
+        assert part % 32 == 0 and part >= 128 and parts >= 1, (S, Hq, Hkv, ctx, even, part, parts)
+        assert part * parts >= ctx and part * (parts - 1) < ctx, (S, Hq, Hkv, ctx, even, part, parts)
+        assert parts <= 64, (S, Hq, Hkv, ctx, even, part, parts)
